@@ -1,0 +1,74 @@
+"""Builds libfrisk_hip.so (HIP kernels + C ABI) for gfx950, in-tree.
+
+    python -m frisk_amd.build          # rebuild everything
+    python -m frisk_amd.build --if-missing
+
+hipcc cross-compiles without a GPU; the resulting library is loaded from
+frisk_amd/lib/ by frisk_amd.runtime.
+"""
+import argparse
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIBDIR = os.path.join(HERE, "lib")
+OBJDIR = os.path.join(CSRC, "build")
+LIB = os.path.join(LIBDIR, "libfrisk_hip.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+COMMON = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # packed-fp32 instructions are kept out of generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+    "-Wno-unused-command-line-argument",
+]
+SOURCES = ["kernels_f16.hip", "kernels_bf16.hip", "kernels_i8.hip", "kernels_e4m3.hip", "kernels_f32.hip", "capi.cpp"]
+
+
+def _compile(src):
+    obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC] + COMMON + (["-x", "hip"] if src.endswith(".cpp") else []) + ["-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and l.strip())
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s" % (src, err))
+    return obj, err
+
+
+def build(jobs=None, verbose=True):
+    os.makedirs(OBJDIR, exist_ok=True)
+    os.makedirs(LIBDIR, exist_ok=True)
+    jobs = jobs or min(6, os.cpu_count() or 1)
+    objs = []
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        for obj, err in pool.map(_compile, SOURCES):
+            objs.append(obj)
+            if verbose and err:
+                print(err, file=sys.stderr)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr)
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--if-missing", action="store_true")
+    ap.add_argument("-j", type=int, default=None)
+    a = ap.parse_args()
+    if a.if_missing and os.path.exists(LIB):
+        print("present", LIB)
+        return
+    build(a.j)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,299 @@
+// C ABI of libfrisk_hip.so: descriptor validation, the planner (tile / wave
+// grid / LDS layout choice) and kernel dispatch.  Host code only.
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "frisk_hip.h"
+#include "gemm_internal.h"
+#include "lds_model.h"
+
+namespace frisk {
+
+static thread_local std::string g_last_error;
+
+static int fail(int status, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return status;
+}
+
+static const std::vector<const KernelEntry*>& kernels() {
+  static const std::vector<const KernelEntry*> all = [] {
+    std::vector<const KernelEntry*> v;
+    for (int i = 0; i < kNumKernelsF16; ++i) v.push_back(&kKernelsF16[i]);
+    for (int i = 0; i < kNumKernelsBF16; ++i) v.push_back(&kKernelsBF16[i]);
+    for (int i = 0; i < kNumKernelsI8; ++i) v.push_back(&kKernelsI8[i]);
+    for (int i = 0; i < kNumKernelsE4M3; ++i) v.push_back(&kKernelsE4M3[i]);
+    for (int i = 0; i < kNumKernelsF32; ++i) v.push_back(&kKernelsF32[i]);
+    return v;
+  }();
+  return all;
+}
+
+static int elem_size(int dt) {
+  switch (dt) {
+    case FRISK_F32: case FRISK_I32: return 4;
+    case FRISK_F16: case FRISK_BF16: return 2;
+    case FRISK_I8: case FRISK_E4M3: return 1;
+    default: return 0;
+  }
+}
+static int frag_bytes(int dt) { return dt == FRISK_E4M3 ? 32 : (dt == FRISK_F32 ? 4 : 16); }
+static int mfma_k(int dt) { return dt == FRISK_F32 ? 2 : (2 * frag_bytes(dt)) / elem_size(dt); }
+
+// Wave partition of a block tile: the reference's computeWarpPartition
+// (lib/Dialect/Frisk/IR/FriskOps.cpp:825-888) with waves of 64 lanes and
+// per-wave granularity kM x kN (32 x 32 for the MFMA atoms used here).
+static void wave_partition(int policy, int64_t M, int64_t N, int num_waves, int kM, int kN, int* wm, int* wn) {
+  int64_t m_w = 1, n_w = num_waves;
+  if (M == 0 || N == 0 || num_waves == 0) { *wm = 1; *wn = 1; return; }
+  if (policy == FRISK_POLICY_FULL_ROW) {
+    m_w = num_waves;
+    if (M % (m_w * kM) != 0) {
+      int64_t max_m = std::max<int64_t>(1, M / kM);
+      m_w = std::max<int64_t>(1, std::min<int64_t>(num_waves, max_m));
+    }
+    n_w = std::max<int64_t>(1, num_waves / m_w);
+  } else if (policy == FRISK_POLICY_FULL_COL) {
+    n_w = num_waves;
+    if (N % (n_w * kN) != 0) {
+      int64_t max_n = std::max<int64_t>(1, N / kN);
+      n_w = std::max<int64_t>(1, std::min<int64_t>(num_waves, max_n));
+    }
+    m_w = std::max<int64_t>(1, num_waves / n_w);
+  } else {
+    float ideal = (float)M / (float)N;
+    float best = INFINITY;
+    for (int64_t m = 1; m <= num_waves; ++m) {
+      if (num_waves % m) continue;
+      int64_t n = num_waves / m;
+      float mp = (float)M / (float)(m * kM), np = (float)N / (float)(n * kN);
+      if (mp < 1 || np < 1) continue;
+      float score = std::fabs(mp / np - ideal);
+      if (score < best) { best = score; m_w = m; n_w = n; }
+    }
+  }
+  *wm = (int)std::max<int64_t>(1, m_w);
+  *wn = (int)std::max<int64_t>(1, n_w);
+}
+
+static int validate(const frisk_gemm_desc* d) {
+  if (!d) return fail(FRISK_ERR_NULL, "descriptor is null");
+  if (d->abi_version != FRISK_HIP_ABI_VERSION)
+    return fail(FRISK_ERR_ABI, "descriptor abi_version %d, library %d", d->abi_version, FRISK_HIP_ABI_VERSION);
+  const int ab = d->dtype_ab, acc = d->dtype_acc, out = d->dtype_out;
+  bool ok = false;
+  switch (ab) {
+    case FRISK_F32: ok = acc == FRISK_F32 && out == FRISK_F32; break;
+    case FRISK_F16: ok = acc == FRISK_F32 && (out == FRISK_F16 || out == FRISK_F32); break;
+    case FRISK_BF16: ok = acc == FRISK_F32 && (out == FRISK_BF16 || out == FRISK_F32); break;
+    case FRISK_I8: ok = acc == FRISK_I32 && (out == FRISK_I32 || out == FRISK_F16 || out == FRISK_F32); break;
+    case FRISK_E4M3: ok = acc == FRISK_F32 && (out == FRISK_BF16 || out == FRISK_F16 || out == FRISK_F32); break;
+    default: ok = false;
+  }
+  if (!ok) return fail(FRISK_ERR_DTYPE, "unsupported element types: ab=%d acc=%d out=%d", ab, acc, out);
+  if (d->epilogue < FRISK_EPI_NONE || d->epilogue > FRISK_EPI_TENSOR_SCALE)
+    return fail(FRISK_ERR_EPILOGUE, "unknown epilogue %d", d->epilogue);
+  if (out == FRISK_I32 && d->epilogue != FRISK_EPI_NONE)
+    return fail(FRISK_ERR_EPILOGUE, "int32 output carries the raw accumulators; scales need a floating output type");
+  if (d->policy < FRISK_POLICY_SQUARE || d->policy > FRISK_POLICY_FULL_COL)
+    return fail(FRISK_ERR_TILE, "unknown wave policy %d", d->policy);
+  if (d->M < 0 || d->N < 0 || d->K < 0) return fail(FRISK_ERR_SHAPE, "negative extent M=%lld N=%lld K=%lld", (long long)d->M, (long long)d->N, (long long)d->K);
+  if (d->M > INT32_MAX || d->N > INT32_MAX || d->K > INT32_MAX) return fail(FRISK_ERR_SHAPE, "extent exceeds 2^31-1");
+  const int64_t a_cols = d->transA ? d->M : d->K, b_cols = d->transB ? d->K : d->N;
+  if (d->lda < std::max<int64_t>(1, a_cols)) return fail(FRISK_ERR_SHAPE, "lda=%lld smaller than the stored row length %lld", (long long)d->lda, (long long)a_cols);
+  if (d->ldb < std::max<int64_t>(1, b_cols)) return fail(FRISK_ERR_SHAPE, "ldb=%lld smaller than the stored row length %lld", (long long)d->ldb, (long long)b_cols);
+  if (d->ldc < std::max<int64_t>(1, d->N)) return fail(FRISK_ERR_SHAPE, "ldc=%lld smaller than N=%lld", (long long)d->ldc, (long long)d->N);
+  const int es = elem_size(ab), os = elem_size(out);
+  if ((d->lda * es) % 16 || (d->ldb * es) % 16) return fail(FRISK_ERR_ALIGNMENT, "rows of A and B must start on 16-byte boundaries (lda, ldb in bytes multiples of 16)");
+  if ((d->ldc * os) % 16) return fail(FRISK_ERR_ALIGNMENT, "rows of C must start on 16-byte boundaries");
+  return FRISK_OK;
+}
+
+static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, int mn, int bk, int nw) {
+  TileShape t{kcontig ? mn : bk, (kcontig ? bk : mn) * es, kcontig, es, fragb, mn, bk};
+  Swizzle s = default_swizzle(kcontig, es, t.rowb);
+  L->rows = t.rows;
+  L->row_bytes = t.rowb;
+  L->k_contiguous = kcontig;
+  L->row_shift = s.sh;
+  L->row_mask = s.mk;
+  L->chunk_shift = s.cs;
+  L->read_instr = es == 4 ? 3 : (kcontig ? 0 : (es == 2 ? 1 : 2));
+  int atoms = mn / 32 < 4 ? mn / 32 : 4;
+  int n_access = atoms * ((bk * es) / (2 * fragb)) * frag_instr_count(kcontig, es, fragb);
+  L->read_cycles = n_access ? (float)swizzle_read_cycles(t, s) / (float)n_access : 0.f;
+  // the direct-to-LDS transfer writes 64 consecutive 16-byte slots: no conflicts by construction
+  L->write_cycles = 16.f;
+  (void)nw;
+}
+
+static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan) {
+  int st = validate(d);
+  if (st != FRISK_OK) return st;
+  if (!plan) return fail(FRISK_ERR_NULL, "plan is null");
+  std::memset(plan, 0, sizeof *plan);
+  plan->kernel_id = -1;
+  const int es = elem_size(d->dtype_ab), os = elem_size(d->dtype_out);
+  plan->flops = 2.0 * (double)d->M * (double)d->N * (double)d->K;
+  plan->bytes = (double)d->M * d->K * es + (double)d->K * d->N * es + (double)d->M * d->N * os;
+  if (d->epilogue == FRISK_EPI_ROW_COL_SCALE) plan->bytes += 4.0 * ((double)d->M + (double)d->N);
+  if (d->epilogue == FRISK_EPI_TENSOR_SCALE) plan->bytes += 8.0;
+  plan->split_k = 1;
+  plan->stages = 2;
+
+  const auto& ks = kernels();
+  int best = -1;
+  int64_t best_tiles = 0;
+  bool any_layout = false, tile_requested = d->tile_m || d->tile_n || d->tile_k || d->waves_m || d->waves_n;
+  for (size_t i = 0; i < ks.size(); ++i) {
+    const KernelEntry* k = ks[i];
+    if (k->dtype != d->dtype_ab || k->transA != (d->transA != 0) || k->transB != (d->transB != 0)) continue;
+    any_layout = true;
+    if (d->tile_m && d->tile_m != k->bm) continue;
+    if (d->tile_n && d->tile_n != k->bn) continue;
+    if (d->tile_k && d->tile_k != k->bk) continue;
+    if (d->waves_m && d->waves_m != k->wm) continue;
+    if (d->waves_n && d->waves_n != k->wn) continue;
+    if (d->M % k->bm || d->N % k->bn || d->K % k->bk) continue;
+    int64_t tiles = (d->M / k->bm) * (d->N / k->bn);
+    // largest tile that still gives every CU a work-group; otherwise the most work-groups
+    bool better;
+    if (best < 0) better = true;
+    else {
+      const KernelEntry* b = ks[best];
+      bool fills = tiles >= 256, bfills = best_tiles >= 256;
+      if (fills != bfills) better = fills;
+      else if (fills) better = (int64_t)k->bm * k->bn > (int64_t)b->bm * b->bn;
+      else better = tiles > best_tiles;
+    }
+    if (better) { best = (int)i; best_tiles = tiles; }
+  }
+  if (d->M == 0 || d->N == 0) {  // nothing to compute
+    plan->grid_x = plan->grid_y = 0;
+    return FRISK_OK;
+  }
+  if (best < 0) {
+    if (!any_layout) return fail(FRISK_ERR_DTYPE, "no kernel compiled for dtype %d transA=%d transB=%d", d->dtype_ab, d->transA, d->transB);
+    if (tile_requested)
+      return fail(FRISK_ERR_TILE, "no compiled kernel with tile %dx%dx%d waves %dx%d divides M=%lld N=%lld K=%lld", d->tile_m, d->tile_n,
+                  d->tile_k, d->waves_m, d->waves_n, (long long)d->M, (long long)d->N, (long long)d->K);
+    return fail(FRISK_ERR_SHAPE, "M=%lld N=%lld K=%lld is not a multiple of any compiled tile", (long long)d->M, (long long)d->N, (long long)d->K);
+  }
+  const KernelEntry* k = ks[best];
+  if (k->lds_bytes > 160 * 1024) return fail(FRISK_ERR_LDS, "tile needs %d bytes of LDS", k->lds_bytes);
+  plan->kernel_id = best;
+  plan->tile_m = k->bm; plan->tile_n = k->bn; plan->tile_k = k->bk;
+  plan->waves_m = k->wm; plan->waves_n = k->wn; plan->threads = k->wm * k->wn * 64;
+  plan->mfma_m = 32; plan->mfma_n = 32; plan->mfma_k = mfma_k(d->dtype_ab);
+  plan->lds_bytes = k->lds_bytes;
+  plan->grid_x = (int)(d->N / k->bn);
+  plan->grid_y = (int)(d->M / k->bm);
+  plan->xcd_remap = ((int64_t)plan->grid_x * plan->grid_y) % 8 == 0;
+  fill_layout(&plan->lds_a, !d->transA, es, frag_bytes(d->dtype_ab), k->bm, k->bk, k->wm * k->wn);
+  fill_layout(&plan->lds_b, d->transB != 0, es, frag_bytes(d->dtype_ab), k->bn, k->bk, k->wm * k->wn);
+  plan->workspace_bytes = 0;
+  return FRISK_OK;
+}
+
+// rows of tiles walked together so that the work-groups resident on one XCD form a compact block
+static int group_rows(int tiles_m, int tiles_n) {
+  int64_t total = (int64_t)tiles_m * tiles_n;
+  int64_t per_xcd = std::max<int64_t>(1, std::min<int64_t>(total / 8, 32));
+  int g = 1;
+  while ((int64_t)(2 * g) * (2 * g) <= per_xcd) g *= 2;
+  return std::max(1, std::min(g, tiles_m));
+}
+
+static int device_ok() {
+  static int cached = -1;
+  if (cached >= 0) return cached;
+  int dev = 0;
+  hipDeviceProp_t prop;
+  if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
+  cached = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
+  return cached;
+}
+
+}  // namespace frisk
+
+using namespace frisk;
+
+extern "C" {
+
+int frisk_hip_abi_version(void) { return FRISK_HIP_ABI_VERSION; }
+
+const char* frisk_hip_last_error(void) { return g_last_error.c_str(); }
+
+int frisk_hip_plan(const frisk_gemm_desc* desc, frisk_gemm_plan* plan) { return make_plan(desc, plan); }
+
+size_t frisk_hip_workspace_bytes(const frisk_gemm_desc* desc) {
+  frisk_gemm_plan plan;
+  if (make_plan(desc, &plan) != FRISK_OK) return 0;
+  return plan.workspace_bytes;
+}
+
+int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, void* C, const float* scaleA,
+                   const float* scaleB, void* workspace, size_t workspace_bytes, void* stream) {
+  frisk_gemm_plan plan;
+  int st = make_plan(desc, &plan);
+  if (st != FRISK_OK) return st;
+  if (desc->M == 0 || desc->N == 0) return FRISK_OK;
+  if (!A || !B || !C) return fail(FRISK_ERR_NULL, "A, B and C must be device pointers");
+  if (desc->epilogue != FRISK_EPI_NONE && (!scaleA || !scaleB)) return fail(FRISK_ERR_EPILOGUE, "epilogue %d needs scaleA and scaleB", desc->epilogue);
+  if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) return fail(FRISK_ERR_ALIGNMENT, "A, B and C must be 16-byte aligned");
+  if (desc->epilogue == FRISK_EPI_ROW_COL_SCALE && ((uintptr_t)scaleB & 15)) return fail(FRISK_ERR_ALIGNMENT, "scaleB must be 16-byte aligned");
+  if (plan.workspace_bytes > 0 && (!workspace || workspace_bytes < plan.workspace_bytes))
+    return fail(FRISK_ERR_WORKSPACE, "needs %zu bytes of workspace", plan.workspace_bytes);
+  if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
+  if (desc->K == 0) return fail(FRISK_ERR_SHAPE, "K = 0 is not launched; fill C instead");
+
+  GemmParams p;
+  p.A = A; p.B = B; p.C = C; p.scaleA = scaleA; p.scaleB = scaleB;
+  p.lda = desc->lda; p.ldb = desc->ldb; p.ldc = desc->ldc;
+  p.M = (int)desc->M; p.N = (int)desc->N; p.K = (int)desc->K;
+  p.tiles_m = plan.grid_y; p.tiles_n = plan.grid_x;
+  p.group_m = group_rows(p.tiles_m, p.tiles_n);
+  p.xcd_remap = plan.xcd_remap;
+  p.epilogue = desc->epilogue; p.dtype_out = desc->dtype_out; p.accumulate = desc->clear_accum ? 0 : 1;
+  hipError_t e = kernels()[plan.kernel_id]->launch(p, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "launch of %s failed: %s", kernels()[plan.kernel_id]->name, hipGetErrorString(e));
+  return FRISK_OK;
+}
+
+float frisk_hip_lds_access_cycles(int instr, const int32_t* lane_byte_addr) {
+  if (!lane_byte_addr) return -1.f;
+  int addr[64];
+  for (int i = 0; i < 64; ++i) addr[i] = lane_byte_addr[i];
+  return (float)lds_access_cycles(instr == 2 ? 1 : instr, addr);
+}
+
+int32_t frisk_hip_lds_offset(const frisk_lds_layout* L, int32_t row, int32_t col_byte) {
+  if (!L) return -1;
+  return lds_offset(L->row_bytes, Swizzle{L->row_shift, L->row_mask, L->chunk_shift}, row, col_byte);
+}
+
+int frisk_hip_wave_partition(int policy, int tile_m, int tile_n, int num_waves, int* waves_m, int* waves_n) {
+  if (!waves_m || !waves_n) return fail(FRISK_ERR_NULL, "output pointers are null");
+  if (policy < FRISK_POLICY_SQUARE || policy > FRISK_POLICY_FULL_COL) return fail(FRISK_ERR_TILE, "unknown wave policy %d", policy);
+  wave_partition(policy, tile_m, tile_n, num_waves, 32, 32, waves_m, waves_n);
+  return FRISK_OK;
+}
+
+int frisk_hip_kernel_count(void) { return (int)kernels().size(); }
+const char* frisk_hip_kernel_name(int id) {
+  if (id < 0 || id >= (int)kernels().size()) return nullptr;
+  return kernels()[id]->name;
+}
+
+}  // extern "C"

@@ -1,0 +1,196 @@
+// LDS addressing and bank-conflict cost model for gfx950, shared by the device
+// kernels (compile-time), the planner (run time) and the C ABI.
+//
+// This takes the place of two things in the reference:
+//  * the shared-memory swizzle selection by column count
+//    (buildAmpereSharedLayout / buildHopperSharedLayout,
+//    lib/Dialect/Frisk/IR/FriskOps.cpp:560-618, built on
+//    makeQuarter/Half/FullBankSwizzle :500-558), and
+//  * the bank histogram of exp/layout/gemm_layout_tool.cpp:135-208, which
+//    models 32 banks x 4 B under a row-major sweep and counts elements of the
+//    same dword as conflicts.
+// Here a layout is scored with the lane->address sets of the instructions the
+// kernel really issues, against a model of the gfx950 LDS fitted to device
+// measurements (cycles per wave-wide instruction, 16 waves resident):
+//   - 64 banks x 4 B; requests for the same dword are one request.
+//   - ds_read_b128: the wave is served as two halves of 32 lanes.  A half is
+//     made of 8 quads (4 consecutive lanes); a quad whose lanes collide needs
+//     as many passes as its worst bank; 4 quad-passes issue per cycle; the half
+//     also needs at least as many cycles as its most loaded bank.
+//     (linear 4, stride-32B 8, unswizzled 128-B rows 32, broadcast 4 cycles.)
+//   - ds_read_b64 and the transpose reads ds_read_b64_tr_b16/_b8: two halves
+//     of 32 lanes, each costs its most loaded bank; never below 3 cycles.
+//   - ds_read_b32: all 64 lanes at once over 32 dword-interleaved banks;
+//     never below 3 cycles.
+// Everything is constexpr so the kernel templates pick their swizzle with the
+// same code the planner reports.
+#pragma once
+#include <stdint.h>
+
+#if defined(__HIPCC__) || defined(__HIP__)
+#define FRISK_HD __host__ __device__ constexpr
+#else
+#define FRISK_HD constexpr
+#endif
+
+namespace frisk {
+
+enum LdsInstr { LDS_READ_B128 = 0, LDS_READ_B64 = 1, LDS_READ_B64_TR16 = 1, LDS_READ_B64_TR8 = 1, LDS_READ_B32 = 3 };
+
+// XOR swizzle: 16-byte chunk c of row r is stored at chunk c ^ (((r >> sh) & mk) << cs)
+struct Swizzle {
+  int sh, mk, cs;
+};
+
+FRISK_HD int lds_swz(Swizzle s, int row) { return ((row >> s.sh) & s.mk) << s.cs; }
+FRISK_HD int lds_offset(int rowb, Swizzle s, int row, int colbyte) {
+  return row * rowb + ((((colbyte >> 4) ^ lds_swz(s, row)) << 4) | (colbyte & 15));
+}
+
+// ---- fragment addressing (32x32 MFMA atoms; lane l serves row/col l%32, K-group l/32)
+// K-contiguous tile: instruction q of FRAGB/16 (or the single 4-byte read when FRAGB == 4)
+FRISK_HD int frag_addr_kc(int rowb, Swizzle s, int fragb, int lane, int mn0, int kb0, int q) {
+  int row = mn0 + (lane & 31);
+  int kb = kb0 + (lane >> 5) * fragb + 16 * q;
+  return lds_offset(rowb, s, row, kb);
+}
+// MN-contiguous tile (rows = K).  16- and 8-bit elements use the transpose
+// reads: in a block of 16 lanes, lane L presents K-row L / lpr and the 8 bytes
+// at column-group L % lpr; it receives column (l % 16) of the block's K rows.
+// 32-bit elements read their single value directly.
+FRISK_HD int frag_addr_mc(int rowb, Swizzle s, int es, int fragb, int lane, int mn0, int kb0, int q) {
+  if (es == 4) return lds_offset(rowb, s, kb0 / 4 + (lane >> 5), (mn0 + (lane & 31)) * 4);
+  int kpi = es == 2 ? 4 : 8;
+  int lpr = 16 / kpi;
+  int blk = lane >> 4, l16 = lane & 15;
+  int col0 = mn0 + 16 * (blk & 1);
+  int krow = kb0 / es + (blk >> 1) * (fragb / es) + q * kpi + l16 / lpr;
+  int colbyte = (col0 + (l16 % lpr) * (8 / es)) * es;
+  return lds_offset(rowb, s, krow, colbyte);
+}
+FRISK_HD int frag_instr_count(bool kcontig, int es, int fragb) { return (es == 4) ? 1 : (kcontig ? fragb / 16 : fragb / 8); }
+FRISK_HD int frag_instr_kind(bool kcontig, int es) { return es == 4 ? LDS_READ_B32 : (kcontig ? LDS_READ_B128 : LDS_READ_B64); }
+FRISK_HD int frag_instr_bytes(bool kcontig, int es) { return es == 4 ? 4 : (kcontig ? 16 : 8); }
+
+// ---- cost of one wave-wide access; addr = 64 byte addresses
+// worst number of distinct dwords any bank must deliver to lanes [first, first+count)
+FRISK_HD int lds_group_load(const int* addr, int first, int count, int width, int nbanks) {
+  int dws[256] = {};
+  int n = 0;
+  for (int i = 0; i < count; ++i)
+    for (int w = 0; w < width; ++w) {
+      int dw = (addr[first + i] >> 2) + w;
+      bool dup = false;
+      for (int t = 0; t < n; ++t) dup = dup || (dws[t] == dw);
+      if (!dup) dws[n++] = dw;
+    }
+  int hist[64] = {};
+  int worst = 0;
+  for (int t = 0; t < n; ++t) {
+    int b = dws[t] % nbanks;
+    hist[b] += 1;
+    if (hist[b] > worst) worst = hist[b];
+  }
+  return worst;
+}
+
+FRISK_HD int lds_access_cycles(int instr, const int* addr) {
+  if (instr == LDS_READ_B128) {
+    int total = 0;
+    for (int h = 0; h < 2; ++h) {
+      int qsum = 0;
+      for (int q = 0; q < 8; ++q) qsum += lds_group_load(addr, 32 * h + 4 * q, 4, 4, 64);
+      int load = lds_group_load(addr, 32 * h, 32, 4, 64);
+      int issue = (qsum + 3) / 4;
+      total += load > issue ? load : issue;
+    }
+    return total;
+  }
+  if (instr == LDS_READ_B64) {
+    int total = 0;
+    for (int h = 0; h < 2; ++h) total += lds_group_load(addr, 32 * h, 32, 2, 64);
+    return total < 3 ? 3 : total;
+  }
+  int c = lds_group_load(addr, 0, 64, 1, 32);
+  return c < 3 ? 3 : c;
+}
+
+// ---- score of a swizzle for one operand tile: LDS cycles spent on fragment
+// reads per K step of a (wave tile rows) x (tile K) slab, all atoms and K steps.
+struct TileShape {
+  int rows, rowb;  // as stored
+  bool kcontig;
+  int es, fragb;   // element bytes, fragment bytes per lane per MFMA
+  int mn, bk;      // logical extent along M (or N) and K, elements
+};
+
+FRISK_HD int swizzle_read_cycles(TileShape t, Swizzle s) {
+  int total = 0;
+  int ksteps = (t.bk * t.es) / (2 * t.fragb);
+  int ninstr = frag_instr_count(t.kcontig, t.es, t.fragb);
+  int kind = frag_instr_kind(t.kcontig, t.es);
+  // bank behaviour repeats with the atom position beyond what the swizzle sees; sample the first atoms
+  int atoms = t.mn / 32 < 4 ? t.mn / 32 : 4;
+  for (int a = 0; a < atoms; ++a)
+    for (int ks = 0; ks < ksteps; ++ks)
+      for (int q = 0; q < ninstr; ++q) {
+        int addr[64] = {};
+        for (int l = 0; l < 64; ++l)
+          addr[l] = t.kcontig ? frag_addr_kc(t.rowb, s, t.fragb, l, a * 32, ks * 2 * t.fragb, q)
+                              : frag_addr_mc(t.rowb, s, t.es, t.fragb, l, a * 32, ks * 2 * t.fragb, q);
+        total += lds_access_cycles(kind, addr);
+      }
+  return total;
+}
+
+// A swizzle is usable when it stays inside the row and repeats with the row
+// step of one wave of the direct-to-LDS stager (nw waves, 1 KiB per transfer),
+// so a lane fetches the same logical chunk on every transfer.
+FRISK_HD bool swizzle_usable(TileShape t, Swizzle s, int nw) {
+  int chunks = t.rowb / 16;
+  if ((s.mk << s.cs) >= chunks && s.mk != 0) return false;
+  int rpc = 1024 / t.rowb;
+  int period = (s.mk + 1) << s.sh;
+  return s.mk == 0 || ((nw * rpc) % period) == 0;
+}
+
+// Exhaustive search over (sh, mk, cs); ties go to the smaller mask, then the
+// smaller chunk shift, then the smaller row shift (the least surprising layout).
+FRISK_HD Swizzle choose_swizzle(TileShape t, int nw) {
+  Swizzle best = {0, 0, 0};
+  int best_cost = swizzle_read_cycles(t, best);
+  const int masks[4] = {1, 3, 7, 15};
+  for (int mi = 0; mi < 4; ++mi)
+    for (int cs = 0; cs < 4; ++cs)
+      for (int sh = 0; sh < 4; ++sh) {
+        Swizzle s = {sh, masks[mi], cs};
+        if (!swizzle_usable(t, s, nw)) continue;
+        int c = swizzle_read_cycles(t, s);
+        if (c < best_cost) { best_cost = c; best = s; }
+      }
+  return best;
+}
+
+// The swizzles compiled into the kernels: the result of choose_swizzle for the
+// tile shapes in use, frozen as constants (a host test re-runs the search and
+// compares).  K-contiguous tiles read with ds_read_b128 want 16 consecutive
+// rows to land in 16 different 16-byte bank groups: XOR the chunk with
+// (row >> 1).  Tiles whose rows run along M or N are read by transpose reads
+// that touch 4 (16-bit) or 8 (8-bit) consecutive K rows per half wave, 64 or
+// 32 bytes wide: XOR with the K row in units of that width.
+FRISK_HD Swizzle default_swizzle(bool kcontig, int es, int rowb) {
+  int chunks = rowb / 16;
+  if (kcontig) {
+    int mk = chunks >= 8 ? 7 : chunks - 1;
+    return Swizzle{es == 4 ? 0 : 1, mk, 0};
+  }
+  if (es == 4) return Swizzle{0, 0, 0};
+  if (es == 2) {
+    int units = chunks >> 2;  // 64-byte units
+    return Swizzle{0, units >= 4 ? 3 : (units >= 2 ? 1 : 0), 2};
+  }
+  if (rowb >= 256) return Swizzle{0, 7, 1};
+  return Swizzle{1, 3, 1};
+}
+
+}  // namespace frisk

@@ -1,0 +1,143 @@
+"""ctypes binding of libfrisk_hip.so (include/frisk_hip.h).
+
+This is the thin host layer the builder front end and the benchmarks use to
+reach the HIP kernels.  It never falls back to another implementation: if the
+library is missing the import fails, and every non-zero status raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libfrisk_hip.so")
+
+ABI_VERSION = 1
+F32, F16, BF16, I8, E4M3, I32 = 0, 1, 2, 3, 4, 5
+EPI_NONE, EPI_ROW_COL_SCALE, EPI_TENSOR_SCALE = 0, 1, 2
+POLICY_SQUARE, POLICY_FULL_ROW, POLICY_FULL_COL = 0, 1, 2
+DTYPE_BYTES = {F32: 4, F16: 2, BF16: 2, I8: 1, E4M3: 1, I32: 4}
+DTYPE_NAMES = {"fp32": F32, "f32": F32, "fp16": F16, "f16": F16, "bf16": BF16, "int8": I8, "i8": I8,
+               "e4m3fn": E4M3, "e4m3": E4M3, "fp8": E4M3, "int32": I32, "i32": I32}
+ACC_OF = {F32: F32, F16: F32, BF16: F32, I8: I32, E4M3: F32}
+
+STATUS_NAMES = {0: "OK", 1: "ERR_NULL", 2: "ERR_ABI", 3: "ERR_DTYPE", 4: "ERR_SHAPE", 5: "ERR_TILE", 6: "ERR_LDS",
+                7: "ERR_EPILOGUE", 8: "ERR_WORKSPACE", 9: "ERR_DEVICE", 10: "ERR_ALIGNMENT"}
+
+
+class GemmDesc(ctypes.Structure):
+    _fields_ = [("abi_version", ctypes.c_int32), ("dtype_ab", ctypes.c_int32), ("dtype_acc", ctypes.c_int32),
+                ("dtype_out", ctypes.c_int32), ("M", ctypes.c_int64), ("N", ctypes.c_int64), ("K", ctypes.c_int64),
+                ("lda", ctypes.c_int64), ("ldb", ctypes.c_int64), ("ldc", ctypes.c_int64),
+                ("transA", ctypes.c_uint8), ("transB", ctypes.c_uint8), ("clear_accum", ctypes.c_uint8),
+                ("reserved0", ctypes.c_uint8), ("epilogue", ctypes.c_int32), ("policy", ctypes.c_int32),
+                ("tile_m", ctypes.c_int32), ("tile_n", ctypes.c_int32), ("tile_k", ctypes.c_int32),
+                ("waves_m", ctypes.c_int32), ("waves_n", ctypes.c_int32)]
+
+
+class LdsLayout(ctypes.Structure):
+    _fields_ = [("rows", ctypes.c_int32), ("row_bytes", ctypes.c_int32), ("k_contiguous", ctypes.c_int32),
+                ("row_shift", ctypes.c_int32), ("row_mask", ctypes.c_int32), ("chunk_shift", ctypes.c_int32),
+                ("read_instr", ctypes.c_int32), ("read_cycles", ctypes.c_float), ("write_cycles", ctypes.c_float)]
+
+
+class GemmPlan(ctypes.Structure):
+    _fields_ = [("kernel_id", ctypes.c_int32), ("tile_m", ctypes.c_int32), ("tile_n", ctypes.c_int32),
+                ("tile_k", ctypes.c_int32), ("waves_m", ctypes.c_int32), ("waves_n", ctypes.c_int32),
+                ("threads", ctypes.c_int32), ("mfma_m", ctypes.c_int32), ("mfma_n", ctypes.c_int32),
+                ("mfma_k", ctypes.c_int32), ("stages", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
+                ("grid_x", ctypes.c_int32), ("grid_y", ctypes.c_int32), ("split_k", ctypes.c_int32),
+                ("xcd_remap", ctypes.c_int32), ("lds_a", LdsLayout), ("lds_b", LdsLayout),
+                ("workspace_bytes", ctypes.c_size_t), ("flops", ctypes.c_double), ("bytes", ctypes.c_double)]
+
+
+class FriskHipError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("frisk_hip status %d (%s): %s" % (status, STATUS_NAMES.get(status, "?"), message))
+        self.status = status
+
+
+_lib = None
+
+EXPORTS = ["frisk_hip_abi_version", "frisk_hip_last_error", "frisk_hip_plan", "frisk_hip_workspace_bytes",
+           "frisk_hip_gemm", "frisk_hip_lds_access_cycles", "frisk_hip_lds_offset", "frisk_hip_wave_partition",
+           "frisk_hip_kernel_count", "frisk_hip_kernel_name"]
+
+
+def lib():
+    """Loads libfrisk_hip.so; raises if it has not been built (python -m frisk_amd.build)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError("libfrisk_hip.so is not built: run `python -m frisk_amd.build` (needs hipcc)")
+    L = ctypes.CDLL(LIB_PATH)
+    L.frisk_hip_abi_version.restype = ctypes.c_int
+    L.frisk_hip_last_error.restype = ctypes.c_char_p
+    L.frisk_hip_plan.argtypes = [ctypes.POINTER(GemmDesc), ctypes.POINTER(GemmPlan)]
+    L.frisk_hip_workspace_bytes.restype = ctypes.c_size_t
+    L.frisk_hip_workspace_bytes.argtypes = [ctypes.POINTER(GemmDesc)]
+    L.frisk_hip_gemm.argtypes = [ctypes.POINTER(GemmDesc), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                 ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    L.frisk_hip_lds_access_cycles.restype = ctypes.c_float
+    L.frisk_hip_lds_access_cycles.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_int32)]
+    L.frisk_hip_lds_offset.restype = ctypes.c_int32
+    L.frisk_hip_lds_offset.argtypes = [ctypes.POINTER(LdsLayout), ctypes.c_int32, ctypes.c_int32]
+    L.frisk_hip_wave_partition.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                           ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
+    L.frisk_hip_kernel_count.restype = ctypes.c_int
+    L.frisk_hip_kernel_name.restype = ctypes.c_char_p
+    L.frisk_hip_kernel_name.argtypes = [ctypes.c_int]
+    if L.frisk_hip_abi_version() != ABI_VERSION:
+        raise ImportError("libfrisk_hip.so has ABI %d, binding expects %d" % (L.frisk_hip_abi_version(), ABI_VERSION))
+    _lib = L
+    return L
+
+
+def _check(status):
+    if status != 0:
+        raise FriskHipError(status, lib().frisk_hip_last_error().decode())
+
+
+def make_desc(dtype_ab, M, N, K, dtype_out=None, transA=False, transB=False, lda=None, ldb=None, ldc=None,
+              clear_accum=True, epilogue=EPI_NONE, policy=POLICY_SQUARE, tile=(0, 0, 0), waves=(0, 0)):
+    d = GemmDesc()
+    d.abi_version = ABI_VERSION
+    d.dtype_ab = dtype_ab
+    d.dtype_acc = ACC_OF.get(dtype_ab, F32)
+    d.dtype_out = dtype_ab if dtype_out is None else dtype_out
+    d.M, d.N, d.K = M, N, K
+    d.lda = lda if lda is not None else (M if transA else K)
+    d.ldb = ldb if ldb is not None else (K if transB else N)
+    d.ldc = ldc if ldc is not None else N
+    d.transA, d.transB, d.clear_accum = int(transA), int(transB), int(clear_accum)
+    d.epilogue, d.policy = epilogue, policy
+    d.tile_m, d.tile_n, d.tile_k = tile
+    d.waves_m, d.waves_n = waves
+    return d
+
+
+def plan(desc):
+    p = GemmPlan()
+    _check(lib().frisk_hip_plan(ctypes.byref(desc), ctypes.byref(p)))
+    return p
+
+
+def gemm(desc, A_ptr, B_ptr, C_ptr, scaleA_ptr=None, scaleB_ptr=None, workspace_ptr=None, workspace_bytes=0, stream=None):
+    """Asynchronous launch on `stream` (a raw hipStream_t value or None). Pointers are raw device addresses."""
+    _check(lib().frisk_hip_gemm(ctypes.byref(desc), A_ptr, B_ptr, C_ptr, scaleA_ptr, scaleB_ptr, workspace_ptr,
+                                workspace_bytes, stream))
+
+
+def wave_partition(policy, tile_m, tile_n, num_waves):
+    wm, wn = ctypes.c_int(), ctypes.c_int()
+    _check(lib().frisk_hip_wave_partition(policy, tile_m, tile_n, num_waves, ctypes.byref(wm), ctypes.byref(wn)))
+    return wm.value, wn.value
+
+
+def lds_access_cycles(instr, lane_addrs):
+    arr = (ctypes.c_int32 * 64)(*lane_addrs)
+    return lib().frisk_hip_lds_access_cycles(instr, arr)
+
+
+def kernel_names():
+    L = lib()
+    return [L.frisk_hip_kernel_name(i).decode() for i in range(L.frisk_hip_kernel_count())]

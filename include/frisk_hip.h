@@ -1,0 +1,156 @@
+/*
+ * frisk_hip.h -- C ABI of libfrisk_hip.so: the gfx950 (MI355X) execution path
+ * of the tiled GEMM that the Frisk dialect describes.
+ *
+ * The reference (Xiebaokang/frisk) stops at IR construction: its pybind11
+ * module exposes only `init_ffi_ir` (ffi/ffi.h:12, ffi/ffi.cpp:3-7) and leaves
+ * the slot for a compile/launch surface commented out (`init_ffi_passes`,
+ * ffi/ffi.h:14).  The entry points below are what a binding in that slot calls:
+ * one descriptor carrying the attributes of `frisk.gemm`
+ * (include/Dialect/Frisk/IR/FriskOps.td:248-289: transA, transB, M, N, K,
+ * clear_accum) plus what the surrounding `frisk.parallel`/`frisk.alloc_buffer`/
+ * `frisk.copy` ops fix (tile shape, wave grid, element types; tmp/ir.mlir:1-17),
+ * and raw device pointers.
+ *
+ * Rules of the boundary: plain C types only; every function returns a status
+ * code and never throws; the caller owns all device buffers and the stream; a
+ * launch is asynchronous on the given stream; the library never allocates or
+ * synchronises behind the caller's back.
+ */
+#ifndef FRISK_HIP_H_
+#define FRISK_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FRISK_HIP_ABI_VERSION 1
+
+/* element types; `dtype = "fp16" | "fp32" | "e4m3fn" ...` strings of
+ * create_alloc_buffer_op (ffi/ir.cpp:407-429) map onto these */
+typedef enum frisk_dtype {
+  FRISK_F32 = 0,
+  FRISK_F16 = 1,
+  FRISK_BF16 = 2,
+  FRISK_I8 = 3,
+  FRISK_E4M3 = 4, /* OCP e4m3fn, the reference's Float8E4M3FNType (ffi/ir.cpp:164,411) */
+  FRISK_I32 = 5
+} frisk_dtype;
+
+typedef enum frisk_epilogue {
+  FRISK_EPI_NONE = 0,          /* out = cast(acc)                                    */
+  FRISK_EPI_ROW_COL_SCALE = 1, /* out = cast((float(acc) * scaleA[m]) * scaleB[n])   */
+  FRISK_EPI_TENSOR_SCALE = 2   /* out = cast((float(acc) * scaleA[0]) * scaleB[0])   */
+} frisk_epilogue;
+
+/* GemmWarpPolicy of the dialect (include/Dialect/Frisk/IR/FriskEnums.td:16-25) */
+typedef enum frisk_wave_policy { FRISK_POLICY_SQUARE = 0, FRISK_POLICY_FULL_ROW = 1, FRISK_POLICY_FULL_COL = 2 } frisk_wave_policy;
+
+typedef enum frisk_status {
+  FRISK_OK = 0,
+  FRISK_ERR_NULL = 1,        /* a required pointer is null                            */
+  FRISK_ERR_ABI = 2,         /* descriptor abi_version mismatch                       */
+  FRISK_ERR_DTYPE = 3,       /* unsupported element-type combination                  */
+  FRISK_ERR_SHAPE = 4,       /* negative extent, leading dimension too small, overflow */
+  FRISK_ERR_TILE = 5,        /* requested tile / wave grid not available              */
+  FRISK_ERR_LDS = 6,         /* tile needs more than the 160 KiB of LDS per CU        */
+  FRISK_ERR_EPILOGUE = 7,    /* epilogue needs scales that were not given             */
+  FRISK_ERR_WORKSPACE = 8,   /* workspace missing or too small                        */
+  FRISK_ERR_DEVICE = 9,      /* no gfx950 device / HIP runtime error                  */
+  FRISK_ERR_ALIGNMENT = 10   /* a pointer or leading dimension breaks 16-byte alignment */
+} frisk_status;
+
+/*
+ * One GEMM:  C[M,N] (+)= op(A)[M,K] . op(B)[K,N]
+ *   transA = 0: A stored row-major [M][K], lda >= K;  transA = 1: stored [K][M], lda >= M
+ *   transB = 0: B stored row-major [K][N], ldb >= N;  transB = 1: stored [N][K], ldb >= K
+ *   C stored row-major [M][N], ldc >= N.  Leading dimensions are in elements.
+ *   clear_accum = 1: C = A.B ;  clear_accum = 0: C = C + A.B  (frisk.gemm, FriskOps.td:262)
+ * Supported (dtype_ab -> dtype_acc -> dtype_out):
+ *   F32->F32->F32, F16->F32->{F16,F32}, BF16->F32->{BF16,F32},
+ *   I8->I32->{I32, F16 with ROW_COL_SCALE}, E4M3->F32->{BF16,F32} (NONE or TENSOR_SCALE)
+ * tile_* and waves_* = 0 let the planner choose.
+ */
+typedef struct frisk_gemm_desc {
+  int32_t abi_version; /* FRISK_HIP_ABI_VERSION */
+  int32_t dtype_ab, dtype_acc, dtype_out;
+  int64_t M, N, K;
+  int64_t lda, ldb, ldc;
+  uint8_t transA, transB, clear_accum, reserved0;
+  int32_t epilogue;
+  int32_t policy;                 /* frisk_wave_policy */
+  int32_t tile_m, tile_n, tile_k; /* block tile = the M,N,K attrs of the tile-level frisk.gemm */
+  int32_t waves_m, waves_n;       /* wave grid inside the work-group */
+} frisk_gemm_desc;
+
+/* XOR swizzle of an LDS tile: 16-byte chunk index c of row r is stored at
+ * chunk  c ^ (((r >> row_shift) & row_mask) << chunk_shift).  This is the
+ * representation of the reference's makeQuarter/Half/FullBankSwizzle layouts
+ * (lib/Dialect/Frisk/IR/FriskOps.cpp:500-558), with the parameters chosen for
+ * the gfx950 LDS instead of by the column-count rule of :560-618. */
+typedef struct frisk_lds_layout {
+  int32_t rows, row_bytes; /* tile as stored in LDS */
+  int32_t k_contiguous;    /* 1: rows index M (or N), K runs along the row */
+  int32_t row_shift, row_mask, chunk_shift;
+  int32_t read_instr;      /* 0 ds_read_b128, 1 ds_read_b64_tr_b16, 2 ds_read_b64_tr_b8, 3 ds_read_b32 */
+  float read_cycles;       /* modelled LDS cycles per wave-wide fragment read */
+  float write_cycles;      /* modelled LDS cycles per KiB staged */
+} frisk_lds_layout;
+
+typedef struct frisk_gemm_plan {
+  int32_t kernel_id;                 /* index into the compiled kernel table, -1 if none */
+  int32_t tile_m, tile_n, tile_k;
+  int32_t waves_m, waves_n, threads; /* result of the wave partition (reference: computeWarpPartition, FriskOps.cpp:825-888) */
+  int32_t mfma_m, mfma_n, mfma_k;    /* MFMA atom */
+  int32_t stages;
+  int32_t lds_bytes;                 /* total, <= 163840 */
+  int32_t grid_x, grid_y;            /* work-group grid (tiles along N, tiles along M) */
+  int32_t split_k;                   /* >1: partial sums go through the workspace */
+  int32_t xcd_remap;                 /* 1: work-group ids are remapped so each XCD owns a compact block of tiles */
+  frisk_lds_layout lds_a, lds_b;
+  size_t workspace_bytes;
+  double flops;                      /* 2.M.N.K */
+  double bytes;                      /* |A| + |B| + |C| (+ scales) */
+} frisk_gemm_plan;
+
+int frisk_hip_abi_version(void);
+
+/* thread-local text of the last non-OK status returned on this thread */
+const char* frisk_hip_last_error(void);
+
+/* Pure host: validate the descriptor and fill the plan.  Needs no GPU. */
+int frisk_hip_plan(const frisk_gemm_desc* desc, frisk_gemm_plan* plan);
+
+/* Pure host: bytes of device workspace `frisk_hip_gemm` needs for this descriptor (0 for most). */
+size_t frisk_hip_workspace_bytes(const frisk_gemm_desc* desc);
+
+/* Launch on `stream` (a hipStream_t, may be NULL for the default stream).
+ * A, B, C, scaleA, scaleB, workspace are device pointers.  scaleA/scaleB are
+ * fp32: M and N entries for ROW_COL_SCALE, one entry each for TENSOR_SCALE. */
+int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, void* C, const float* scaleA,
+                   const float* scaleB, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Pure host: modelled LDS cycles for one wave-wide access given the 64 byte
+ * addresses the lanes present.  instr: 0 ds_read_b128, 1 ds_read_b64 /
+ * ds_read_b64_tr_b16 / ds_read_b64_tr_b8, 3 ds_read_b32.  Replaces the bank
+ * histogram of the reference's layout tool (exp/layout/gemm_layout_tool.cpp:135-208). */
+float frisk_hip_lds_access_cycles(int instr, const int32_t* lane_byte_addr);
+
+/* Pure host: byte offset inside an LDS tile of element (row, col_byte) under `layout`. */
+int32_t frisk_hip_lds_offset(const frisk_lds_layout* layout, int32_t row, int32_t col_byte);
+
+/* Pure host: wave partition for a block tile (restates computeWarpPartition for 64-wide waves
+ * and 32x32 MFMA atoms). Returns FRISK_OK and writes waves_m, waves_n. */
+int frisk_hip_wave_partition(int policy, int tile_m, int tile_n, int num_waves, int* waves_m, int* waves_n);
+
+/* Number of kernels compiled into the library and a printable name for each. */
+int frisk_hip_kernel_count(void);
+const char* frisk_hip_kernel_name(int kernel_id);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FRISK_HIP_H_ */

@@ -1,0 +1,56 @@
+"""Shared helpers of the parity tests: seeded inputs from the oracle's RNG,
+device buffers through torch (plumbing only), launches through the C ABI."""
+import numpy as np
+
+import oracle as O
+
+TOL = {O.F32: 1e-4, O.F16: 1e-2, O.BF16: 1e-2, O.E4M3: 1e-2, O.I8: 1e-2}
+NAMES = {O.F32: "f32", O.F16: "f16", O.BF16: "bf16", O.I8: "i8", O.E4M3: "e4m3"}
+DEFAULT_OUT = {O.F32: O.F32, O.F16: O.F16, O.BF16: O.BF16, O.I8: O.I32, O.E4M3: O.BF16}
+
+
+def make_operand(dtype, rows, cols, seed, tensor, kind="normal", scale=1.0):
+    """rows x cols stored operand in the storage type of `dtype`"""
+    n = rows * cols
+    if dtype == O.I8:
+        return O.int8_uniform(n, seed, tensor).reshape(rows, cols)
+    if kind == "uniform":
+        f = O.uniform(n, seed, tensor, -1.0, 1.0)
+    else:
+        f = O.normal(n, seed, tensor, scale)
+    return O.encode(dtype, f).reshape(rows, cols)
+
+
+def to_dev(arr):
+    import torch
+    a = np.ascontiguousarray(arr)
+    return torch.from_numpy(a.view(np.uint8).reshape(-1).copy()).cuda()
+
+
+def from_dev(t, np_dtype, shape):
+    return t.cpu().numpy().view(np_dtype).reshape(shape)
+
+
+def run_gemm(R, dtype, A, B, transA, transB, dtype_out, M, N, K, epilogue=0, sA=None, sB=None, C_init=None,
+             clear_accum=True, tile=(0, 0, 0), waves=(0, 0)):
+    """launch through the C ABI; returns the output as a numpy array in storage type"""
+    import torch
+    dA, dB = to_dev(A), to_dev(B)
+    out_np = O.NP_STORAGE[dtype_out]
+    if C_init is None:
+        dC = torch.full((M * N * np.dtype(out_np).itemsize,), 0xFF, dtype=torch.uint8, device="cuda")
+    else:
+        dC = to_dev(C_init)
+    dsA = to_dev(np.asarray(sA, dtype=np.float32)) if sA is not None else None
+    dsB = to_dev(np.asarray(sB, dtype=np.float32)) if sB is not None else None
+    desc = R.make_desc(dtype, M, N, K, dtype_out=dtype_out, transA=transA, transB=transB, clear_accum=clear_accum,
+                       epilogue=epilogue, tile=tile, waves=waves)
+    stream = torch.cuda.current_stream().cuda_stream
+    R.gemm(desc, dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), dsA.data_ptr() if dsA is not None else None,
+           dsB.data_ptr() if dsB is not None else None, None, 0, stream)
+    torch.cuda.synchronize()
+    return from_dev(dC, out_np, (M, N))
+
+
+def stored_shapes(M, N, K, transA, transB):
+    return ((K, M) if transA else (M, K)), ((N, K) if transB else (K, N))

@@ -1,0 +1,188 @@
+"""Parity of the HIP GEMM path against the CPU oracle, through the C ABI.
+
+Bars: int8 -> int32 bit-exact; the dequant epilogue bit-exact (fixed fp32
+operation order); fp16 / bf16 / fp8 within 1e-2 and fp32 within 1e-4, both as
+max |d-r| / max(|r|, rms(R)) over all elements and as ||D-R||_F / ||R||_F.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import oracle as O
+from helpers import DEFAULT_OUT, NAMES, TOL, make_operand, run_gemm, stored_shapes
+
+pytestmark = pytest.mark.gpu
+
+BK = {O.F32: 32, O.F16: 64, O.BF16: 64, O.I8: 128, O.E4M3: 128}
+BIG = {O.F32: 128, O.F16: 256, O.BF16: 256, O.I8: 256, O.E4M3: 256}
+SMALL = {O.F32: 64, O.F16: 128, O.BF16: 128, O.I8: 128, O.E4M3: 128}
+
+
+def note(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def check(dtype, dtype_out, got, ref64):
+    r = O.compare(dtype_out, got, ref64)
+    tol = TOL[dtype]
+    assert r["nonfinite"] == 0, r
+    assert r["max_rel"] <= tol and r["fro_rel"] <= tol, (r, tol)
+    return r
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.I8, O.E4M3, O.F32])
+@pytest.mark.parametrize("transA,transB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("which", ["big", "small"])
+def test_layouts_small_shapes(hip, dtype, transA, transB, which):
+    t = BIG[dtype] if which == "big" else SMALL[dtype]
+    M, N, K = 2 * t, 3 * t, 3 * BK[dtype]
+    note(f"case layouts {NAMES[dtype]} tA={transA} tB={transB} tile={t} M={M} N={N} K={K}")
+    sa, sb = stored_shapes(M, N, K, transA, transB)
+    A = make_operand(dtype, *sa, seed=11, tensor=0, scale=0.5)
+    B = make_operand(dtype, *sb, seed=11, tensor=1, scale=0.5)
+    out_dt = DEFAULT_OUT[dtype]
+    got = run_gemm(hip, dtype, A, B, transA, transB, out_dt, M, N, K, tile=(t, t, BK[dtype]))
+    if dtype == O.I8:
+        ref = O.gemm_i32(A, B, transA, transB)
+        assert np.array_equal(got, ref)
+    else:
+        check(dtype, out_dt, got, O.gemm_f64(dtype, A, B, transA, transB))
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.E4M3, O.F32])
+def test_identity_is_exact(hip, dtype):
+    """A = I  =>  C == B bit for bit (every product is exact, every sum has one non-zero term)"""
+    n = 2 * BIG[dtype]
+    K = n
+    eye = O.encode(dtype, np.eye(n, dtype=np.float32))
+    B = make_operand(dtype, K, n, seed=5, tensor=1, scale=1.0)
+    out_dt = dtype if dtype != O.E4M3 else O.F32
+    got = run_gemm(hip, dtype, eye, B, 0, 0, out_dt, n, n, K)
+    if dtype == O.E4M3:
+        assert np.array_equal(got, O.decode(dtype, B))
+    else:
+        assert np.array_equal(got.view(np.uint8), B.view(np.uint8))
+
+
+def test_all_ones_gives_k(hip):
+    M = N = 256
+    K = 64 * 7
+    ones = O.encode(O.F16, np.ones((M, K), dtype=np.float32))
+    onesB = O.encode(O.F16, np.ones((K, N), dtype=np.float32))
+    got = run_gemm(hip, O.F16, ones, onesB, 0, 0, O.F32, M, N, K)
+    assert np.all(got == float(K))
+
+
+def test_accumulate_into_c(hip):
+    """clear_accum = 0: C = C + A.B  (frisk.gemm clear_accum attribute)"""
+    M = N = 256
+    K = 128
+    A = make_operand(O.F16, M, K, seed=7, tensor=0, scale=0.25)
+    B = make_operand(O.F16, K, N, seed=7, tensor=1, scale=0.25)
+    C0 = O.uniform(M * N, 7, 2, -1.0, 1.0).reshape(M, N).astype(np.float32)
+    got = run_gemm(hip, O.F16, A, B, 0, 0, O.F32, M, N, K, C_init=C0, clear_accum=False)
+    ref = O.gemm_f64(O.F16, A, B) + C0.astype(np.float64)
+    check(O.F16, O.F32, got, ref)
+    A8 = make_operand(O.I8, M, K, seed=8, tensor=0)
+    B8 = make_operand(O.I8, K, N, seed=8, tensor=1)
+    Ci = (np.arange(M * N, dtype=np.int64).reshape(M, N) % 1000 - 500).astype(np.int32)
+    goti = run_gemm(hip, O.I8, A8, B8, 0, 0, O.I32, M, N, K, C_init=Ci, clear_accum=False)
+    assert np.array_equal(goti, O.gemm_i32(A8, B8) + Ci)
+
+
+def test_int8_dequant_epilogue_bit_exact(hip):
+    """out = f16((float(acc) * sA[m]) * sB[n]) with the multiplication order fixed: bit-exact against the oracle"""
+    M, N, K = 512, 512, 1024
+    A = make_operand(O.I8, M, K, seed=3, tensor=0)
+    B = make_operand(O.I8, K, N, seed=3, tensor=1)
+    sA = O.uniform(M, 3, 2, 0.001, 0.02)
+    sB = O.uniform(N, 3, 3, 0.001, 0.02)
+    got = run_gemm(hip, O.I8, A, B, 0, 0, O.F16, M, N, K, epilogue=hip.EPI_ROW_COL_SCALE, sA=sA, sB=sB)
+    acc = O.gemm_i32(A, B)
+    assert np.array_equal(got, O.epilogue_rowcol_f16(acc, sA, sB))
+    # power-of-two scales: closed form, exact
+    sA2 = np.full(M, 2.0 ** -10, dtype=np.float32)
+    sB2 = np.full(N, 2.0 ** -6, dtype=np.float32)
+    got2 = run_gemm(hip, O.I8, A, B, 0, 0, O.F32, M, N, K, epilogue=hip.EPI_ROW_COL_SCALE, sA=sA2, sB=sB2)
+    assert np.array_equal(got2, acc.astype(np.float32) * np.float32(2.0 ** -16))
+
+
+def test_fp8_tensor_scale_epilogue(hip):
+    M, N, K = 256, 512, 512
+    xa, xb = O.normal(M * K, 4, 0, 1.0), O.normal(N * K, 4, 1, 1.0)
+    sA, sB = np.float32(np.abs(xa).max() / 448.0), np.float32(np.abs(xb).max() / 448.0)
+    A = O.encode(O.E4M3, xa / sA).reshape(M, K)
+    B = O.encode(O.E4M3, xb / sB).reshape(N, K)  # stored [N][K]
+    got = run_gemm(hip, O.E4M3, A, B, 0, 1, O.BF16, M, N, K, epilogue=hip.EPI_TENSOR_SCALE, sA=[sA], sB=[sB])
+    ref = O.epilogue_tensor(O.gemm_f64(O.E4M3, A, B, False, True), sA, sB)
+    check(O.E4M3, O.BF16, got, ref)
+
+
+# ------------------------------------------------------------------ full-size configurations
+def test_config_fp32_1024(hip):
+    M = N = K = 1024
+    A = make_operand(O.F32, M, K, seed=0, tensor=0, kind="uniform")
+    B = make_operand(O.F32, K, N, seed=0, tensor=1, kind="uniform")
+    got = run_gemm(hip, O.F32, A, B, 0, 0, O.F32, M, N, K)
+    r = check(O.F32, O.F32, got, O.gemm_f64(O.F32, A, B))
+    note(f"fp32 1024^3: {r}")
+
+
+def test_config_fp16_4096(hip):
+    M = N = K = 4096
+    A = make_operand(O.F16, M, K, seed=1, tensor=0, scale=1.0 / 64.0)
+    B = make_operand(O.F16, K, N, seed=1, tensor=1, scale=1.0 / 64.0)
+    got = run_gemm(hip, O.F16, A, B, 0, 0, O.F16, M, N, K)
+    r = check(O.F16, O.F16, got, O.gemm_f64(O.F16, A, B))
+    note(f"fp16 4096^3: {r}")
+
+
+def test_config_int8_4096(hip):
+    M = N = K = 4096
+    A = make_operand(O.I8, M, K, seed=3, tensor=0)
+    B = make_operand(O.I8, K, N, seed=3, tensor=1)
+    sA = O.uniform(M, 3, 2, 0.001, 0.02)
+    sB = O.uniform(N, 3, 3, 0.001, 0.02)
+    acc = O.gemm_i32(A, B)
+    got_i32 = run_gemm(hip, O.I8, A, B, 0, 0, O.I32, M, N, K)
+    assert np.array_equal(got_i32, acc)
+    got = run_gemm(hip, O.I8, A, B, 0, 0, O.F16, M, N, K, epilogue=hip.EPI_ROW_COL_SCALE, sA=sA, sB=sB)
+    assert np.array_equal(got, O.epilogue_rowcol_f16(acc, sA, sB))
+    # and within tolerance of the un-narrowed value
+    check(O.I8, O.F16, got, O.epilogue_rowcol_f32(acc, sA, sB).astype(np.float64))
+
+
+def _sampled_rows(M, tile, count=64):
+    rows = set(range(0, M, max(1, M // count)))
+    for t in range(0, M, tile):
+        rows.add(t)
+        rows.add(t + tile - 1)
+    return sorted(rows)
+
+
+def test_config_bf16_8192_nt(hip):
+    """8192^3: the oracle checks 64 evenly spaced rows plus the first and last row of every tile band"""
+    M = N = K = 8192
+    A = make_operand(O.BF16, M, K, seed=2, tensor=0, scale=0.02)
+    B = make_operand(O.BF16, N, K, seed=2, tensor=1, scale=0.02)
+    got = run_gemm(hip, O.BF16, A, B, 0, 1, O.BF16, M, N, K)
+    rows = _sampled_rows(M, 256)
+    ref = np.concatenate([O.gemm_f64(O.BF16, A, B, False, True, r, 1) for r in rows])
+    r = check(O.BF16, O.BF16, np.ascontiguousarray(got[rows]), ref)
+    note(f"bf16 8192^3 NT ({len(rows)} rows): {r}")
+
+
+def test_config_fp8_8192(hip):
+    M = N = K = 8192
+    xa, xb = O.normal(M * K, 4, 0, 1.0), O.normal(N * K, 4, 1, 1.0)
+    sA, sB = np.float32(np.abs(xa).max() / 448.0), np.float32(np.abs(xb).max() / 448.0)
+    A = O.encode(O.E4M3, xa / sA).reshape(M, K)
+    B = O.encode(O.E4M3, xb / sB).reshape(N, K)
+    del xa, xb
+    got = run_gemm(hip, O.E4M3, A, B, 0, 1, O.BF16, M, N, K, epilogue=hip.EPI_TENSOR_SCALE, sA=[sA], sB=[sB])
+    rows = _sampled_rows(M, 256)
+    ref = np.concatenate([O.gemm_f64(O.E4M3, A, B, False, True, r, 1) for r in rows])
+    r = check(O.E4M3, O.BF16, np.ascontiguousarray(got[rows]), O.epilogue_tensor(ref, sA, sB))
+    note(f"fp8 8192^3 NT ({len(rows)} rows): {r}")
