@@ -1,0 +1,120 @@
+#!/usr/bin/env python3
+"""Benchmark of the GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one launch of the fp16 4096^3 NN GEMM (fp32 accumulate, fp16 out,
+inputs N(0,1)/sqrt(K), seed 1) through the C ABI, inputs resident in HBM.
+Prints ONE JSON line: whole-job TFLOP/s, the MFMA roofline of the kernel and
+the CPU oracle timed on the host cores beside it.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "i8": 5033.2, "e4m3": 5033.2, "f32": 157.3}
+
+
+def gpu_time_gemm(R, torch, desc, ptrs, steps, warmup):
+    """returns (wall seconds for `steps` launches, mean kernel ms from HIP events on the launch stream)"""
+    stream = torch.cuda.current_stream()
+    s = stream.cuda_stream
+    for _ in range(warmup):
+        R.gemm(desc, *ptrs, None, 0, s)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(steps):
+        R.gemm(desc, *ptrs, None, 0, s)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, e0.elapsed_time(e1) / steps
+
+
+def cpu_baseline(M, N, K):
+    """the CPU oracle (fp32 arithmetic, OpenMP over all host cores) on the same workload"""
+    import numpy as np
+    import oracle as O
+    A = O.encode(O.F16, O.normal(M * K, 1, 0, 1.0 / np.sqrt(K))).reshape(M, K)
+    B = O.encode(O.F16, O.normal(K * N, 1, 1, 1.0 / np.sqrt(K))).reshape(K, N)
+    O.gemm_f32(O.F16, A, B, nrows=256)  # warm-up: thread pool, first touch
+    runs = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        O.gemm_f32(O.F16, A, B)
+        runs.append(time.perf_counter() - t0)
+    best = min(runs)
+    return {"value": round(2.0 * M * N * K / best / 1e12, 4), "unit": "TFLOP/s", "cores": O.num_threads(), "kind": "port",
+            "sample": "full fp16 4096^3 NN GEMM, fp32 arithmetic, best of 3 runs (%.2f s each)" % best}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one GPU: the GEMM path has no multi-GPU leg (run with --gpus 1)")
+
+    import torch
+    from frisk_amd import runtime as R
+
+    R.lib()
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    dev = torch.device("cuda:0")
+    M = N = K = 4096
+    g = torch.Generator(device=dev)
+    g.manual_seed(1)
+    A = (torch.randn(M, K, device=dev, generator=g) / K ** 0.5).half()
+    B = (torch.randn(K, N, device=dev, generator=g) / K ** 0.5).half()
+    C = torch.empty(M, N, device=dev, dtype=torch.float16)
+    desc = R.make_desc(R.F16, M, N, K, dtype_out=R.F16)
+    plan = R.plan(desc)
+    ptrs = (A.data_ptr(), B.data_ptr(), C.data_ptr(), None, None)
+    wall, kern_ms = gpu_time_gemm(R, torch, desc, ptrs, a.steps, a.warmup)
+    flops = 2.0 * M * N * K
+    value = flops * a.steps / wall / 1e12
+    achieved = flops / (kern_ms * 1e-3) / 1e12
+
+    # second headline shape of the metric: W8A8 int8 4096^3 with the dequant epilogue (reported, not the timed value)
+    A8 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
+    B8 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev, generator=g)
+    sA = torch.rand(M, device=dev, generator=g) * 0.019 + 0.001
+    sB = torch.rand(N, device=dev, generator=g) * 0.019 + 0.001
+    C8 = torch.empty(M, N, device=dev, dtype=torch.float16)
+    d8 = R.make_desc(R.I8, M, N, K, dtype_out=R.F16, epilogue=R.EPI_ROW_COL_SCALE)
+    _, i8_ms = gpu_time_gemm(R, torch, d8, (A8.data_ptr(), B8.data_ptr(), C8.data_ptr(), sA.data_ptr(), sB.data_ptr()),
+                             a.steps, a.warmup)
+    i8_tops = flops / (i8_ms * 1e-3) / 1e12
+
+    line = {
+        "metric": "GEMM TFLOP/s at 4096^3 fp16 (fp32 accumulate), 1 GPU",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(wall / a.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "fp16 GEMM M=N=K=4096 NN row-major, N(0,1)/sqrt(K) seed 1, fp32 accumulate, fp16 out",
+                   "kernel": R.kernel_names()[plan.kernel_id], "grid": [plan.grid_x, plan.grid_y],
+                   "lds_bytes": plan.lds_bytes},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_TFLOPS["f16"], 4), "traffic": None,
+                     "kernel_ms": round(kern_ms, 5)},
+        "int8_4096": {"value": round(i8_tops, 2), "unit": "TOPS", "peak": PEAK_TFLOPS["i8"],
+                      "frac": round(i8_tops / PEAK_TFLOPS["i8"], 4), "kernel_ms": round(i8_ms, 5),
+                      "workload": "W8A8 int8 4096^3 NN, int32 accumulate, per-row/per-column fp32 scales, fp16 out"},
+    }
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(M, N, K)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
