@@ -120,7 +120,7 @@ static int validate(const frisk_gemm_desc* d) {
   return FRISK_OK;
 }
 
-static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, int mn, int bk, int nw) {
+static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, int mn, int bk, int nw, bool with_model) {
   TileShape t{kcontig ? mn : bk, (kcontig ? bk : mn) * es, kcontig, es, fragb, mn, bk};
   Swizzle s = default_swizzle(kcontig, es, t.rowb);
   L->rows = t.rows;
@@ -132,13 +132,14 @@ static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, in
   L->read_instr = es == 4 ? 3 : (kcontig ? 0 : (es == 2 ? 1 : 2));
   int atoms = mn / 32 < 4 ? mn / 32 : 4;
   int n_access = atoms * ((bk * es) / (2 * fragb)) * frag_instr_count(kcontig, es, fragb);
-  L->read_cycles = n_access ? (float)swizzle_read_cycles(t, s) / (float)n_access : 0.f;
+  // evaluating the bank model costs ~0.1 ms of host time: only when the caller asks for the plan
+  L->read_cycles = (with_model && n_access) ? (float)swizzle_read_cycles(t, s) / (float)n_access : 0.f;
   // the direct-to-LDS transfer writes 64 consecutive 16-byte slots: no conflicts by construction
   L->write_cycles = 16.f;
   (void)nw;
 }
 
-static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan) {
+static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_model) {
   int st = validate(d);
   if (st != FRISK_OK) return st;
   if (!plan) return fail(FRISK_ERR_NULL, "plan is null");
@@ -150,12 +151,11 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan) {
   if (d->epilogue == FRISK_EPI_ROW_COL_SCALE) plan->bytes += 4.0 * ((double)d->M + (double)d->N);
   if (d->epilogue == FRISK_EPI_TENSOR_SCALE) plan->bytes += 8.0;
   plan->split_k = 1;
-  plan->stages = 2;
 
   const auto& ks = kernels();
   int best = -1;
   int64_t best_tiles = 0;
-  bool any_layout = false, tile_requested = d->tile_m || d->tile_n || d->tile_k || d->waves_m || d->waves_n;
+  bool any_layout = false, tile_requested = d->tile_m || d->tile_n || d->tile_k || d->waves_m || d->waves_n || d->stages;
   for (size_t i = 0; i < ks.size(); ++i) {
     const KernelEntry* k = ks[i];
     if (k->dtype != d->dtype_ab || k->transA != (d->transA != 0) || k->transB != (d->transB != 0)) continue;
@@ -165,6 +165,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan) {
     if (d->tile_k && d->tile_k != k->bk) continue;
     if (d->waves_m && d->waves_m != k->wm) continue;
     if (d->waves_n && d->waves_n != k->wn) continue;
+    if (d->stages && d->stages != k->stages) continue;
     if (d->M % k->bm || d->N % k->bn || d->K % k->bk) continue;
     int64_t tiles = (d->M / k->bm) * (d->N / k->bn);
     // largest tile that still gives every CU a work-group; otherwise the most work-groups
@@ -174,8 +175,9 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan) {
       const KernelEntry* b = ks[best];
       bool fills = tiles >= 256, bfills = best_tiles >= 256;
       if (fills != bfills) better = fills;
-      else if (fills) better = (int64_t)k->bm * k->bn > (int64_t)b->bm * b->bn;
-      else better = tiles > best_tiles;
+      else if (fills && (int64_t)k->bm * k->bn != (int64_t)b->bm * b->bn) better = (int64_t)k->bm * k->bn > (int64_t)b->bm * b->bn;
+      else if (!fills && tiles != best_tiles) better = tiles > best_tiles;
+      else better = false;  // same tile: the first listed variant is the tuned default
     }
     if (better) { best = (int)i; best_tiles = tiles; }
   }
@@ -197,11 +199,12 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan) {
   plan->waves_m = k->wm; plan->waves_n = k->wn; plan->threads = k->wm * k->wn * 64;
   plan->mfma_m = 32; plan->mfma_n = 32; plan->mfma_k = mfma_k(d->dtype_ab);
   plan->lds_bytes = k->lds_bytes;
+  plan->stages = k->stages;
   plan->grid_x = (int)(d->N / k->bn);
   plan->grid_y = (int)(d->M / k->bm);
   plan->xcd_remap = ((int64_t)plan->grid_x * plan->grid_y) % 8 == 0;
-  fill_layout(&plan->lds_a, !d->transA, es, frag_bytes(d->dtype_ab), k->bm, k->bk, k->wm * k->wn);
-  fill_layout(&plan->lds_b, d->transB != 0, es, frag_bytes(d->dtype_ab), k->bn, k->bk, k->wm * k->wn);
+  fill_layout(&plan->lds_a, !d->transA, es, frag_bytes(d->dtype_ab), k->bm, k->bk, k->wm * k->wn, with_model);
+  fill_layout(&plan->lds_b, d->transB != 0, es, frag_bytes(d->dtype_ab), k->bn, k->bk, k->wm * k->wn, with_model);
   plan->workspace_bytes = 0;
   return FRISK_OK;
 }
@@ -235,18 +238,18 @@ int frisk_hip_abi_version(void) { return FRISK_HIP_ABI_VERSION; }
 
 const char* frisk_hip_last_error(void) { return g_last_error.c_str(); }
 
-int frisk_hip_plan(const frisk_gemm_desc* desc, frisk_gemm_plan* plan) { return make_plan(desc, plan); }
+int frisk_hip_plan(const frisk_gemm_desc* desc, frisk_gemm_plan* plan) { return make_plan(desc, plan, true); }
 
 size_t frisk_hip_workspace_bytes(const frisk_gemm_desc* desc) {
   frisk_gemm_plan plan;
-  if (make_plan(desc, &plan) != FRISK_OK) return 0;
+  if (make_plan(desc, &plan, false) != FRISK_OK) return 0;
   return plan.workspace_bytes;
 }
 
 int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, void* C, const float* scaleA,
                    const float* scaleB, void* workspace, size_t workspace_bytes, void* stream) {
   frisk_gemm_plan plan;
-  int st = make_plan(desc, &plan);
+  int st = make_plan(desc, &plan, false);
   if (st != FRISK_OK) return st;
   if (desc->M == 0 || desc->N == 0) return FRISK_OK;
   if (!A || !B || !C) return fail(FRISK_ERR_NULL, "A, B and C must be device pointers");

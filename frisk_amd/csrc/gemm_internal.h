@@ -24,7 +24,7 @@ struct KernelEntry {
   const char* name;
   int dtype;  // frisk_dtype of A and B
   int transA, transB;
-  int bm, bn, bk, wm, wn;
+  int bm, bn, bk, wm, wn, stages;
   int lds_bytes;
   hipError_t (*launch)(const GemmParams&, hipStream_t);
 };

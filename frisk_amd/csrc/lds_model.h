@@ -181,8 +181,13 @@ FRISK_HD Swizzle choose_swizzle(TileShape t, int nw) {
 FRISK_HD Swizzle default_swizzle(bool kcontig, int es, int rowb) {
   int chunks = rowb / 16;
   if (kcontig) {
-    int mk = chunks >= 8 ? 7 : chunks - 1;
-    return Swizzle{es == 4 ? 0 : 1, mk, 0};
+    // 16 consecutive rows must cover the 16 bank groups of 16 bytes: rows of 128 B
+    // bring 2 groups by themselves, rows of 64 B bring 4, rows of 256 B none
+    if (es == 4) return Swizzle{0, chunks >= 8 ? 7 : chunks - 1, 0};
+    if (chunks >= 16) return Swizzle{0, 15, 0};
+    if (chunks == 8) return Swizzle{1, 7, 0};
+    if (chunks == 4) return Swizzle{2, 3, 0};
+    return Swizzle{3, chunks - 1, 0};
   }
   if (es == 4) return Swizzle{0, 0, 0};
   if (es == 2) {

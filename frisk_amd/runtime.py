@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libfrisk_hip.so")
+# FRISK_HIP_LIB points kernel developers at another build of the same library
+LIB_PATH = os.environ.get("FRISK_HIP_LIB") or os.path.join(_HERE, "lib", "libfrisk_hip.so")
 
 ABI_VERSION = 1
 F32, F16, BF16, I8, E4M3, I32 = 0, 1, 2, 3, 4, 5
@@ -30,7 +31,7 @@ class GemmDesc(ctypes.Structure):
                 ("transA", ctypes.c_uint8), ("transB", ctypes.c_uint8), ("clear_accum", ctypes.c_uint8),
                 ("reserved0", ctypes.c_uint8), ("epilogue", ctypes.c_int32), ("policy", ctypes.c_int32),
                 ("tile_m", ctypes.c_int32), ("tile_n", ctypes.c_int32), ("tile_k", ctypes.c_int32),
-                ("waves_m", ctypes.c_int32), ("waves_n", ctypes.c_int32)]
+                ("waves_m", ctypes.c_int32), ("waves_n", ctypes.c_int32), ("stages", ctypes.c_int32)]
 
 
 class LdsLayout(ctypes.Structure):
@@ -98,7 +99,7 @@ def _check(status):
 
 
 def make_desc(dtype_ab, M, N, K, dtype_out=None, transA=False, transB=False, lda=None, ldb=None, ldc=None,
-              clear_accum=True, epilogue=EPI_NONE, policy=POLICY_SQUARE, tile=(0, 0, 0), waves=(0, 0)):
+              clear_accum=True, epilogue=EPI_NONE, policy=POLICY_SQUARE, tile=(0, 0, 0), waves=(0, 0), stages=0):
     d = GemmDesc()
     d.abi_version = ABI_VERSION
     d.dtype_ab = dtype_ab
@@ -112,6 +113,7 @@ def make_desc(dtype_ab, M, N, K, dtype_out=None, transA=False, transB=False, lda
     d.epilogue, d.policy = epilogue, policy
     d.tile_m, d.tile_n, d.tile_k = tile
     d.waves_m, d.waves_n = waves
+    d.stages = stages
     return d
 
 

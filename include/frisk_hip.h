@@ -84,6 +84,7 @@ typedef struct frisk_gemm_desc {
   int32_t policy;                 /* frisk_wave_policy */
   int32_t tile_m, tile_n, tile_k; /* block tile = the M,N,K attrs of the tile-level frisk.gemm */
   int32_t waves_m, waves_n;       /* wave grid inside the work-group */
+  int32_t stages;                 /* LDS stages of the global->LDS pipeline, 0 = planner's choice */
 } frisk_gemm_desc;
 
 /* XOR swizzle of an LDS tile: 16-byte chunk index c of row r is stored at
