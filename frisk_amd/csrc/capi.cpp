@@ -281,6 +281,28 @@ float frisk_hip_lds_access_cycles(int instr, const int32_t* lane_byte_addr) {
   return (float)lds_access_cycles(instr == 2 ? 1 : instr, addr);
 }
 
+int frisk_hip_lds_search(const frisk_lds_layout* shape, int elem_bytes, int frag_bytes, int tile_mn, int tile_k, int waves,
+                         frisk_lds_layout* best, float* unswizzled_cycles) {
+  if (!shape || !best) return fail(FRISK_ERR_NULL, "shape and best must be given");
+  if (shape->rows <= 0 || shape->row_bytes < 16 || shape->row_bytes % 16 || shape->row_bytes > 1024 || 1024 % shape->row_bytes)
+    return fail(FRISK_ERR_TILE, "tile rows must be 16..1024 bytes and divide 1024");
+  if ((elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) || frag_bytes < elem_bytes || waves <= 0 || tile_mn < 32 || tile_k <= 0)
+    return fail(FRISK_ERR_TILE, "unsupported operand description");
+  const bool kc = shape->k_contiguous != 0;
+  TileShape t{shape->rows, shape->row_bytes, kc, elem_bytes, frag_bytes, tile_mn, tile_k};
+  const Swizzle s = choose_swizzle(t, waves);
+  const int atoms = tile_mn / 32 < 4 ? tile_mn / 32 : 4;
+  const int n_access = atoms * ((tile_k * elem_bytes) / (2 * frag_bytes)) * frag_instr_count(kc, elem_bytes, frag_bytes);
+  if (n_access <= 0) return fail(FRISK_ERR_TILE, "tile holds no whole MFMA step");
+  *best = *shape;
+  best->row_shift = s.sh; best->row_mask = s.mk; best->chunk_shift = s.cs;
+  best->read_instr = elem_bytes == 4 ? 3 : (kc ? 0 : (elem_bytes == 2 ? 1 : 2));
+  best->read_cycles = (float)swizzle_read_cycles(t, s) / (float)n_access;
+  best->write_cycles = 16.f;
+  if (unswizzled_cycles) *unswizzled_cycles = (float)swizzle_read_cycles(t, Swizzle{0, 0, 0}) / (float)n_access;
+  return FRISK_OK;
+}
+
 int32_t frisk_hip_lds_offset(const frisk_lds_layout* L, int32_t row, int32_t col_byte) {
   if (!L) return -1;
   return lds_offset(L->row_bytes, Swizzle{L->row_shift, L->row_mask, L->chunk_shift}, row, col_byte);

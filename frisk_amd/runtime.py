@@ -59,7 +59,7 @@ class FriskHipError(RuntimeError):
 _lib = None
 
 EXPORTS = ["frisk_hip_abi_version", "frisk_hip_last_error", "frisk_hip_plan", "frisk_hip_workspace_bytes",
-           "frisk_hip_gemm", "frisk_hip_lds_access_cycles", "frisk_hip_lds_offset", "frisk_hip_wave_partition",
+           "frisk_hip_gemm", "frisk_hip_lds_access_cycles", "frisk_hip_lds_search", "frisk_hip_lds_offset", "frisk_hip_wave_partition",
            "frisk_hip_kernel_count", "frisk_hip_kernel_name"]
 
 
@@ -80,6 +80,8 @@ def lib():
                                  ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
     L.frisk_hip_lds_access_cycles.restype = ctypes.c_float
     L.frisk_hip_lds_access_cycles.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_int32)]
+    L.frisk_hip_lds_search.argtypes = [ctypes.POINTER(LdsLayout), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                       ctypes.c_int, ctypes.POINTER(LdsLayout), ctypes.POINTER(ctypes.c_float)]
     L.frisk_hip_lds_offset.restype = ctypes.c_int32
     L.frisk_hip_lds_offset.argtypes = [ctypes.POINTER(LdsLayout), ctypes.c_int32, ctypes.c_int32]
     L.frisk_hip_wave_partition.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -138,6 +140,19 @@ def wave_partition(policy, tile_m, tile_n, num_waves):
 def lds_access_cycles(instr, lane_addrs):
     arr = (ctypes.c_int32 * 64)(*lane_addrs)
     return lib().frisk_hip_lds_access_cycles(instr, arr)
+
+
+def lds_search(rows, row_bytes, k_contiguous, elem_bytes, frag_bytes, tile_mn, tile_k, waves):
+    """exhaustive swizzle search for one operand tile; returns (LdsLayout best, unswizzled cycles per access)"""
+    shape, best, base = LdsLayout(), LdsLayout(), ctypes.c_float()
+    shape.rows, shape.row_bytes, shape.k_contiguous = rows, row_bytes, int(k_contiguous)
+    _check(lib().frisk_hip_lds_search(ctypes.byref(shape), elem_bytes, frag_bytes, tile_mn, tile_k, waves,
+                                      ctypes.byref(best), ctypes.byref(base)))
+    return best, base.value
+
+
+def lds_offset(layout, row, col_byte):
+    return lib().frisk_hip_lds_offset(ctypes.byref(layout), row, col_byte)
 
 
 def kernel_names():

@@ -140,6 +140,15 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
  * histogram of the reference's layout tool (exp/layout/gemm_layout_tool.cpp:135-208). */
 float frisk_hip_lds_access_cycles(int instr, const int32_t* lane_byte_addr);
 
+/* Pure host: exhaustive swizzle search for one operand tile.  `shape` gives rows, row_bytes and
+ * k_contiguous of the tile as stored; elem_bytes / frag_bytes describe the MFMA operand (bytes per
+ * element, bytes per lane per MFMA); tile_mn / tile_k the logical extents in elements; waves the
+ * number of waves staging the tile.  Writes the best layout (swizzle fields, read_instr and the
+ * modelled read_cycles per access) to `best`; `unswizzled_cycles` (may be NULL) receives the
+ * modelled cycles per access of the same tile without a swizzle. */
+int frisk_hip_lds_search(const frisk_lds_layout* shape, int elem_bytes, int frag_bytes, int tile_mn, int tile_k, int waves,
+                         frisk_lds_layout* best, float* unswizzled_cycles);
+
 /* Pure host: byte offset inside an LDS tile of element (row, col_byte) under `layout`. */
 int32_t frisk_hip_lds_offset(const frisk_lds_layout* layout, int32_t row, int32_t col_byte);
 
