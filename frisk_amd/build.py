@@ -1,6 +1,6 @@
 """Builds libfrisk_hip.so (HIP kernels + C ABI) for gfx950, in-tree.
 
-    python -m frisk_amd.build          # rebuild everything
+    python -m frisk_amd.build          # rebuild everything (HIP library + frisk_ffi extension)
     python -m frisk_amd.build --if-missing
 
 hipcc cross-compiles without a GPU; the resulting library is loaded from
@@ -59,6 +59,27 @@ def build(jobs=None, verbose=True):
     return LIB
 
 
+FFI_DIR = os.path.join(HERE, "ffi")
+FFI_SOURCES = ["ffi.cpp", "ir.cpp", "runtime.cpp"]
+
+
+def build_ffi(verbose=True):
+    """the `frisk_ffi` CPython extension (IR builder + runtime), host code only"""
+    import sysconfig
+
+    import pybind11
+    out = os.path.join(HERE, "frisk", "frisk_ffi" + sysconfig.get_config_var("EXT_SUFFIX"))
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
+           "-I" + pybind11.get_include(), "-I" + sysconfig.get_paths()["include"], "-I" + os.path.join(ROOT, "include")]
+    cmd += [os.path.join(FFI_DIR, f) for f in FFI_SOURCES] + ["-o", out, "-ldl"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building frisk_ffi failed:\n" + r.stderr)
+    if verbose:
+        print("built", out)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--if-missing", action="store_true")
@@ -68,6 +89,7 @@ def main():
         print("present", LIB)
         return
     build(a.j)
+    build_ffi()
 
 
 if __name__ == "__main__":

@@ -1,0 +1,562 @@
+// Builder surface of the Frisk Python API over the MLIR-free IR of mini_ir.h.
+// Names, argument orders, defaults and error behaviour follow the reference's
+// ffi/ir.cpp (cited per binding); only the calls the GEMM path uses are provided.
+#include <iostream>
+#include <optional>
+
+#include "ffi.h"
+#include "mini_ir.h"
+
+namespace frisk_ffi {
+
+using namespace frisk_ir;
+using ret = py::return_value_policy;
+
+struct PyContext {
+  std::shared_ptr<Context> ctx = std::make_shared<Context>();
+};
+
+// non-owning op handle, as mlir::OpState is
+struct OpState {
+  Operation* op = nullptr;
+  Context* ctx = nullptr;
+};
+template <int Tag> struct OpT : OpState {};
+using ModuleOp = OpT<0>;
+using KernelOp = OpT<1>;
+using ParallelOp = OpT<2>;
+using BlockOp = OpT<3>;
+using ForOp = OpT<4>;
+using AllocBufferOp = OpT<5>;
+using CopyOp = OpT<6>;
+using FillOp = OpT<7>;
+using ReduceOp = OpT<8>;
+using GemmOp = OpT<9>;
+using EndOp = OpT<10>;
+
+struct PyBlock {
+  Block* block = nullptr;
+  Context* ctx = nullptr;
+};
+struct PyRegion {
+  Region* region = nullptr;
+  Context* ctx = nullptr;
+};
+
+// OpBuilder + insertion point (the reference's OpBuilderWithLoc, include/Dialect/Frisk/Utils/Utils.h:17-92).
+// An insertion point is "before `before` in `block`"; before == nullptr means the end of the block.
+struct Builder {
+  Context* ctx;
+  std::shared_ptr<Context> keep;
+  Block* block = nullptr;
+  Operation* before = nullptr;
+  explicit Builder(PyContext& c) : ctx(c.ctx.get()), keep(c.ctx) {}
+
+  void insert(Operation* op) {
+    if (!block) return;  // detached, like an OpBuilder without insertion point
+    op->block = block;
+    auto& ops = block->ops;
+    auto it = ops.end();
+    if (before)
+      for (auto i = ops.begin(); i != ops.end(); ++i)
+        if (*i == before) { it = i; break; }
+    ops.insert(it, op);
+  }
+  void set_to_start(Block* b) { block = b; before = b->ops.empty() ? nullptr : b->ops.front(); }
+  void set_to_end(Block* b) { block = b; before = nullptr; }
+  void set_after(Operation* op) {
+    block = op->block;
+    before = nullptr;
+    if (!block) return;
+    for (size_t i = 0; i + 1 < block->ops.size(); ++i)
+      if (block->ops[i] == op) before = block->ops[i + 1];
+  }
+  Operation* make_end() { return ctx->new_op("frisk.end"); }
+  template <class T> T wrap(Operation* op) { T t; t.op = op; t.ctx = ctx; return t; }
+};
+
+static Type parse_dtype(const std::string& dtype) {
+  // the reference accepts e4m3fn, e5m2, fp16, fp32, fp64 (ffi/ir.cpp:411-423); bf16, int8 and
+  // int32 are added because the GEMM path computes in them
+  if (dtype == "e4m3fn") return Type::scalar(TypeKind::F8E4M3FN);
+  if (dtype == "e5m2") return Type::scalar(TypeKind::F8E5M2);
+  if (dtype == "fp16") return Type::scalar(TypeKind::F16);
+  if (dtype == "bf16") return Type::scalar(TypeKind::BF16);
+  if (dtype == "fp32") return Type::scalar(TypeKind::F32);
+  if (dtype == "fp64") return Type::scalar(TypeKind::F64);
+  if (dtype == "int8") return Type::scalar(TypeKind::I8);
+  if (dtype == "int32") return Type::scalar(TypeKind::I32);
+  throw std::invalid_argument("invalid float type");
+}
+
+static Block* add_body_block(Context* ctx, Operation* op, const std::vector<Type>& arg_types) {
+  Region* rg = op->regions[0];
+  if (!rg->blocks.empty()) throw std::invalid_argument("entry block already exists");
+  Block* b = ctx->new_block();
+  b->parent = rg;
+  rg->blocks.push_back(b);
+  for (auto& t : arg_types) ctx->add_block_arg(b, t);
+  Operation* end = ctx->new_op("frisk.end");
+  end->block = b;
+  b->ops.push_back(end);
+  return b;
+}
+
+static void print_diagnostics(const Diagnostics& d) {
+  for (auto& e : d.errors) std::cerr << "error: " << e << "\n";
+}
+
+template <class OpClass> static void def_common(py::class_<OpClass, OpState>&) {}
+
+void init_ffi_ir(py::module_&& m) {
+  // ---------------------------------------------------------------- context, types, values (ffi/ir.cpp:883-1078)
+  py::class_<PyContext>(m, "context", py::module_local())
+      .def(py::init<>())
+      .def("disable_multithreading", [](PyContext& self) { self.ctx->multithreading = false; });
+
+  py::enum_<MemorySpace>(m, "MemorySpace", py::arithmetic())  // ffi/ir.cpp:137-141
+      .value("GLOBAL", MemorySpace::Global)
+      .value("SHARED", MemorySpace::Shared)
+      .value("LOCAL", MemorySpace::Local)
+      .export_values();
+
+  py::class_<AffineExpr>(m, "AffineExpr", py::module_local())  // ffi/ir.cpp:700-810, the arithmetic subset
+      .def(py::init<>())
+      .def("__eq__", [](const AffineExpr& a, const AffineExpr& b) { return a.equals(b); })
+      .def("__eq__", [](const AffineExpr& a, int64_t v) { return a.is_constant() && a.constant_value() == v; })
+      .def("__ne__", [](const AffineExpr& a, const AffineExpr& b) { return !a.equals(b); })
+      .def("__bool__", [](const AffineExpr& a) { return (bool)a; })
+      .def("__str__", [](const AffineExpr& a) { return a.str(); })
+      .def("__repr__", [](const AffineExpr& a) { return a.str(); })
+      .def("get_kind", [](const AffineExpr& a) { return (int)a.kind(); })
+      .def("__add__", [](const AffineExpr& a, int64_t v) { return a + v; })
+      .def("__add__", [](const AffineExpr& a, const AffineExpr& b) { return a + b; })
+      .def("__radd__", [](const AffineExpr& a, int64_t v) { return a + v; })
+      .def("__neg__", [](const AffineExpr& a) { return -a; })
+      .def("__sub__", [](const AffineExpr& a, int64_t v) { return a - v; })
+      .def("__sub__", [](const AffineExpr& a, const AffineExpr& b) { return a - b; })
+      .def("__mul__", [](const AffineExpr& a, int64_t v) { return a * v; })
+      .def("__mul__", [](const AffineExpr& a, const AffineExpr& b) { return a * b; })
+      .def("__rmul__", [](const AffineExpr& a, int64_t v) { return a * v; })
+      .def("floor_div", [](const AffineExpr& a, int64_t v) { return a.floor_div(AffineExpr::constant(v)); })
+      .def("floor_div", [](const AffineExpr& a, const AffineExpr& b) { return a.floor_div(b); })
+      .def("ceil_div", [](const AffineExpr& a, int64_t v) { return a.ceil_div(AffineExpr::constant(v)); })
+      .def("ceil_div", [](const AffineExpr& a, const AffineExpr& b) { return a.ceil_div(b); })
+      .def("__mod__", [](const AffineExpr& a, int64_t v) { return a.mod(AffineExpr::constant(v)); })
+      .def("__mod__", [](const AffineExpr& a, const AffineExpr& b) { return a.mod(b); })
+      .def("evaluate", [](const AffineExpr& a, std::vector<int64_t> dims, std::vector<int64_t> syms) { return a.eval(dims, syms); },
+           py::arg("dims"), py::arg("symbols") = std::vector<int64_t>());
+
+  py::class_<AffineMap>(m, "AffineMap", py::module_local())  // ffi/ir.cpp:646-699
+      .def(py::init<>())
+      .def_static("get", [](unsigned dims, unsigned syms, AffineExpr result) { return AffineMap((int)dims, (int)syms, {result}); })
+      .def_static("get", [](unsigned dims, unsigned syms, std::vector<AffineExpr> results, PyContext*) { return AffineMap((int)dims, (int)syms, results); },
+                  py::arg("dim_count"), py::arg("symbol_count"), py::arg("results"), py::arg("context") = nullptr)
+      .def_static("get_multi_dim_identity_map", [](unsigned n, PyContext*) { return AffineMap::identity((int)n); }, py::arg("num_dims"),
+                  py::arg("context") = nullptr)
+      .def("__eq__", [](const AffineMap& a, const AffineMap& b) { return a.equals(b); })
+      .def("__ne__", [](const AffineMap& a, const AffineMap& b) { return !a.equals(b); })
+      .def("__bool__", [](const AffineMap& a) { return (bool)a; })
+      .def("__str__", [](const AffineMap& a) { return a.str(); })
+      .def("__repr__", [](const AffineMap& a) { return a.str(); })
+      .def("get_num_dims", &AffineMap::num_dims)
+      .def("get_num_symbols", &AffineMap::num_symbols)
+      .def("get_num_results", &AffineMap::num_results)
+      .def("get_num_inputs", &AffineMap::num_inputs)
+      .def("get_results", [](const AffineMap& a) { return a.impl ? a.impl->results : std::vector<AffineExpr>(); })
+      .def("get_result", [](const AffineMap& a, unsigned i) { return a.impl->results.at(i); })
+      .def("is_identity", &AffineMap::is_identity);
+
+  py::class_<Type>(m, "type", py::module_local())  // ffi/ir.cpp:888-937
+      .def("__str__", [](const Type& t) { return t.str(); })
+      .def("__repr__", [](const Type& t) { return t.str(); })
+      .def("__eq__", [](const Type& a, const Type& b) { return a.equals(b); })
+      .def("is_f16", [](const Type& t) { return t.kind() == TypeKind::F16; })
+      .def("is_bf16", [](const Type& t) { return t.kind() == TypeKind::BF16; })
+      .def("is_f32", [](const Type& t) { return t.kind() == TypeKind::F32; })
+      .def("is_f64", [](const Type& t) { return t.kind() == TypeKind::F64; })
+      .def("is_float", &Type::is_float)
+      .def("is_index", [](const Type& t) { return t.kind() == TypeKind::Index; })
+      .def("is_int", &Type::is_int)
+      .def("get_rank", [](const Type& t) { return (int64_t)t.impl->shape.size(); })
+      .def("get_dim_size", [](const Type& t, unsigned i) { return t.impl->shape.at(i); })
+      .def("get_elem_width", [](const Type& t) { return t.element().bit_width(); })
+      .def("get_shape", [](const Type& t) { return t.impl->shape; })
+      .def("get_element_ty", [](const Type& t) { return t.element(); })
+      .def("get_memory_space", [](const Type& t) -> std::optional<MemorySpace> {
+        if (!t.is_memref()) return std::nullopt;
+        return (MemorySpace)t.impl->memory_space;
+      })
+      .def("get_layout_map", [](const Type& t) { return t.impl->layout ? t.impl->layout : AffineMap::identity((int)t.impl->shape.size()); })
+      .def("param_types", [](const Type& t) {
+        std::vector<Type> out;
+        for (auto& i : t.impl->inputs) out.push_back(Type(i));
+        return out;
+      });
+  m.attr("memref_buffer") = m.attr("type");
+  m.attr("function_type") = m.attr("type");
+  m.attr("ranked_tensor") = m.attr("type");
+
+  py::class_<Value>(m, "value", py::module_local())  // ffi/ir.cpp:949-975
+      .def("get_type", &Value::type)
+      .def("id", [](const Value& v) { return (uint64_t)(uintptr_t)v.impl; })
+      .def("__eq__", [](const Value& a, const Value& b) { return a == b; })
+      .def("__hash__", [](const Value& v) { return (size_t)(uintptr_t)v.impl; })
+      .def("__repr__", [](const Value& v) { return "<value of type " + v.type().str() + ">"; })
+      .def("__str__", [](const Value& v) { return "<value of type " + v.type().str() + ">"; });
+  m.attr("block_argument") = m.attr("value");
+  m.attr("op_result") = m.attr("value");
+
+  py::class_<PyRegion>(m, "region", py::module_local())
+      .def("size", [](PyRegion& r) { return r.region->blocks.size(); })
+      .def("empty", [](PyRegion& r) { return r.region->blocks.empty(); })
+      .def("push_back", [](PyRegion& r, PyBlock& b) { b.block->parent = r.region; r.region->blocks.push_back(b.block); })
+      .def("id", [](PyRegion& r) { return (uint64_t)(uintptr_t)r.region; });
+
+  py::class_<PyBlock>(m, "block", py::module_local())  // ffi/ir.cpp:1021-1073
+      .def("arg", [](PyBlock& b, unsigned i) {
+        if (i >= b.block->args.size()) throw py::index_error("Block argument index out of range");
+        return Value{b.block->args[i]};
+      })
+      .def("get_argument", [](PyBlock& b, unsigned i) {
+        if (i >= b.block->args.size()) throw py::index_error("Block argument index out of range");
+        return Value{b.block->args[i]};
+      })
+      .def("add_argument", [](PyBlock& b, Type t) { return b.ctx->add_block_arg(b.block, t); })
+      .def("get_num_arguments", [](PyBlock& b) { return b.block->args.size(); })
+      .def("has_terminator", [](PyBlock& b) { return b.block->has_terminator(); })
+      .def("get_num_operations", [](PyBlock& b) { return b.block->ops.size(); })
+      .def("id", [](PyBlock& b) { return (uint64_t)(uintptr_t)b.block; });
+
+  // ---------------------------------------------------------------- op handles (ffi/ir.cpp:476-644, 33-130)
+  py::class_<OpState>(m, "OpState", py::module_local())
+      .def("get_num_results", [](OpState& s) { return s.op->results.size(); })
+      .def("get_result", [](OpState& s, unsigned i) {
+        if (i >= s.op->results.size()) throw py::index_error("Op result index out of range");
+        return Value{s.op->results[i]};
+      })
+      .def("get_region", [](OpState& s, unsigned i) {
+        if (i >= s.op->regions.size()) throw py::index_error("Op region index out of range");
+        return PyRegion{s.op->regions[i], s.ctx};
+      })
+      .def("get_name", [](OpState& s) { return s.op->name; })
+      .def("set_attr", [](OpState& s, const std::string& name, py::object v) {
+        if (py::isinstance<py::bool_>(v)) s.op->attrs[name] = Attribute::boolean(v.cast<bool>());
+        else if (py::isinstance<py::int_>(v)) s.op->attrs[name] = Attribute::integer(v.cast<int64_t>());
+        else if (py::isinstance<py::str>(v)) s.op->attrs[name] = Attribute::string(v.cast<std::string>());
+        else throw std::invalid_argument("set_attr takes a bool, an int or a str");
+      })
+      .def("get_str_attr", [](OpState& s, const std::string& name) -> py::object {
+        auto a = s.op->attr(name);
+        if (!a || a->kind != Attribute::String) return py::none();
+        return py::str(a->s);
+      })
+      .def("dump", [](OpState& s) { std::cerr << print_operation(s.op) << std::endl; })
+      .def("__str__", [](OpState& s) { return print_operation(s.op); })
+      .def("verify", [](OpState& s) {  // failures are reported on stderr, not raised (ffi/ir.cpp:595)
+        Diagnostics d;
+        bool ok = verify_operation(s.op, d);
+        print_diagnostics(d);
+        return ok;
+      });
+
+  py::class_<ModuleOp, OpState>(m, "module", py::module_local(), py::dynamic_attr())
+      .def("dump", [](ModuleOp& s, const std::string& log) {
+        if (!log.empty()) std::cout << log << "\n";
+        std::cout << print_operation(s.op) << std::endl;
+      }, py::arg("log") = "")
+      .def("push_back", [](ModuleOp& s, KernelOp& k) {
+        Block* body = s.op->regions[0]->blocks[0];
+        if (k.op->block) throw std::invalid_argument("kernel is already in a module");
+        k.op->block = body;
+        body->ops.push_back(k.op);
+      })
+      .def("get_kernel", [](ModuleOp& s, const std::string& name) -> py::object {
+        for (Operation* op : s.op->regions[0]->blocks[0]->ops)
+          if (op->name == "frisk.kernel" && op->attr("sym_name")->s == name) { KernelOp k; k.op = op; k.ctx = s.ctx; return py::cast(k); }
+        return py::none();
+      })
+      .def("has_kernel", [](ModuleOp& s, const std::string& name) {
+        for (Operation* op : s.op->regions[0]->blocks[0]->ops)
+          if (op->name == "frisk.kernel" && op->attr("sym_name")->s == name) return true;
+        return false;
+      });
+
+  py::class_<GemmOp, OpState>(m, "GemmOp", py::module_local())
+      .def("get_matrix_A", [](GemmOp& s) { return s.op->operands[0]; })
+      .def("get_matrix_B", [](GemmOp& s) { return s.op->operands[1]; })
+      .def("get_matrix_C", [](GemmOp& s) { return s.op->operands[2]; })
+      .def("get_all_matrix", [](GemmOp& s) { return s.op->operands; })
+      .def("get_m", [](GemmOp& s) { return s.op->int_attr("M"); })
+      .def("get_n", [](GemmOp& s) { return s.op->int_attr("N"); })
+      .def("get_k", [](GemmOp& s) { return s.op->int_attr("K"); });
+  py::class_<KernelOp, OpState>(m, "KernelOp", py::module_local())
+      .def("arg", [](KernelOp& s, unsigned i) {
+        if (s.op->regions[0]->blocks.empty() || i >= s.op->regions[0]->blocks[0]->args.size()) throw py::index_error("Kernel argument index out of range");
+        return Value{s.op->regions[0]->blocks[0]->args[i]};
+      })
+      .def("get_num_arguments", [](KernelOp& s) { return s.op->attr("function_type")->type.impl->inputs.size(); })
+      .def("add_entry_block", [](KernelOp& s) {  // block arguments of the kernel type + frisk.end (FriskOps.td:56-73)
+        std::vector<Type> types;
+        for (auto& t : s.op->attr("function_type")->type.impl->inputs) types.push_back(Type(t));
+        return PyBlock{add_body_block(s.ctx, s.op, types), s.ctx};
+      })
+      .def_property_readonly("type", [](KernelOp& s) { return s.op->attr("function_type")->type; });
+  py::class_<ParallelOp, OpState>(m, "ParallelOp", py::module_local())
+      .def("get_ivs", [](ParallelOp& s) {
+        std::vector<Value> v;
+        if (!s.op->regions[0]->blocks.empty()) for (auto* a : s.op->regions[0]->blocks[0]->args) v.push_back(Value{a});
+        return v;
+      })
+      .def("get_grid", [](ParallelOp& s) { return s.op->attr("ranges")->ints; })
+      .def("get_thread_num", [](ParallelOp& s) { return s.op->int_attr("threads"); })
+      .def("get_grid_dim", [](ParallelOp& s) { return s.op->attr("ranges")->ints.size(); })
+      .def("add_entry_block", [](ParallelOp& s) {  // one index argument per grid dimension + frisk.end (FriskOps.td:119-132)
+        std::vector<Type> types(s.op->attr("ranges")->ints.size(), Type::scalar(TypeKind::Index));
+        return PyBlock{add_body_block(s.ctx, s.op, types), s.ctx};
+      });
+  py::class_<BlockOp, OpState>(m, "BlockOp", py::module_local())
+      .def("get_ivs", [](BlockOp& s) {
+        std::vector<Value> v;
+        for (auto* a : s.op->regions[0]->blocks[0]->args) v.push_back(Value{a});
+        return v;
+      })
+      .def("get_block_ranges", [](BlockOp& s) { return s.op->attr("ranges")->ints; })
+      .def("get_block_dim", [](BlockOp& s) { return s.op->attr("ranges")->ints.size(); });
+  py::class_<ForOp, OpState>(m, "ForOp", py::module_local())
+      .def("get_induction_var", [](ForOp& s) { return Value{s.op->regions[0]->blocks[0]->args[0]}; })
+      .def("get_lower_bound", [](ForOp& s) { return s.op->int_attr("lower"); })
+      .def("get_upper_bound", [](ForOp& s) { return s.op->int_attr("upper"); })
+      .def("get_step", [](ForOp& s) { return s.op->int_attr("step"); });
+  py::class_<AllocBufferOp, OpState>(m, "AllocBufferOp", py::module_local())
+      .def("get_alignment", [](AllocBufferOp& s) { return s.op->int_attr("alignment"); })
+      .def("get_memroy_space", [](AllocBufferOp& s) { return (MemorySpace)s.op->int_attr("memory_space"); })
+      .def("get_result", [](AllocBufferOp& s) { return Value{s.op->results[0]}; })
+      .def("get_memref_ty", [](AllocBufferOp& s) { return s.op->results[0]->type; });
+  py::class_<CopyOp, OpState>(m, "CopyOp", py::module_local())
+      .def("get_src_affine_map", [](CopyOp& s) { return s.op->attr("srcMap")->map; })
+      .def("get_dst_affine_map", [](CopyOp& s) { return s.op->attr("dstMap")->map; })
+      .def("get_src_memref", [](CopyOp& s) { return s.op->operands[0]; })
+      .def("get_dst_memref", [](CopyOp& s) { return s.op->operands[1]; })
+      .def("get_src_indices", [](CopyOp& s) { return std::vector<Value>(s.op->operands.begin() + 2, s.op->operands.begin() + 2 + s.op->src_index_count); })
+      .def("get_dst_indices", [](CopyOp& s) { return std::vector<Value>(s.op->operands.begin() + 2 + s.op->src_index_count, s.op->operands.end()); })
+      .def("get_src_extents", [](CopyOp& s) { return s.op->attr("srcExtents")->ints; })
+      .def("get_dst_extents", [](CopyOp& s) { return s.op->attr("dstExtents")->ints; });
+  py::class_<FillOp, OpState>(m, "FillOp", py::module_local()).def("get_memref", [](FillOp& s) { return s.op->operands[0]; });
+  py::class_<ReduceOp, OpState>(m, "ReduceOp", py::module_local())
+      .def("get_src_memref", [](ReduceOp& s) { return s.op->operands[0]; })
+      .def("get_dst_memref", [](ReduceOp& s) { return s.op->operands[1]; })
+      .def("get_reduce_dim", [](ReduceOp& s) { return s.op->int_attr("dim"); });
+
+  // ---------------------------------------------------------------- builder (ffi/ir.cpp:144-471)
+  py::class_<Builder>(m, "builder")
+      .def(py::init<PyContext&>())
+      .def("create_module", [](Builder& b) {
+        Operation* op = b.ctx->new_op("builtin.module");
+        Region* rg = b.ctx->new_region(op);
+        Block* body = b.ctx->new_block();
+        body->parent = rg;
+        rg->blocks.push_back(body);
+        return b.wrap<ModuleOp>(op);
+      })
+      .def("set_insertion_point_to_start", [](Builder& b, PyBlock& blk) { b.set_to_start(blk.block); })
+      .def("set_insertion_point_to_end", [](Builder& b, PyBlock& blk) { b.set_to_end(blk.block); })
+      .def("set_insertion_point_after", [](Builder& b, OpState& op) { b.set_after(op.op); })
+      .def("get_insertion_block", [](Builder& b) -> py::object {
+        if (!b.block) return py::none();
+        return py::cast(PyBlock{b.block, b.ctx});
+      })
+      .def("new_block", [](Builder& b) { return PyBlock{b.ctx->new_block(), b.ctx}; })
+      .def("get_bool_ty", [](Builder&) { return Type::scalar(TypeKind::I8); })
+      .def("get_int8_ty", [](Builder&) { return Type::scalar(TypeKind::I8); })
+      .def("get_int32_ty", [](Builder&) { return Type::scalar(TypeKind::I32); })
+      .def("get_int64_ty", [](Builder&) { return Type::scalar(TypeKind::I64); })
+      .def("get_index_ty", [](Builder&) { return Type::scalar(TypeKind::Index); })
+      .def("get_f64_ty", [](Builder&) { return Type::scalar(TypeKind::F64); })
+      .def("get_f32_ty", [](Builder&) { return Type::scalar(TypeKind::F32); })
+      .def("get_f16_ty", [](Builder&) { return Type::scalar(TypeKind::F16); })
+      .def("get_bf16_ty", [](Builder&) { return Type::scalar(TypeKind::BF16); })
+      .def("get_f8e4m3fn_ty", [](Builder&) { return Type::scalar(TypeKind::F8E4M3FN); })
+      .def("get_memref_ty", [](Builder&, Type elem, std::vector<int64_t> shape, AffineMap map, MemorySpace space) {
+        return Type::memref(shape, elem, map, (int)space);
+      }, py::arg("elementType"), py::arg("shape"), py::arg("map") = AffineMap(), py::arg("space") = MemorySpace::Global)
+      .def("get_function_ty", [](Builder&, std::vector<Type> in, std::vector<Type> out) { return Type::function(in, out); })
+      .def("get_kernel_ty", [](Builder&, std::vector<Type> in) { return Type::function(in, {}); })
+      .def("get_affine_dim_expr", [](Builder&, unsigned p) { return AffineExpr::dim(p); })
+      .def("get_affine_symbol_expr", [](Builder&, unsigned p) { return AffineExpr::symbol(p); })
+      .def("get_affine_constant_expr", [](Builder&, int64_t v) { return AffineExpr::constant(v); })
+      .def("get_multi_dim_identity_map", [](Builder&, unsigned n) { return AffineMap::identity((int)n); })
+      // ---- frisk ops
+      .def("create_gemm_op", [](Builder& b, Value& A, Value& B, Value& C, bool transA, bool transB, bool clearAccum) {
+        auto require_memref = [](Value& v, const char* name) -> const TypeImpl* {
+          if (!v.type().is_memref()) throw std::invalid_argument(std::string("create_gemm_op expects memref for operand ") + name);
+          return v.type().impl.get();
+        };
+        auto require_static = [](int64_t dim, const char* desc) -> int64_t {
+          if (dim < 0) throw std::invalid_argument(std::string("create_gemm_op requires static ") + desc);
+          return dim;
+        };
+        const TypeImpl *a = require_memref(A, "A"), *bt = require_memref(B, "B"), *c = require_memref(C, "C");
+        if (a->shape.size() != 2 || bt->shape.size() != 2 || c->shape.size() != 2) throw std::invalid_argument("create_gemm_op expects rank-2 memrefs");
+        // Without transpose flags: M, K from A and N from B as stored (ffi/ir.cpp:346-355).  The reference
+        // applies the same reading when a flag is set, which no transposed operand can satisfy; here a set
+        // flag means the operand is stored transposed ([K][M] for A, [N][K] for B).
+        int64_t mm = require_static(a->shape[transA ? 1 : 0], "M dimension of A"), k = require_static(a->shape[transA ? 0 : 1], "K dimension of A");
+        int64_t kb = require_static(bt->shape[transB ? 1 : 0], "K dimension of B");
+        if (k != kb) throw std::invalid_argument("create_gemm_op expects A and B inner dimensions to match");
+        int64_t n = require_static(bt->shape[transB ? 0 : 1], "N dimension of B");
+        int64_t cm = require_static(c->shape[0], "M dimension of C"), cn = require_static(c->shape[1], "N dimension of C");
+        if (mm != cm || n != cn) throw std::invalid_argument("create_gemm_op expects C shape to match A/B product");
+        Type ea(a->element), eb(bt->element), ec(c->element);
+        // same element type for all three as in the reference (ffi/ir.cpp:357-359), or C in the accumulator
+        // type of the inputs (f32 for floating inputs, i32 for i8), which the MFMA path needs
+        bool acc_ok = (ea.is_float() && ec.kind() == TypeKind::F32) || (ea.kind() == TypeKind::I8 && ec.kind() == TypeKind::I32);
+        if (!ea.equals(eb) || !(ea.equals(ec) || acc_ok)) throw std::invalid_argument("create_gemm_op expects operands to have matching element types");
+        Operation* op = b.ctx->new_op("frisk.gemm");
+        op->operands = {A, B, C};
+        op->attrs["transA"] = Attribute::boolean(transA);
+        op->attrs["transB"] = Attribute::boolean(transB);
+        op->attrs["M"] = Attribute::integer(mm);
+        op->attrs["N"] = Attribute::integer(n);
+        op->attrs["K"] = Attribute::integer(k);
+        op->attrs["policy"] = Attribute::policy(GemmWarpPolicy::Square);
+        op->attrs["clear_accum"] = Attribute::boolean(clearAccum);
+        b.insert(op);
+        return b.wrap<GemmOp>(op);
+      }, py::arg("A"), py::arg("B"), py::arg("C"), py::arg("transA") = false, py::arg("transB") = false, py::arg("clear_accum") = false)
+      .def("create_kernel_op", [](Builder& b, ModuleOp& module, const std::string& name, Type& type) {
+        for (Operation* op : module.op->regions[0]->blocks[0]->ops)
+          if (op->name == "frisk.kernel" && op->attr("sym_name")->s == name) return b.wrap<KernelOp>(op);
+        if (type.kind() != TypeKind::Function) throw std::invalid_argument("invalid kernel function type");
+        Operation* op = b.ctx->new_op("frisk.kernel");  // created detached; the caller pushes it into the module
+        op->attrs["sym_name"] = Attribute::string(name);
+        op->attrs["function_type"] = Attribute::type_attr(type);
+        b.ctx->new_region(op);
+        return b.wrap<KernelOp>(op);
+      })
+      .def("create_parallel_op", [](Builder& b, std::vector<int64_t>& grid, int64_t threads) {
+        // only as the first op of a block that so far holds just its terminator (ffi/ir.cpp:375-382)
+        if (!b.block || b.block->ops.size() != 1) throw std::invalid_argument("invalid parallel create");
+        Operation* op = b.ctx->new_op("frisk.parallel");
+        op->attrs["threads"] = Attribute::integer(threads);
+        op->attrs["ranges"] = Attribute::int_array(grid);
+        b.ctx->new_region(op);
+        b.insert(op);
+        return b.wrap<ParallelOp>(op);
+      })
+      .def("create_block_op", [](py::object self, std::vector<int64_t>& ranges, py::function fn) {
+        Builder& b = self.cast<Builder&>();
+        Operation* op = b.ctx->new_op("frisk.block");
+        op->attrs["ranges"] = Attribute::int_array(ranges);
+        Region* rg = b.ctx->new_region(op);
+        Block* body = b.ctx->new_block();
+        body->parent = rg;
+        rg->blocks.push_back(body);
+        std::vector<Value> ivs;
+        for (size_t i = 0; i < ranges.size(); ++i) ivs.push_back(b.ctx->add_block_arg(body, Type::scalar(TypeKind::Index)));
+        Block* saved_block = b.block; Operation* saved_before = b.before;  // InsertionGuard (FriskOps.cpp:1097-1116)
+        b.set_to_start(body);
+        try { fn(self, ivs); } catch (py::error_already_set& e) {
+          std::cerr << "Python exception in frisk block op: " << e.what() << "\n";
+          b.block = saved_block; b.before = saved_before;
+          throw;
+        }
+        Operation* end = b.make_end(); end->block = body; body->ops.push_back(end);
+        b.block = saved_block; b.before = saved_before;
+        b.insert(op);
+        return b.wrap<BlockOp>(op);
+      })
+      .def("create_for_op", [](py::object self, int64_t lower, int64_t upper, int64_t step, py::function fn) {
+        Builder& b = self.cast<Builder&>();
+        Operation* op = b.ctx->new_op("frisk.for");
+        op->attrs["lower"] = Attribute::integer(lower);
+        op->attrs["upper"] = Attribute::integer(upper);
+        op->attrs["step"] = Attribute::integer(step);
+        Region* rg = b.ctx->new_region(op);
+        Block* body = b.ctx->new_block();
+        body->parent = rg;
+        rg->blocks.push_back(body);
+        Value iv = b.ctx->add_block_arg(body, Type::scalar(TypeKind::Index));
+        Block* saved_block = b.block; Operation* saved_before = b.before;  // InsertionGuard (FriskOps.cpp:1198-1218)
+        b.set_to_start(body);
+        try { fn(self, iv); } catch (py::error_already_set& e) {
+          std::cerr << "Python exception in frisk for op: " << e.what() << "\n";
+          b.block = saved_block; b.before = saved_before;
+          throw;
+        }
+        Operation* end = b.make_end(); end->block = body; body->ops.push_back(end);
+        b.block = saved_block; b.before = saved_before;
+        b.insert(op);
+        return b.wrap<ForOp>(op);
+      })
+      .def("create_alloc_buffer_op", [](Builder& b, std::vector<int64_t> shape, const std::string& dtype, MemorySpace space, int64_t alignment) {
+        Type elem = parse_dtype(dtype);
+        if (alignment < 0) throw std::invalid_argument("alignment must be non-negative");
+        Operation* op = b.ctx->new_op("frisk.alloc_buffer");
+        op->attrs["shape"] = Attribute::int_array(shape);
+        op->attrs["elementType"] = Attribute::type_attr(elem);
+        op->attrs["alignment"] = Attribute::integer(alignment);
+        op->attrs["memory_space"] = Attribute::integer((int)space);
+        b.ctx->add_result(op, Type::memref(shape, elem, AffineMap(), (int)space));
+        b.insert(op);
+        return b.wrap<AllocBufferOp>(op);
+      }, py::arg("shape"), py::arg("dtype"), py::arg("space") = MemorySpace::Global, py::arg("alignment") = 0)
+      .def("create_copy_op", [](Builder& b, Value src, Value dst, std::vector<Value> srcIndices, std::vector<Value> dstIndices, AffineMap srcMap,
+                                AffineMap dstMap, std::vector<int64_t> srcExtents, std::vector<int64_t> dstExtents) {
+        if (!src.type().is_memref() || !dst.type().is_memref()) throw std::invalid_argument("create_copy_op expects memref operands");
+        const auto& sshape = src.type().impl->shape; const auto& dshape = dst.type().impl->shape;
+        bool no_maps = !srcMap && !dstMap, both_maps = srcMap && dstMap, no_ext = srcExtents.empty() && dstExtents.empty();
+        bool both_ext = !srcExtents.empty() && !dstExtents.empty();
+        // identity maps + extents from the destination shape, explicit maps, or explicit maps and extents;
+        // the fourth form (extents with default maps) is what a tile copy with plain tile indices needs.
+        // Any other mix ends the process in the reference (a bare `throw;`, ffi/ir.cpp:443-446); here it raises.
+        if (!((no_maps || both_maps) && (no_ext || both_ext))) throw std::invalid_argument("copy op map error.");
+        if (no_maps) { srcMap = AffineMap::identity((int)sshape.size()); dstMap = AffineMap::identity((int)dshape.size()); }
+        if ((int)srcIndices.size() != srcMap.num_inputs()) throw std::invalid_argument("source map inputs must match source indices count");
+        if ((int)dstIndices.size() != dstMap.num_inputs()) throw std::invalid_argument("destination map inputs must match destination indices count");
+        if (no_ext) {  // destination shape, left-padded with 1s to the source rank (FriskOps.cpp:1564-1591)
+          if (sshape.size() < dshape.size()) throw std::invalid_argument("src rank must be >= dst rank");
+          size_t pad = sshape.size() - dshape.size();
+          for (size_t i = 0; i < sshape.size(); ++i) srcExtents.push_back(i < pad ? 1 : dshape[i - pad]);
+          dstExtents = dshape;
+        }
+        Operation* op = b.ctx->new_op("frisk.copy");
+        op->operands = {src, dst};
+        op->operands.insert(op->operands.end(), srcIndices.begin(), srcIndices.end());
+        op->operands.insert(op->operands.end(), dstIndices.begin(), dstIndices.end());
+        op->src_index_count = (int)srcIndices.size();
+        op->attrs["srcMap"] = Attribute::affine_map(srcMap);
+        op->attrs["dstMap"] = Attribute::affine_map(dstMap);
+        op->attrs["srcExtents"] = Attribute::int_array(srcExtents);
+        op->attrs["dstExtents"] = Attribute::int_array(dstExtents);
+        b.insert(op);
+        return b.wrap<CopyOp>(op);
+      }, py::arg("src"), py::arg("dst"), py::arg("srcIndices"), py::arg("dstIndices"), py::arg("srcMap") = AffineMap(), py::arg("dstMap") = AffineMap(),
+         py::arg("srcExtents") = std::vector<int64_t>(), py::arg("dstExtents") = std::vector<int64_t>())
+      .def("create_fill_op", [](Builder& b, Value memref, float value, const std::string& dtype) {
+        Type t = parse_dtype(dtype);
+        Operation* op = b.ctx->new_op("frisk.fill");
+        op->operands = {memref};
+        op->attrs["value"] = Attribute::floating((double)value, t);
+        b.insert(op);
+        return b.wrap<FillOp>(op);
+      })
+      .def("create_reduce_op", [](Builder& b, Value src, Value dst, const std::string& kind, int64_t dim, bool clear) {
+        Operation* op = b.ctx->new_op("frisk.reduce");
+        op->operands = {src, dst};
+        op->attrs["kind"] = Attribute::string(kind);
+        op->attrs["dim"] = Attribute::integer(dim);
+        op->attrs["clear"] = Attribute::boolean(clear);
+        b.insert(op);
+        return b.wrap<ReduceOp>(op);
+      }, py::arg("src"), py::arg("dst"), py::arg("kind"), py::arg("dim"), py::arg("clear") = true);
+
+  // ---------------------------------------------------------------- dialect registration (ffi/ir.cpp:33-47)
+  auto frisk = m.def_submodule("frisk");
+  frisk.def("load_dialects", [](PyContext& c) { c.ctx->dialects_loaded = true; });
+}
+
+// used by runtime.cpp
+frisk_ir::Operation* op_of_handle(py::handle h) { return h.cast<OpState&>().op; }
+
+}  // namespace frisk_ffi

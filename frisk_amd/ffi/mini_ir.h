@@ -1,0 +1,815 @@
+// A small, MLIR-free IR that carries the Frisk dialect's GEMM program:
+// module / kernel / parallel / block / for / end / alloc_buffer / copy / fill /
+// reduce / gemm, memref and function types, affine maps, and the textual form
+// MLIR prints for them.
+//
+// The reference builds these ops with MLIR (include/Dialect/Frisk/IR/FriskOps.td,
+// lib/Dialect/Frisk/IR/FriskOps.cpp) and exposes an OpBuilder to Python
+// (ffi/ir.cpp).  MLIR is not available where this runs, so the data model,
+// the custom printers (FriskOps.cpp:953-973 kernel, :1023-1038 parallel,
+// :1147-1162 block, :1250-1259 for, :1519-1545 alloc_buffer, :1642-1665 copy,
+// assembly formats FriskOps.td:244,288,409,442) and the verifiers
+// (:901-920 kernel, :1264-1283 gemm, :1436-1481 alloc_buffer, :1666-1683 copy,
+// :1688-1701 fill, :1725-1767 reduce) are restated here over plain structs.
+#pragma once
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <deque>
+#include <functional>
+#include <map>
+#include <memory>
+#include <sstream>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace frisk_ir {
+
+// ------------------------------------------------------------------ enums
+// numeric values as in include/Dialect/Frisk/IR/FriskEnums.td:6-25; the memory
+// space number is what a memref type prints (", 1>" global, ", 3>" shared, nothing for local)
+enum class MemorySpace : int { Local = 0, Global = 1, Shared = 3 };
+enum class GemmWarpPolicy : int { Square = 0, FullRow = 1, FullCol = 2 };
+
+inline const char* policy_name(GemmWarpPolicy p) {
+  switch (p) {
+    case GemmWarpPolicy::Square: return "Square";
+    case GemmWarpPolicy::FullRow: return "FullRow";
+    default: return "FullCol";
+  }
+}
+
+// ------------------------------------------------------------------ affine expressions
+enum class ExprKind : int { Add = 0, Mul = 1, Mod = 2, FloorDiv = 3, CeilDiv = 4, Constant = 5, DimId = 6, SymbolId = 7, Null = -1 };
+
+struct AffineExprImpl {
+  ExprKind kind;
+  int64_t value;  // constant value or position
+  std::shared_ptr<const AffineExprImpl> lhs, rhs;
+};
+
+struct AffineExpr {
+  std::shared_ptr<const AffineExprImpl> impl;
+  AffineExpr() = default;
+  explicit AffineExpr(std::shared_ptr<const AffineExprImpl> i) : impl(std::move(i)) {}
+  explicit operator bool() const { return (bool)impl; }
+  ExprKind kind() const { return impl ? impl->kind : ExprKind::Null; }
+  static AffineExpr constant(int64_t v) { return AffineExpr(std::make_shared<AffineExprImpl>(AffineExprImpl{ExprKind::Constant, v, nullptr, nullptr})); }
+  static AffineExpr dim(int64_t p) { return AffineExpr(std::make_shared<AffineExprImpl>(AffineExprImpl{ExprKind::DimId, p, nullptr, nullptr})); }
+  static AffineExpr symbol(int64_t p) { return AffineExpr(std::make_shared<AffineExprImpl>(AffineExprImpl{ExprKind::SymbolId, p, nullptr, nullptr})); }
+  bool is_constant() const { return kind() == ExprKind::Constant; }
+  int64_t constant_value() const { return impl->value; }
+  bool equals(const AffineExpr& o) const {
+    if (!impl || !o.impl) return !impl && !o.impl;
+    if (impl->kind != o.impl->kind) return false;
+    if (impl->kind >= ExprKind::Constant) return impl->value == o.impl->value;
+    return AffineExpr(impl->lhs).equals(AffineExpr(o.impl->lhs)) && AffineExpr(impl->rhs).equals(AffineExpr(o.impl->rhs));
+  }
+  static int64_t floordiv(int64_t a, int64_t b) { int64_t q = a / b; return (a % b != 0 && ((a < 0) != (b < 0))) ? q - 1 : q; }
+  static AffineExpr binary(ExprKind k, AffineExpr l, AffineExpr r) {
+    if (!l || !r) throw std::invalid_argument("affine expression operand is null");
+    if (l.is_constant() && r.is_constant()) {
+      int64_t a = l.constant_value(), b = r.constant_value();
+      switch (k) {
+        case ExprKind::Add: return constant(a + b);
+        case ExprKind::Mul: return constant(a * b);
+        case ExprKind::Mod: if (b > 0) return constant(a - floordiv(a, b) * b); break;
+        case ExprKind::FloorDiv: if (b > 0) return constant(floordiv(a, b)); break;
+        case ExprKind::CeilDiv: if (b > 0) return constant(-floordiv(-a, b)); break;
+        default: break;
+      }
+    }
+    // canonical position of the constant: right-hand side (as MLIR does)
+    if ((k == ExprKind::Add || k == ExprKind::Mul) && l.is_constant()) std::swap(l, r);
+    if (r.is_constant()) {
+      int64_t c = r.constant_value();
+      if (k == ExprKind::Add && c == 0) return l;
+      if (k == ExprKind::Mul && c == 1) return l;
+      if (k == ExprKind::Mul && c == 0) return constant(0);
+      if ((k == ExprKind::FloorDiv || k == ExprKind::CeilDiv) && c == 1) return l;
+      if (k == ExprKind::Mod && c == 1) return constant(0);
+    }
+    return AffineExpr(std::make_shared<AffineExprImpl>(AffineExprImpl{k, 0, l.impl, r.impl}));
+  }
+  AffineExpr operator+(const AffineExpr& o) const { return binary(ExprKind::Add, *this, o); }
+  AffineExpr operator+(int64_t v) const { return *this + constant(v); }
+  AffineExpr operator*(const AffineExpr& o) const { return binary(ExprKind::Mul, *this, o); }
+  AffineExpr operator*(int64_t v) const { return *this * constant(v); }
+  AffineExpr operator-() const { return *this * constant(-1); }
+  AffineExpr operator-(const AffineExpr& o) const { return *this + (-o); }
+  AffineExpr operator-(int64_t v) const { return *this + constant(-v); }
+  AffineExpr floor_div(const AffineExpr& o) const { return binary(ExprKind::FloorDiv, *this, o); }
+  AffineExpr ceil_div(const AffineExpr& o) const { return binary(ExprKind::CeilDiv, *this, o); }
+  AffineExpr mod(const AffineExpr& o) const { return binary(ExprKind::Mod, *this, o); }
+
+  int64_t eval(const std::vector<int64_t>& dims, const std::vector<int64_t>& syms) const {
+    switch (kind()) {
+      case ExprKind::Constant: return impl->value;
+      case ExprKind::DimId: return dims.at((size_t)impl->value);
+      case ExprKind::SymbolId: return syms.at((size_t)impl->value);
+      default: break;
+    }
+    int64_t a = AffineExpr(impl->lhs).eval(dims, syms), b = AffineExpr(impl->rhs).eval(dims, syms);
+    switch (kind()) {
+      case ExprKind::Add: return a + b;
+      case ExprKind::Mul: return a * b;
+      case ExprKind::Mod: return a - floordiv(a, b) * b;
+      case ExprKind::FloorDiv: return floordiv(a, b);
+      case ExprKind::CeilDiv: return -floordiv(-a, b);
+      default: throw std::invalid_argument("cannot evaluate a null affine expression");
+    }
+  }
+  // MLIR's spelling; `names` substitutes SSA names for dims (then symbols) when given
+  std::string str(const std::vector<std::string>* names = nullptr, int num_dims = 0, bool nested = false) const {
+    switch (kind()) {
+      case ExprKind::Null: return "<<NULL AFFINE EXPR>>";
+      case ExprKind::Constant: return std::to_string(impl->value);
+      case ExprKind::DimId: return names ? names->at((size_t)impl->value) : "d" + std::to_string(impl->value);
+      case ExprKind::SymbolId: return names ? names->at((size_t)(num_dims + impl->value)) : "s" + std::to_string(impl->value);
+      default: break;
+    }
+    AffineExpr l(impl->lhs), r(impl->rhs);
+    std::string out;
+    // binding strength as in MLIR's printer: operands of * mod floordiv ceildiv are parenthesised when
+    // they are sums; operands of a sum never are
+    if (kind() == ExprKind::Add) {
+      // a + (-1) * b and a + (-c) print as subtractions
+      if (r.kind() == ExprKind::Mul && AffineExpr(r.impl->rhs).is_constant() && AffineExpr(r.impl->rhs).constant_value() == -1)
+        out = l.str(names, num_dims, false) + " - " + AffineExpr(r.impl->lhs).str(names, num_dims, true);
+      else if (r.is_constant() && r.constant_value() < 0)
+        out = l.str(names, num_dims, false) + " - " + std::to_string(-r.constant_value());
+      else
+        out = l.str(names, num_dims, false) + " + " + r.str(names, num_dims, false);
+      return nested ? "(" + out + ")" : out;
+    }
+    const char* op = kind() == ExprKind::Mul ? " * " : kind() == ExprKind::Mod ? " mod " : kind() == ExprKind::FloorDiv ? " floordiv " : " ceildiv ";
+    if (kind() == ExprKind::Mul && r.is_constant() && r.constant_value() == -1) return "-" + l.str(names, num_dims, true);
+    return l.str(names, num_dims, true) + op + r.str(names, num_dims, true);
+  }
+  std::string unused_tail_(bool nested, const std::string& out) const {
+    return nested ? "(" + out + ")" : out;
+  }
+};
+
+struct AffineMapImpl {
+  int num_dims, num_symbols;
+  std::vector<AffineExpr> results;
+};
+
+// default-constructed = "no map" (falsy), as the reference's AffineMap() default argument (ffi/ir.cpp:252-256, 649)
+struct AffineMap {
+  std::shared_ptr<const AffineMapImpl> impl;
+  AffineMap() = default;
+  AffineMap(int dims, int syms, std::vector<AffineExpr> results) : impl(std::make_shared<AffineMapImpl>(AffineMapImpl{dims, syms, std::move(results)})) {}
+  explicit operator bool() const { return (bool)impl; }
+  static AffineMap identity(int n) {
+    std::vector<AffineExpr> r;
+    for (int i = 0; i < n; ++i) r.push_back(AffineExpr::dim(i));
+    return AffineMap(n, 0, r);
+  }
+  int num_dims() const { return impl ? impl->num_dims : 0; }
+  int num_symbols() const { return impl ? impl->num_symbols : 0; }
+  int num_inputs() const { return num_dims() + num_symbols(); }
+  int num_results() const { return impl ? (int)impl->results.size() : 0; }
+  bool is_identity() const {
+    if (!impl || impl->num_symbols || num_results() != num_dims()) return false;
+    for (int i = 0; i < num_results(); ++i)
+      if (impl->results[i].kind() != ExprKind::DimId || impl->results[i].impl->value != i) return false;
+    return true;
+  }
+  bool equals(const AffineMap& o) const {
+    if (!impl || !o.impl) return !impl && !o.impl;
+    if (impl->num_dims != o.impl->num_dims || impl->num_symbols != o.impl->num_symbols || impl->results.size() != o.impl->results.size()) return false;
+    for (size_t i = 0; i < impl->results.size(); ++i)
+      if (!impl->results[i].equals(o.impl->results[i])) return false;
+    return true;
+  }
+  std::string str() const {
+    if (!impl) return "<<NULL AFFINE MAP>>";
+    std::ostringstream os;
+    os << "(";
+    for (int i = 0; i < impl->num_dims; ++i) os << (i ? ", " : "") << "d" << i;
+    os << ")";
+    if (impl->num_symbols) {
+      os << "[";
+      for (int i = 0; i < impl->num_symbols; ++i) os << (i ? ", " : "") << "s" << i;
+      os << "]";
+    }
+    os << " -> (";
+    for (size_t i = 0; i < impl->results.size(); ++i) os << (i ? ", " : "") << impl->results[i].str();
+    os << ")";
+    return os.str();
+  }
+};
+
+// ------------------------------------------------------------------ types
+enum class TypeKind { None, F16, BF16, F32, F64, F8E4M3FN, F8E5M2, I1, I8, I32, I64, Index, MemRef, Function, RankedTensor };
+
+struct TypeImpl {
+  TypeKind kind = TypeKind::None;
+  std::vector<int64_t> shape;                            // memref / tensor
+  std::shared_ptr<const TypeImpl> element;               // memref / tensor
+  int memory_space = 0;                                  // memref
+  AffineMap layout;                                      // memref (only the default is printed away)
+  std::vector<std::shared_ptr<const TypeImpl>> inputs, results;  // function
+};
+
+struct Type {
+  std::shared_ptr<const TypeImpl> impl;
+  Type() = default;
+  explicit Type(std::shared_ptr<const TypeImpl> i) : impl(std::move(i)) {}
+  explicit operator bool() const { return (bool)impl; }
+  TypeKind kind() const { return impl ? impl->kind : TypeKind::None; }
+  static Type scalar(TypeKind k) { auto t = std::make_shared<TypeImpl>(); t->kind = k; return Type(t); }
+  static Type memref(std::vector<int64_t> shape, Type elem, AffineMap layout, int space) {
+    auto t = std::make_shared<TypeImpl>();
+    t->kind = TypeKind::MemRef; t->shape = std::move(shape); t->element = elem.impl; t->memory_space = space; t->layout = layout;
+    return Type(t);
+  }
+  static Type tensor(std::vector<int64_t> shape, Type elem) {
+    auto t = std::make_shared<TypeImpl>();
+    t->kind = TypeKind::RankedTensor; t->shape = std::move(shape); t->element = elem.impl;
+    return Type(t);
+  }
+  static Type function(const std::vector<Type>& in, const std::vector<Type>& out) {
+    auto t = std::make_shared<TypeImpl>();
+    t->kind = TypeKind::Function;
+    for (auto& x : in) t->inputs.push_back(x.impl);
+    for (auto& x : out) t->results.push_back(x.impl);
+    return Type(t);
+  }
+  bool is_float() const {
+    switch (kind()) { case TypeKind::F16: case TypeKind::BF16: case TypeKind::F32: case TypeKind::F64: case TypeKind::F8E4M3FN: case TypeKind::F8E5M2: return true; default: return false; }
+  }
+  bool is_int() const { return kind() == TypeKind::I1 || kind() == TypeKind::I8 || kind() == TypeKind::I32 || kind() == TypeKind::I64; }
+  bool is_memref() const { return kind() == TypeKind::MemRef; }
+  Type element() const { return Type(impl->element); }
+  int bit_width() const {
+    switch (kind()) {
+      case TypeKind::F16: case TypeKind::BF16: return 16;
+      case TypeKind::F32: case TypeKind::I32: return 32;
+      case TypeKind::F64: case TypeKind::I64: case TypeKind::Index: return 64;
+      case TypeKind::F8E4M3FN: case TypeKind::F8E5M2: case TypeKind::I8: return 8;
+      case TypeKind::I1: return 1;
+      default: return 0;
+    }
+  }
+  bool equals(const Type& o) const {
+    if (!impl || !o.impl) return !impl && !o.impl;
+    if (impl->kind != o.impl->kind) return false;
+    if (impl->kind == TypeKind::MemRef || impl->kind == TypeKind::RankedTensor)
+      return impl->shape == o.impl->shape && element().equals(o.element()) && impl->memory_space == o.impl->memory_space &&
+             impl->layout.equals(o.impl->layout);
+    if (impl->kind == TypeKind::Function) {
+      if (impl->inputs.size() != o.impl->inputs.size() || impl->results.size() != o.impl->results.size()) return false;
+      for (size_t i = 0; i < impl->inputs.size(); ++i) if (!Type(impl->inputs[i]).equals(Type(o.impl->inputs[i]))) return false;
+      for (size_t i = 0; i < impl->results.size(); ++i) if (!Type(impl->results[i]).equals(Type(o.impl->results[i]))) return false;
+    }
+    return true;
+  }
+  std::string str() const {
+    switch (kind()) {
+      case TypeKind::None: return "<<NULL TYPE>>";
+      case TypeKind::F16: return "f16";
+      case TypeKind::BF16: return "bf16";
+      case TypeKind::F32: return "f32";
+      case TypeKind::F64: return "f64";
+      case TypeKind::F8E4M3FN: return "f8E4M3FN";
+      case TypeKind::F8E5M2: return "f8E5M2";
+      case TypeKind::I1: return "i1";
+      case TypeKind::I8: return "i8";
+      case TypeKind::I32: return "i32";
+      case TypeKind::I64: return "i64";
+      case TypeKind::Index: return "index";
+      default: break;
+    }
+    std::ostringstream os;
+    if (kind() == TypeKind::MemRef || kind() == TypeKind::RankedTensor) {
+      os << (kind() == TypeKind::MemRef ? "memref<" : "tensor<");
+      for (int64_t d : impl->shape) { if (d < 0) os << "?x"; else os << d << "x"; }
+      os << element().str();
+      if (kind() == TypeKind::MemRef) {
+        if (impl->layout && !impl->layout.is_identity()) os << ", affine_map<" << impl->layout.str() << ">";
+        if (impl->memory_space != 0) os << ", " << impl->memory_space;
+      }
+      os << ">";
+      return os.str();
+    }
+    os << "(";
+    for (size_t i = 0; i < impl->inputs.size(); ++i) os << (i ? ", " : "") << Type(impl->inputs[i]).str();
+    os << ") -> ";
+    if (impl->results.size() == 1 && Type(impl->results[0]).kind() != TypeKind::Function) os << Type(impl->results[0]).str();
+    else {
+      os << "(";
+      for (size_t i = 0; i < impl->results.size(); ++i) os << (i ? ", " : "") << Type(impl->results[i]).str();
+      os << ")";
+    }
+    return os.str();
+  }
+};
+
+// ------------------------------------------------------------------ attributes
+struct Attribute {
+  enum Kind { None, Bool, Int, Float, String, Policy, IntArray, Map, TypeAttr } kind = None;
+  bool b = false;
+  int64_t i = 0;
+  int int_width = 64;
+  double f = 0.0;
+  Type type;  // of a float / type attribute
+  std::string s;
+  std::vector<int64_t> ints;
+  AffineMap map;
+  static Attribute boolean(bool v) { Attribute a; a.kind = Bool; a.b = v; return a; }
+  static Attribute integer(int64_t v, int width = 64) { Attribute a; a.kind = Int; a.i = v; a.int_width = width; return a; }
+  static Attribute floating(double v, Type t) { Attribute a; a.kind = Float; a.f = v; a.type = t; return a; }
+  static Attribute string(std::string v) { Attribute a; a.kind = String; a.s = std::move(v); return a; }
+  static Attribute policy(GemmWarpPolicy p) { Attribute a; a.kind = Policy; a.i = (int)p; return a; }
+  static Attribute int_array(std::vector<int64_t> v) { Attribute a; a.kind = IntArray; a.ints = std::move(v); return a; }
+  static Attribute affine_map(AffineMap m) { Attribute a; a.kind = Map; a.map = m; return a; }
+  static Attribute type_attr(Type t) { Attribute a; a.kind = TypeAttr; a.type = t; return a; }
+
+  static std::string float_str(double v) {
+    // MLIR prints "%.6e" style when that round-trips, otherwise more digits
+    if (std::isnan(v)) return "0x7FC00000";
+    if (std::isinf(v)) return v > 0 ? "0x7F800000" : "0xFF800000";
+    char buf[64];
+    std::snprintf(buf, sizeof buf, "%.6e", v);
+    if (std::strtod(buf, nullptr) == v) return buf;
+    std::snprintf(buf, sizeof buf, "%.17g", v);
+    return buf;
+  }
+  std::string str() const {
+    switch (kind) {
+      case Bool: return b ? "true" : "false";
+      case Int: return std::to_string(i) + " : i" + std::to_string(int_width);
+      case Float: return float_str(f) + " : " + type.str();
+      case String: return "\"" + s + "\"";
+      case Policy: return std::string("#frisk<gemm_warp_policy ") + policy_name((GemmWarpPolicy)i) + ">";
+      case IntArray: {
+        std::string o = "array<i64";
+        for (size_t k = 0; k < ints.size(); ++k) o += (k ? ", " : ": ") + std::to_string(ints[k]);
+        return o + ">";
+      }
+      case Map: return "affine_map<" + map.str() + ">";
+      case TypeAttr: return type.str();
+      default: return "<<NULL ATTRIBUTE>>";
+    }
+  }
+};
+
+// ------------------------------------------------------------------ values, operations, blocks, regions
+struct Operation;
+struct Block;
+struct Region;
+
+struct ValueImpl {
+  Type type;
+  Operation* def = nullptr;  // result of this operation ...
+  Block* block = nullptr;    // ... or argument of this block
+  int index = 0;
+};
+
+struct Value {
+  ValueImpl* impl = nullptr;
+  explicit operator bool() const { return impl != nullptr; }
+  Type type() const { return impl ? impl->type : Type(); }
+  bool operator==(const Value& o) const { return impl == o.impl; }
+};
+
+struct Region {
+  Operation* parent = nullptr;
+  std::vector<Block*> blocks;
+};
+
+struct Block {
+  Region* parent = nullptr;
+  std::vector<ValueImpl*> args;
+  std::vector<Operation*> ops;
+  bool has_terminator() const;
+};
+
+struct Operation {
+  std::string name;  // "frisk.gemm", "builtin.module", ...
+  std::vector<Value> operands;
+  std::vector<ValueImpl*> results;
+  std::map<std::string, Attribute> attrs;  // sorted by name, as MLIR stores them
+  std::vector<Region*> regions;
+  Block* block = nullptr;  // where it is inserted
+  int src_index_count = 0; // frisk.copy: operands are [src, dst, srcIndices..., dstIndices...]
+  bool is_terminator() const { return name == "frisk.end" || name == "func.return"; }
+  const Attribute* attr(const std::string& n) const { auto it = attrs.find(n); return it == attrs.end() ? nullptr : &it->second; }
+  int64_t int_attr(const std::string& n) const { auto a = attr(n); if (!a) throw std::invalid_argument("missing attribute " + n); return a->i; }
+  bool bool_attr(const std::string& n) const { auto a = attr(n); return a && a->b; }
+};
+
+inline bool Block::has_terminator() const { return !ops.empty() && ops.back()->is_terminator(); }
+
+// Owns every IR object created through it; handles on the Python side are raw
+// pointers, valid for as long as the context lives (the tests keep it alive by
+// stashing it on the module, as they do for the reference).
+struct Context {
+  std::deque<std::unique_ptr<Operation>> ops;
+  std::deque<std::unique_ptr<Block>> blocks;
+  std::deque<std::unique_ptr<Region>> regions;
+  std::deque<std::unique_ptr<ValueImpl>> values;
+  bool dialects_loaded = false;
+  bool multithreading = true;
+  Operation* new_op(const std::string& name) { ops.emplace_back(new Operation()); ops.back()->name = name; return ops.back().get(); }
+  Block* new_block() { blocks.emplace_back(new Block()); return blocks.back().get(); }
+  Region* new_region(Operation* parent) { regions.emplace_back(new Region()); regions.back()->parent = parent; parent->regions.push_back(regions.back().get()); return regions.back().get(); }
+  ValueImpl* new_value(Type t) { values.emplace_back(new ValueImpl()); values.back()->type = t; return values.back().get(); }
+  Value add_result(Operation* op, Type t) { ValueImpl* v = new_value(t); v->def = op; v->index = (int)op->results.size(); op->results.push_back(v); return Value{v}; }
+  Value add_block_arg(Block* b, Type t) { ValueImpl* v = new_value(t); v->block = b; v->index = (int)b->args.size(); b->args.push_back(v); return Value{v}; }
+};
+
+// ------------------------------------------------------------------ printer
+struct Printer {
+  std::map<const ValueImpl*, std::string> names;
+  int next_arg = 0, next_result = 0;
+  std::ostringstream os;
+
+  void number_block(Block* b) {
+    for (ValueImpl* a : b->args) names[a] = "%arg" + std::to_string(next_arg++);
+    for (Operation* op : b->ops) {
+      for (ValueImpl* r : op->results) names[r] = "%" + std::to_string(next_result++);
+      for (Region* rg : op->regions) for (Block* nb : rg->blocks) number_block(nb);
+    }
+  }
+  // SSA names restart inside every kernel / function (they are isolated from above)
+  void number_isolated(Operation* op) {
+    next_arg = next_result = 0;
+    for (Region* rg : op->regions) for (Block* b : rg->blocks) number_block(b);
+  }
+  std::string name(Value v) {
+    auto it = names.find(v.impl);
+    return it == names.end() ? "<<UNKNOWN SSA VALUE>>" : it->second;
+  }
+  void indent(int n) { for (int i = 0; i < n; ++i) os << "  "; }
+  void attr_dict(const Operation* op, const std::vector<std::string>& elided, bool leading_space = true) {
+    std::vector<std::pair<std::string, const Attribute*>> shown;
+    for (auto& kv : op->attrs) {
+      bool skip = false;
+      for (auto& e : elided) skip = skip || e == kv.first;
+      if (!skip) shown.push_back({kv.first, &kv.second});
+    }
+    if (shown.empty()) return;
+    os << (leading_space ? " {" : "{");
+    for (size_t i = 0; i < shown.size(); ++i) os << (i ? ", " : "") << shown[i].first << " = " << shown[i].second->str();
+    os << "}";
+  }
+  void region(Region* rg, int ind) {
+    os << "{\n";
+    for (Block* b : rg->blocks)
+      for (Operation* op : b->ops) {
+        if (op->name == "frisk.end") continue;  // printBlockTerminators = false
+        operation(op, ind + 1);
+      }
+    indent(ind);
+    os << "}";
+  }
+  void map_of_ssa_ids(const AffineMap& m, const std::vector<Value>& ids) {
+    std::vector<std::string> n;
+    for (auto& v : ids) n.push_back(name(v));
+    for (int i = 0; i < m.num_results(); ++i) os << (i ? ", " : "") << m.impl->results[i].str(&n, m.num_dims());
+  }
+  void operation(Operation* op, int ind) {
+    indent(ind);
+    if (!op->results.empty()) {
+      for (size_t i = 0; i < op->results.size(); ++i) os << (i ? ", " : "") << names[op->results[i]];
+      os << " = ";
+    }
+    const std::string& n = op->name;
+    if (n == "builtin.module") {
+      os << "module";
+      attr_dict(op, {}, true);
+      if (!op->attrs.empty()) os << " ";
+      else os << " ";
+      for (Operation* k : op->regions[0]->blocks[0]->ops) (void)k;
+      os << "{\n";
+      for (Operation* k : op->regions[0]->blocks[0]->ops) {
+        if (k->name == "frisk.kernel" || k->name == "func.func") number_isolated(k);
+        operation(k, ind + 1);
+      }
+      indent(ind);
+      os << "}";
+    } else if (n == "frisk.kernel") {
+      os << "frisk.kernel @" << op->attr("sym_name")->s << "(";
+      const Type& ft = op->attr("function_type")->type;
+      for (size_t i = 0; i < ft.impl->inputs.size(); ++i) os << (i ? ", " : "") << Type(ft.impl->inputs[i]).str();
+      os << ")";
+      if (!ft.impl->results.empty()) {
+        os << " -> (";
+        for (size_t i = 0; i < ft.impl->results.size(); ++i) os << (i ? ", " : "") << Type(ft.impl->results[i]).str();
+        os << ")";
+      }
+      os << " ";
+      region(op->regions[0], ind);
+      attr_dict(op, {"sym_name", "function_type"});
+    } else if (n == "frisk.parallel" || n == "frisk.block") {
+      os << n << " (";
+      Block* body = op->regions[0]->blocks.empty() ? nullptr : op->regions[0]->blocks[0];
+      if (body) for (size_t i = 0; i < body->args.size(); ++i) os << (i ? ", " : "") << names[body->args[i]];
+      os << ")";
+      const auto& r = op->attr(n == "frisk.parallel" ? "ranges" : "ranges")->ints;
+      os << (n == "frisk.parallel" ? " = (" : " to (");
+      for (size_t i = 0; i < r.size(); ++i) os << (i ? ", " : "") << r[i];
+      os << ")";
+      if (n == "frisk.parallel") os << ", threads = " << op->int_attr("threads");
+      os << " ";
+      region(op->regions[0], ind);
+    } else if (n == "frisk.for") {
+      Block* body = op->regions[0]->blocks[0];
+      os << "frisk.for " << names[body->args[0]] << " = " << op->int_attr("lower") << " to " << op->int_attr("upper");
+      if (op->int_attr("step") > 1) os << " step = " << op->int_attr("step");
+      os << " ";
+      region(op->regions[0], ind);
+    } else if (n == "frisk.alloc_buffer") {
+      os << "frisk.alloc_buffer {scope = \"";
+      switch ((MemorySpace)op->int_attr("memory_space")) {
+        case MemorySpace::Local: os << "local"; break;
+        case MemorySpace::Global: os << "global"; break;
+        case MemorySpace::Shared: os << "shared"; break;
+        default: os << "unknown";
+      }
+      os << "\"";
+      if (op->int_attr("alignment") != 0) os << ", alignment = " << op->int_attr("alignment");
+      os << "} -> " << op->results[0]->type.str();
+    } else if (n == "frisk.copy") {
+      std::vector<Value> si(op->operands.begin() + 2, op->operands.begin() + 2 + op->src_index_count);
+      std::vector<Value> di(op->operands.begin() + 2 + op->src_index_count, op->operands.end());
+      os << "frisk.copy " << name(op->operands[0]) << "[";
+      map_of_ssa_ids(op->attr("srcMap")->map, si);
+      os << "], " << name(op->operands[1]) << "[";
+      map_of_ssa_ids(op->attr("dstMap")->map, di);
+      os << "] {src_extents = [";
+      const auto& se = op->attr("srcExtents")->ints;
+      const auto& de = op->attr("dstExtents")->ints;
+      for (size_t i = 0; i < se.size(); ++i) os << (i ? ", " : "") << se[i];
+      os << "], dst_extents = [";
+      for (size_t i = 0; i < de.size(); ++i) os << (i ? ", " : "") << de[i];
+      os << "]} ";
+      attr_dict(op, {"srcMap", "dstMap", "srcExtents", "dstExtents"});
+      os << " : " << op->operands[0].type().str() << ", " << op->operands[1].type().str();
+    } else if (n == "frisk.gemm") {
+      os << "frisk.gemm(" << name(op->operands[0]) << ", " << name(op->operands[1]) << ", " << name(op->operands[2]) << ")";
+      attr_dict(op, {});
+      os << " : " << op->operands[0].type().str() << ", " << op->operands[1].type().str() << ", " << op->operands[2].type().str();
+    } else if (n == "frisk.fill") {
+      os << "frisk.fill " << name(op->operands[0]);
+      attr_dict(op, {});
+      os << " : " << op->operands[0].type().str();
+    } else if (n == "frisk.reduce") {
+      os << "frisk.reduce " << name(op->operands[0]) << ", " << name(op->operands[1]);
+      attr_dict(op, {});
+      os << " : " << op->operands[0].type().str() << ", " << op->operands[1].type().str();
+    } else if (n == "frisk.end") {
+      os << "frisk.end";
+    } else {
+      os << "\"" << n << "\"(";
+      for (size_t i = 0; i < op->operands.size(); ++i) os << (i ? ", " : "") << name(op->operands[i]);
+      os << ")";
+      attr_dict(op, {});
+    }
+    os << "\n";
+  }
+};
+
+inline Operation* enclosing_isolated(Operation* op) {
+  Operation* cur = op;
+  while (cur && cur->name != "frisk.kernel" && cur->name != "func.func" && cur->name != "builtin.module")
+    cur = (cur->block && cur->block->parent) ? cur->block->parent->parent : nullptr;
+  return cur ? cur : op;
+}
+
+inline std::string print_operation(Operation* op) {
+  Printer p;
+  Operation* root = enclosing_isolated(op);
+  if (root->name != "builtin.module") p.number_isolated(root);
+  p.operation(op, 0);
+  std::string s = p.os.str();
+  if (!s.empty() && s.back() == '\n') s.pop_back();
+  return s;
+}
+
+// ------------------------------------------------------------------ verifier
+struct Diagnostics {
+  std::vector<std::string> errors;
+  void error(const Operation* op, const std::string& msg) { errors.push_back("'" + op->name + "' op " + msg); }
+};
+
+inline bool verify_operation(const Operation* op, Diagnostics& d);
+
+inline bool verify_region_ops(const Operation* op, Diagnostics& d) {
+  bool ok = true;
+  for (Region* rg : op->regions)
+    for (Block* b : rg->blocks)
+      for (Operation* inner : b->ops) ok = verify_operation(inner, d) && ok;
+  return ok;
+}
+
+inline bool verify_operation(const Operation* op, Diagnostics& d) {
+  bool ok = true;
+  auto fail = [&](const std::string& m) { d.error(op, m); ok = false; };
+  const std::string& n = op->name;
+  auto memref_operand = [&](size_t i, const char* what) -> const TypeImpl* {
+    if (i >= op->operands.size() || !op->operands[i].type().is_memref()) { fail(std::string("operand ") + what + " must be a memref"); return nullptr; }
+    return op->operands[i].type().impl.get();
+  };
+  if (n == "frisk.kernel") {
+    const Attribute* ft = op->attr("function_type");
+    if (!ft || ft->type.kind() != TypeKind::Function) fail("requires a 'function_type' attribute");
+    else if (op->regions.empty() || op->regions[0]->blocks.empty()) fail("requires an entry block");
+    else {
+      Block* body = op->regions[0]->blocks[0];
+      if (body->args.size() != ft->type.impl->inputs.size()) fail("region argument count does not match function type");
+      else for (size_t i = 0; i < body->args.size(); ++i)
+        if (!body->args[i]->type.equals(Type(ft->type.impl->inputs[i]))) fail("region argument type mismatch");
+      if (!body->has_terminator()) fail("entry block must end with frisk.end");
+    }
+  } else if (n == "frisk.parallel" || n == "frisk.block" || n == "frisk.for") {
+    if (op->regions.empty() || op->regions[0]->blocks.empty()) fail("requires a body block");
+    else {
+      Block* body = op->regions[0]->blocks[0];
+      size_t want = n == "frisk.for" ? 1 : op->attr(n == "frisk.parallel" ? "ranges" : "ranges")->ints.size();
+      if (body->args.size() != want) fail("body block must carry one index argument per range");
+      if (!body->has_terminator()) fail("body block must end with frisk.end");
+    }
+    if (n == "frisk.parallel") {
+      if (op->int_attr("threads") <= 0) fail("requires a positive thread count");
+      for (int64_t r : op->attr("ranges")->ints) if (r <= 0) fail("grid ranges must be positive");
+    }
+    if (n == "frisk.for" && op->int_attr("step") <= 0) fail("requires a positive step");
+  } else if (n == "frisk.gemm") {
+    const TypeImpl *a = memref_operand(0, "A"), *b = memref_operand(1, "B"), *c = memref_operand(2, "C");
+    if (a && b && c) {
+      if (a->shape.size() != 2 || b->shape.size() != 2 || c->shape.size() != 2) fail("expects rank-2 memrefs");
+      else {
+        // FriskOps.cpp:1274-1281 checks the shapes as stored; a set transpose flag swaps the operand's two extents
+        const bool ta = op->bool_attr("transA"), tb = op->bool_attr("transB");
+        if (a->shape[ta ? 1 : 0] != op->int_attr("M") || a->shape[ta ? 0 : 1] != op->int_attr("K")) fail("A shape does not match M x K");
+        if (b->shape[tb ? 1 : 0] != op->int_attr("K") || b->shape[tb ? 0 : 1] != op->int_attr("N")) fail("B shape does not match K x N");
+        if (c->shape[0] != op->int_attr("M") || c->shape[1] != op->int_attr("N")) fail("C shape does not match M x N");
+      }
+      if (!Type(a->element).equals(Type(b->element))) fail("A and B must have the same element type");
+    }
+  } else if (n == "frisk.alloc_buffer") {
+    const Type& t = op->results[0]->type;
+    if (!t.is_memref()) fail("result must be a memref");
+    else {
+      if (t.impl->shape != op->attr("shape")->ints) fail("result shape does not match the shape attribute");
+      for (int64_t s : t.impl->shape) if (s <= 0) fail("shape must be static and positive");
+      if (!t.element().equals(op->attr("elementType")->type)) fail("result element type does not match the elementType attribute");
+      if (t.impl->memory_space != op->int_attr("memory_space")) fail("result memory space does not match the memory_space attribute");
+      int64_t al = op->int_attr("alignment");
+      if (al < 0 || (al & (al - 1)) != 0) fail("alignment must be zero or a power of two");
+    }
+  } else if (n == "frisk.copy") {
+    const TypeImpl *s = memref_operand(0, "src"), *t = memref_operand(1, "dst");
+    const AffineMap& sm = op->attr("srcMap")->map;
+    const AffineMap& dm = op->attr("dstMap")->map;
+    int ns = op->src_index_count, nd = (int)op->operands.size() - 2 - ns;
+    if (ns != sm.num_inputs()) fail("expected " + std::to_string(sm.num_inputs()) + " source indices, but got " + std::to_string(ns));
+    if (nd != dm.num_inputs()) fail("expected " + std::to_string(dm.num_inputs()) + " destination indices, but got " + std::to_string(nd));
+    if (s && sm.num_results() != (int)s->shape.size()) fail("source map must produce one index per source dimension");
+    if (t && dm.num_results() != (int)t->shape.size()) fail("destination map must produce one index per destination dimension");
+  } else if (n == "frisk.fill") {
+    const TypeImpl* m = memref_operand(0, "memref");
+    if (m && !Type(m->element).equals(op->attr("value")->type)) fail("fill value type does not match the memref element type");
+  } else if (n == "frisk.reduce") {
+    const TypeImpl *s = memref_operand(0, "src"), *t = memref_operand(1, "dst");
+    const std::string& kind = op->attr("kind")->s;
+    if (kind != "add" && kind != "mul" && kind != "min" && kind != "max" && kind != "sum") fail("unknown reduce kind '" + kind + "'");
+    if (s) {
+      int64_t dim = op->int_attr("dim");
+      if (dim < 0 || dim >= (int64_t)s->shape.size()) fail("reduce dimension out of range");
+      else if (t) {
+        std::vector<int64_t> want = s->shape;
+        want.erase(want.begin() + dim);
+        std::vector<int64_t> keep = s->shape;
+        keep[(size_t)dim] = 1;
+        if (t->shape != want && t->shape != keep) fail("destination shape must be the source shape without (or with extent 1 in) the reduced dimension");
+      }
+    }
+  }
+  return verify_region_ops(op, d) && ok;
+}
+
+// ------------------------------------------------------------------ the tiled GEMM program
+// What the runtime extracts from
+//   kernel(A, B, C [, ...]) { parallel (by, bx) = (gm, gn), threads = T {
+//     sA = alloc_buffer shared; sB = alloc_buffer shared; acc = alloc_buffer local
+//     fill acc, 0 ; for k { copy A -> sA ; copy B -> sB ; gemm(sA, sB, acc) } ; copy acc -> C } }
+// (the program shape of the reference's tmp/ir.mlir:1-17).
+struct GemmProgram {
+  std::string kernel_name;
+  int arg_a = -1, arg_b = -1, arg_c = -1;  // kernel argument positions
+  Type elem_ab, elem_acc, elem_out;
+  int64_t M = 0, N = 0, K = 0;
+  int64_t tile_m = 0, tile_n = 0, tile_k = 0;
+  int64_t grid_m = 0, grid_n = 0, threads = 0;
+  bool transA = false, transB = false, clear_accum = true;
+  GemmWarpPolicy policy = GemmWarpPolicy::Square;
+  std::string target = "gfx950";
+};
+
+inline int kernel_arg_index(const Operation* kernel, Value v) {
+  Block* entry = kernel->regions[0]->blocks[0];
+  if (v.impl && v.impl->block == entry) return v.impl->index;
+  return -1;
+}
+
+inline GemmProgram match_tiled_gemm(Operation* kernel, Operation* module = nullptr) {
+  auto bad = [](const std::string& m) -> GemmProgram { throw std::invalid_argument("not a tiled GEMM kernel: " + m); };
+  if (!kernel || kernel->name != "frisk.kernel") return bad("expected a frisk.kernel");
+  if (kernel->regions.empty() || kernel->regions[0]->blocks.empty()) return bad("kernel has no entry block");
+  GemmProgram g;
+  g.kernel_name = kernel->attr("sym_name")->s;
+  for (const Operation* scope : {(const Operation*)kernel, (const Operation*)module})
+    if (scope) if (auto t = scope->attr("frisk.target")) { g.target = t->s; break; }
+  if (g.target.rfind("gfx950", 0) != 0) return bad("frisk.target '" + g.target + "' is not gfx950");
+  Block* entry = kernel->regions[0]->blocks[0];
+  Operation* par = nullptr;
+  for (Operation* op : entry->ops) {
+    if (op->name == "frisk.parallel") { if (par) return bad("more than one frisk.parallel"); par = op; }
+    else if (op->name != "frisk.end") return bad("unexpected '" + op->name + "' at kernel level");
+  }
+  if (!par) return bad("no frisk.parallel");
+  const auto& grid = par->attr("ranges")->ints;
+  if (grid.size() != 2) return bad("frisk.parallel must have a 2-D grid (tiles along M, tiles along N)");
+  g.grid_m = grid[0]; g.grid_n = grid[1]; g.threads = par->int_attr("threads");
+  if (par->regions[0]->blocks.empty()) return bad("frisk.parallel has no body");
+  Block* body = par->regions[0]->blocks[0];
+
+  Operation *loop = nullptr, *gemm = nullptr, *store = nullptr, *fill = nullptr;
+  std::vector<Operation*> allocs;
+  for (Operation* op : body->ops) {
+    if (op->name == "frisk.alloc_buffer") allocs.push_back(op);
+    else if (op->name == "frisk.fill") fill = op;
+    else if (op->name == "frisk.for") { if (loop) return bad("more than one frisk.for"); loop = op; }
+    else if (op->name == "frisk.copy") { if (store) return bad("more than one copy after the K loop"); if (!loop) return bad("copy before the K loop"); store = op; }
+    else if (op->name != "frisk.end") return bad("unexpected '" + op->name + "' in frisk.parallel");
+  }
+  if (!loop) return bad("no frisk.for over K");
+  if (!store) return bad("no copy of the accumulator to global memory");
+  std::vector<Operation*> loads;
+  for (Operation* op : loop->regions[0]->blocks[0]->ops) {
+    if (op->name == "frisk.copy") loads.push_back(op);
+    else if (op->name == "frisk.gemm") { if (gemm) return bad("more than one frisk.gemm"); gemm = op; }
+    else if (op->name != "frisk.end") return bad("unexpected '" + op->name + "' in the K loop");
+  }
+  if (!gemm) return bad("no frisk.gemm in the K loop");
+  if (loads.size() != 2) return bad("the K loop must stage exactly A and B");
+
+  Value sA = gemm->operands[0], sB = gemm->operands[1], acc = gemm->operands[2];
+  auto space_of = [](Value v) { return v.type().impl->memory_space; };
+  if (space_of(sA) != (int)MemorySpace::Shared || space_of(sB) != (int)MemorySpace::Shared) return bad("gemm operands A and B must live in shared memory");
+  if (space_of(acc) != (int)MemorySpace::Local) return bad("gemm operand C must be a local fragment");
+  Value gA, gB;
+  for (Operation* cp : loads) {
+    if (cp->operands[1] == sA) gA = cp->operands[0];
+    else if (cp->operands[1] == sB) gB = cp->operands[0];
+    else return bad("a copy in the K loop does not feed the gemm");
+  }
+  if (!gA || !gB) return bad("A or B is not staged in the K loop");
+  if (!(store->operands[0] == acc)) return bad("the copy after the K loop must read the accumulator");
+  Value gC = store->operands[1];
+  g.arg_a = kernel_arg_index(kernel, gA); g.arg_b = kernel_arg_index(kernel, gB); g.arg_c = kernel_arg_index(kernel, gC);
+  if (g.arg_a < 0 || g.arg_b < 0 || g.arg_c < 0) return bad("A, B and C must be kernel arguments");
+  for (Value v : {gA, gB, gC}) if (space_of(v) != (int)MemorySpace::Global) return bad("kernel arguments must be global memrefs");
+
+  g.transA = gemm->bool_attr("transA"); g.transB = gemm->bool_attr("transB");
+  g.policy = (GemmWarpPolicy)gemm->attr("policy")->i;
+  // clear_accum on the gemm restarts the sum every K step; the tiled program clears once with fill 0
+  if (gemm->bool_attr("clear_accum")) return bad("gemm inside the K loop must accumulate (clear_accum = false)");
+  g.clear_accum = fill && fill->operands[0] == acc && fill->attr("value")->f == 0.0;
+  g.tile_m = gemm->int_attr("M"); g.tile_n = gemm->int_attr("N"); g.tile_k = gemm->int_attr("K");
+  const auto& sa = sA.type().impl->shape; const auto& sb = sB.type().impl->shape; const auto& sc = acc.type().impl->shape;
+  // with a transposed operand the staged tile is stored transposed, like the global operand
+  if (g.transA) { if (sa[0] != g.tile_k && sa[1] != g.tile_k) return bad("shared A tile does not match the gemm K"); }
+  (void)sb; (void)sc;
+  const auto& ga = gA.type().impl->shape; const auto& gb = gB.type().impl->shape; const auto& gc = gC.type().impl->shape;
+  if (ga.size() != 2 || gb.size() != 2 || gc.size() != 2) return bad("A, B and C must be rank-2");
+  g.M = gc[0]; g.N = gc[1];
+  g.K = g.transA ? ga[0] : ga[1];
+  int64_t mA = g.transA ? ga[1] : ga[0], kB = g.transB ? gb[1] : gb[0], nB = g.transB ? gb[0] : gb[1];
+  if (mA != g.M || nB != g.N || kB != g.K) return bad("global operand shapes are inconsistent");
+  // tile extents as staged: op(A) tile is tile_m x tile_k, op(B) tile is tile_k x tile_n
+  int64_t tm = g.transA ? sa[1] : sa[0], tkA = g.transA ? sa[0] : sa[1];
+  int64_t tkB = g.transB ? sb[1] : sb[0], tn = g.transB ? sb[0] : sb[1];
+  if (tkA != tkB) return bad("shared A and B tiles disagree on the K extent");
+  if (sc.size() != 2 || sc[0] != tm || sc[1] != tn) return bad("accumulator fragment does not match the staged tiles");
+  g.tile_m = tm; g.tile_n = tn; g.tile_k = tkA;
+  if (g.grid_m * g.tile_m != g.M || g.grid_n * g.tile_n != g.N) return bad("grid x tile does not cover C exactly");
+  int64_t lo = loop->int_attr("lower"), hi = loop->int_attr("upper"), step = loop->int_attr("step");
+  int64_t trips = (hi - lo + step - 1) / step;
+  if (trips * g.tile_k != g.K && (hi - lo) != g.K) return bad("the K loop does not cover K exactly");
+  g.elem_ab = sA.type().element();
+  if (!g.elem_ab.equals(sB.type().element()) || !g.elem_ab.equals(gA.type().element()) || !g.elem_ab.equals(gB.type().element()))
+    return bad("A and B element types differ between global and shared memory");
+  g.elem_acc = acc.type().element();
+  g.elem_out = gC.type().element();
+  return g;
+}
+
+}  // namespace frisk_ir

@@ -1,0 +1,163 @@
+// `frisk_ffi.runtime`: lowers a tiled-GEMM kernel built with the IR builder to a
+// frisk_gemm_desc and launches it through the C ABI of libfrisk_hip.so
+// (include/frisk_hip.h).  This fills the slot the reference reserves for
+// `init_ffi_passes` (ffi/ffi.h:14, ffi/ffi.cpp:6): the reference has nothing
+// below its builder, so what it would lower to is the library's entry points.
+// There is no other execution path: without the library every call here raises.
+#include <dlfcn.h>
+
+#include <mutex>
+
+#include "ffi.h"
+#include "frisk_hip.h"
+#include "mini_ir.h"
+
+namespace frisk_ffi {
+
+using namespace frisk_ir;
+frisk_ir::Operation* op_of_handle(py::handle h);
+
+namespace {
+
+struct HipLibrary {
+  void* handle = nullptr;
+  std::string path;
+  decltype(&frisk_hip_plan) plan = nullptr;
+  decltype(&frisk_hip_gemm) gemm = nullptr;
+  decltype(&frisk_hip_last_error) last_error = nullptr;
+  decltype(&frisk_hip_abi_version) abi_version = nullptr;
+  decltype(&frisk_hip_kernel_name) kernel_name = nullptr;
+};
+
+HipLibrary g_lib;
+std::string g_lib_path;
+std::mutex g_lib_mutex;
+
+HipLibrary& library() {
+  std::lock_guard<std::mutex> lock(g_lib_mutex);
+  if (g_lib.handle) return g_lib;
+  if (g_lib_path.empty()) throw std::runtime_error("frisk runtime: the path of libfrisk_hip.so has not been set (runtime.set_library)");
+  void* h = dlopen(g_lib_path.c_str(), RTLD_NOW | RTLD_LOCAL);
+  if (!h) throw std::runtime_error(std::string("frisk runtime: cannot load ") + g_lib_path + ": " + dlerror());
+  HipLibrary lib;
+  lib.handle = h;
+  lib.path = g_lib_path;
+  lib.plan = (decltype(lib.plan))dlsym(h, "frisk_hip_plan");
+  lib.gemm = (decltype(lib.gemm))dlsym(h, "frisk_hip_gemm");
+  lib.last_error = (decltype(lib.last_error))dlsym(h, "frisk_hip_last_error");
+  lib.abi_version = (decltype(lib.abi_version))dlsym(h, "frisk_hip_abi_version");
+  lib.kernel_name = (decltype(lib.kernel_name))dlsym(h, "frisk_hip_kernel_name");
+  if (!lib.plan || !lib.gemm || !lib.last_error || !lib.abi_version || !lib.kernel_name)
+    throw std::runtime_error("frisk runtime: " + g_lib_path + " does not export the frisk_hip entry points");
+  if (lib.abi_version() != FRISK_HIP_ABI_VERSION) throw std::runtime_error("frisk runtime: libfrisk_hip.so ABI version mismatch");
+  g_lib = lib;
+  return g_lib;
+}
+
+int dtype_of(const Type& t) {
+  switch (t.kind()) {
+    case TypeKind::F32: return FRISK_F32;
+    case TypeKind::F16: return FRISK_F16;
+    case TypeKind::BF16: return FRISK_BF16;
+    case TypeKind::I8: return FRISK_I8;
+    case TypeKind::F8E4M3FN: return FRISK_E4M3;
+    case TypeKind::I32: return FRISK_I32;
+    default: throw std::invalid_argument("element type " + t.str() + " has no gfx950 GEMM kernel");
+  }
+}
+
+int epilogue_of(const std::string& e) {
+  if (e == "none") return FRISK_EPI_NONE;
+  if (e == "row_col_scale") return FRISK_EPI_ROW_COL_SCALE;
+  if (e == "tensor_scale") return FRISK_EPI_TENSOR_SCALE;
+  throw std::invalid_argument("unknown epilogue '" + e + "' (none, row_col_scale, tensor_scale)");
+}
+
+frisk_gemm_desc desc_of(const GemmProgram& g, int epilogue) {
+  frisk_gemm_desc d{};
+  d.abi_version = FRISK_HIP_ABI_VERSION;
+  d.dtype_ab = dtype_of(g.elem_ab);
+  d.dtype_acc = dtype_of(g.elem_acc);
+  d.dtype_out = dtype_of(g.elem_out);
+  d.M = g.M; d.N = g.N; d.K = g.K;
+  d.lda = g.transA ? g.M : g.K;
+  d.ldb = g.transB ? g.K : g.N;
+  d.ldc = g.N;
+  d.transA = g.transA; d.transB = g.transB; d.clear_accum = g.clear_accum;
+  d.epilogue = epilogue;
+  d.policy = (int)g.policy;
+  d.tile_m = (int)g.tile_m; d.tile_n = (int)g.tile_n; d.tile_k = (int)g.tile_k;
+  return d;
+}
+
+GemmProgram program_of(py::object kernel, py::object module) {
+  Operation* k = op_of_handle(kernel);
+  Operation* m = module.is_none() ? nullptr : op_of_handle(module);
+  return match_tiled_gemm(k, m);
+}
+
+py::dict program_dict(const GemmProgram& g) {
+  py::dict d;
+  d["kernel"] = g.kernel_name;
+  d["M"] = g.M; d["N"] = g.N; d["K"] = g.K;
+  d["tile"] = py::make_tuple(g.tile_m, g.tile_n, g.tile_k);
+  d["grid"] = py::make_tuple(g.grid_m, g.grid_n);
+  d["threads"] = g.threads;
+  d["transA"] = g.transA; d["transB"] = g.transB; d["clear_accum"] = g.clear_accum;
+  d["dtype_ab"] = g.elem_ab.str(); d["dtype_acc"] = g.elem_acc.str(); d["dtype_out"] = g.elem_out.str();
+  d["args"] = py::make_tuple(g.arg_a, g.arg_b, g.arg_c);
+  d["target"] = g.target;
+  return d;
+}
+
+}  // namespace
+
+void init_ffi_runtime(py::module_&& m) {
+  m.def("set_library", [](const std::string& path) {
+    std::lock_guard<std::mutex> lock(g_lib_mutex);
+    g_lib_path = path;
+  }, "path of libfrisk_hip.so; loaded on first use");
+  m.def("library_path", []() { return g_lib_path; });
+
+  m.def("match", [](py::object kernel, py::object module) { return program_dict(program_of(kernel, module)); }, py::arg("kernel"),
+        py::arg("module") = py::none(),
+        "recognise kernel{parallel{alloc, alloc, alloc, fill, for{copy, copy, gemm}, copy}} and return the GEMM it describes; pure host");
+
+  m.def("plan", [](py::object kernel, py::object module, const std::string& epilogue) {
+    GemmProgram g = program_of(kernel, module);
+    frisk_gemm_desc d = desc_of(g, epilogue_of(epilogue));
+    HipLibrary& lib = library();
+    frisk_gemm_plan p{};
+    if (int st = lib.plan(&d, &p)) throw std::invalid_argument(std::string("frisk_hip_plan: ") + lib.last_error() + " (status " + std::to_string(st) + ")");
+    py::dict out = program_dict(g);
+    out["hip_kernel"] = p.kernel_id >= 0 ? std::string(lib.kernel_name(p.kernel_id)) : std::string();
+    out["hip_tile"] = py::make_tuple(p.tile_m, p.tile_n, p.tile_k);
+    out["hip_waves"] = py::make_tuple(p.waves_m, p.waves_n);
+    out["hip_grid"] = py::make_tuple(p.grid_y, p.grid_x);
+    out["lds_bytes"] = p.lds_bytes;
+    out["stages"] = p.stages;
+    out["flops"] = p.flops;
+    out["bytes"] = p.bytes;
+    return out;
+  }, py::arg("kernel"), py::arg("module") = py::none(), py::arg("epilogue") = "none");
+
+  m.def("launch", [](py::object kernel, std::vector<uint64_t> args, uint64_t stream, py::object module, const std::string& epilogue,
+                     uint64_t scale_a, uint64_t scale_b) {
+    GemmProgram g = program_of(kernel, module);
+    size_t need = (size_t)std::max(g.arg_a, std::max(g.arg_b, g.arg_c)) + 1;
+    if (args.size() < need) throw std::invalid_argument("launch needs one device pointer per kernel argument");
+    frisk_gemm_desc d = desc_of(g, epilogue_of(epilogue));
+    HipLibrary& lib = library();
+    int st;
+    {
+      py::gil_scoped_release release;
+      st = lib.gemm(&d, (const void*)args[(size_t)g.arg_a], (const void*)args[(size_t)g.arg_b], (void*)args[(size_t)g.arg_c], (const float*)scale_a,
+                    (const float*)scale_b, nullptr, 0, (void*)stream);
+    }
+    if (st) throw std::runtime_error(std::string("frisk_hip_gemm: ") + lib.last_error() + " (status " + std::to_string(st) + ")");
+  }, py::arg("kernel"), py::arg("args"), py::arg("stream") = 0, py::arg("module") = py::none(), py::arg("epilogue") = "none",
+     py::arg("scale_a") = 0, py::arg("scale_b") = 0,
+     "asynchronous launch on `stream` (a hipStream_t value); `args` holds one raw device pointer per kernel argument");
+}
+
+}  // namespace frisk_ffi

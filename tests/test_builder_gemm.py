@@ -1,0 +1,184 @@
+"""The builder surface, driven exactly as the reference's own scripts drive it
+(test/python/bind_test.py:3-62, test/python/helper_test.py:4-24), and checked against the
+output the reference saved for bind_test.py (tmp/log_11_18, kept as tests/golden/bind_test_module.mlir)."""
+import os
+
+import pytest
+
+import frisk_amd  # noqa: F401  (puts the `frisk` package on the path)
+import frisk as F
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def create_gemmop():
+    """call for call the body of bind_test.py:create_gemmop"""
+    context = F.context()
+    F.frisk.load_dialects(context)
+    builder = F.builder(context)
+    module = builder.create_module()
+    module.context = context
+
+    shape = [4096, 4096]
+    shape2 = [4096]
+    dtype = builder.get_f16_ty()
+    mem_type = builder.get_memref_ty(dtype, shape, F.AffineMap(), F.MemorySpace.GLOBAL)
+    mem2_type = builder.get_memref_ty(dtype, shape2, F.AffineMap(), F.MemorySpace.GLOBAL)
+    kernel_type = builder.get_kernel_ty([mem_type, mem_type, mem_type, mem2_type])
+    kernel = builder.create_kernel_op(module, "test_gemm", kernel_type)
+    module.push_back(kernel)
+    entry1 = kernel.add_entry_block()
+    builder.set_insertion_point_to_start(entry1)
+    prarllel = builder.create_parallel_op([8, 8], 128)
+    entry2 = prarllel.add_entry_block()
+    builder.set_insertion_point_to_start(entry2)
+
+    input_val = [entry1.get_argument(0), entry1.get_argument(1), entry1.get_argument(2), entry1.get_argument(3)]
+
+    builder.create_alloc_buffer_op([128, 32], "fp16", F.MemorySpace.SHARED, 1024)
+    builder.create_alloc_buffer_op([32, 128], "fp16", F.MemorySpace.SHARED, 1024)
+    builder.create_alloc_buffer_op([128, 128], "fp16", F.MemorySpace.LOCAL)
+
+    def for_body_test(b, iv):
+        builder.create_fill_op(input_val[0], 0.0, "fp16")
+        builder.create_reduce_op(input_val[0], input_val[3], "max", 1, True)
+        builder.create_copy_op(input_val[0], input_val[1], [iv, iv], [iv, iv])
+
+        def block_body_test(b, ivs):
+            b.create_gemm_op(input_val[0], input_val[1], input_val[2])
+
+        builder.create_block_op([128, 128], block_body_test)
+
+    builder.create_for_op(0, 128, 1, for_body_test)
+    return module
+
+
+def test_bind_test_module_prints_as_the_reference_saved_it():
+    module = create_gemmop()
+    want = open(os.path.join(GOLDEN, "bind_test_module.mlir")).read().strip("\n")
+    assert str(module) == want
+    assert module.verify()
+
+
+def test_helper_test_sequence():
+    """call for call helper_test.py:build_sample_module, with its three asserts"""
+    helper = F.create_session()
+    f16 = helper.builder.get_f16_ty()
+    a_ty = helper.memref_type((128, 64), f16, space=F.MemorySpace.SHARED)
+    b_ty = helper.memref_type((64, 128), f16, space=F.MemorySpace.SHARED)
+    c_ty = helper.memref_type((128, 128), f16, space=F.MemorySpace.LOCAL)
+    kernel, entry = helper.new_kernel("helper_demo", [a_ty, b_ty, c_ty])
+    args = [entry.get_argument(i) for i in range(3)]
+    gemm = helper.create_gemm(args[0], args[1], args[2])
+    scratch = helper.alloc_buffer((32, 32), "fp16", space=F.MemorySpace.SHARED, alignment=64)
+    assert "memref" in str(scratch.get_type())
+    assert kernel.verify()
+    assert helper.module.verify()
+    assert (gemm.get_m(), gemm.get_n(), gemm.get_k()) == (128, 128, 64)
+    text = str(helper.module)
+    assert "frisk.kernel @helper_demo(memref<128x64xf16, 3>, memref<64x128xf16, 3>, memref<128x128xf16>)" in text
+    assert '%0 = frisk.alloc_buffer {scope = "shared", alignment = 64} -> memref<32x32xf16, 3>' in text
+
+
+def test_enum_values_and_type_printing():
+    # Local = 0, Global = 1, Shared = 3 (reference output tmp/log_11_25:5-8); the number is what a memref prints
+    assert int(F.MemorySpace.LOCAL) == 0 and int(F.MemorySpace.GLOBAL) == 1 and int(F.MemorySpace.SHARED) == 3
+    h = F.create_session()
+    assert str(h.memref_type((4, 8), "fp32")) == "memref<4x8xf32, 1>"
+    assert str(h.memref_type((4, 8), "bf16", space=F.MemorySpace.LOCAL)) == "memref<4x8xbf16>"
+    assert not F.AffineMap() and F.AffineMap.get_multi_dim_identity_map(2)
+    t = h.memref_type((16, 32), "fp16", space=F.MemorySpace.SHARED)
+    assert t.get_shape() == [16, 32] and t.get_rank() == 2 and t.get_elem_width() == 16 and t.get_memory_space() == F.MemorySpace.SHARED
+
+
+def test_error_conventions():
+    h = F.create_session()
+    f16, f32 = h.builder.get_f16_ty(), h.builder.get_f32_ty()
+    kernel, entry = h.new_kernel("k", [h.memref_type((128, 64), f16), h.memref_type((32, 128), f16), h.memref_type((128, 128), f16),
+                                       h.memref_type((64, 128), f32), h.memref_type((128,), f16)])
+    a, b_bad, c, b_f32, vec = (entry.get_argument(i) for i in range(5))
+    with pytest.raises(ValueError, match="inner dimensions"):
+        h.builder.create_gemm_op(a, b_bad, c)
+    with pytest.raises(ValueError, match="matching element types"):
+        h.builder.create_gemm_op(a, b_f32, c)
+    with pytest.raises(ValueError, match="rank-2"):
+        h.builder.create_gemm_op(a, vec, c)
+    with pytest.raises(ValueError, match="invalid float type"):
+        h.builder.create_alloc_buffer_op([8, 8], "fp13")
+    with pytest.raises(ValueError, match="non-negative"):
+        h.builder.create_alloc_buffer_op([8, 8], "fp16", F.MemorySpace.SHARED, -4)
+    with pytest.raises(IndexError):
+        entry.get_argument(9)
+    with pytest.raises(ValueError, match="copy op map error"):
+        h.builder.create_copy_op(a, c, [], [], F.AffineMap.get_multi_dim_identity_map(2))   # only one of the two maps
+    # parallel must be the first op of a block that holds only its terminator
+    h.builder.create_alloc_buffer_op([8, 8], "fp16")
+    with pytest.raises(ValueError, match="invalid parallel create"):
+        h.builder.create_parallel_op([2, 2], 64)
+    # verifier failures are reported through the return value, not raised
+    h2 = F.create_session()
+    k2, e2 = h2.new_kernel("k2", [h2.memref_type((8, 8), f16)])
+    h2.builder.create_fill_op(e2.get_argument(0), 1.0, "fp32")
+    assert not k2.verify() and not h2.module.verify()
+
+
+def test_body_callbacks_propagate_python_errors_and_restore_the_insertion_point():
+    h = F.create_session()
+    kernel, entry = h.new_kernel("k", [h.memref_type((8, 8), "fp16")])
+
+    def boom(b, iv):
+        raise KeyError("inside the body")
+
+    with pytest.raises(KeyError):
+        h.builder.create_for_op(0, 4, 1, boom)
+    h.builder.create_fill_op(entry.get_argument(0), 0.0, "fp16")   # lands in the kernel body, not in the abandoned loop
+    assert str(h.module).count("frisk.fill") == 1 and "frisk.for" not in str(h.module)
+
+
+def test_affine_maps_of_a_tiled_copy_print_like_mlir():
+    h = F.create_session()
+    b = h.builder
+    d0, d1 = b.get_affine_dim_expr(0), b.get_affine_dim_expr(1)
+    m = F.AffineMap.get(2, 0, [d0 * 128, d1 * 32 + 5])
+    assert str(m) == "(d0, d1) -> (d0 * 128, d1 * 32 + 5)"
+    assert (d0 * 128).evaluate([3, 0]) == 384 and ((d0 + d1 * 2) % 3).evaluate([4, 1]) == 0
+    assert str((d0 + 7).floor_div(4)) == "(d0 + 7) floordiv 4" and str(d0 - d1) == "d0 - d1"
+
+
+def test_tiled_gemm_program_matches_the_design_sketch():
+    """fp32 1024^3, grid 8x8, 128 threads, shared A 128x32, shared B 32x128, fragment C 128x128:
+    the matmul program of the reference's tmp/ir.mlir:1-17, built through the builder"""
+    h = F.create_session()
+    kernel = h.tiled_gemm("matmul", 1024, 1024, 1024, "fp32", tile=(128, 128, 32), threads=128)
+    assert kernel.verify() and h.module.verify()
+    text = str(h.module)
+    assert "frisk.parallel (%arg3, %arg4) = (8, 8), threads = 128 {" in text
+    assert "frisk.for %arg5 = 0 to 32 {" in text
+    assert "frisk.copy %arg0[%arg3 * 128, %arg5 * 32], %0[0, 0] {src_extents = [128, 32], dst_extents = [128, 32]}" in text
+    assert "frisk.copy %arg1[%arg5 * 32, %arg4 * 128], %1[0, 0] {src_extents = [32, 128], dst_extents = [32, 128]}" in text
+    assert "frisk.copy %2[0, 0], %arg2[%arg3 * 128, %arg4 * 128]" in text
+    p = F.runtime.match(kernel)
+    assert (p["M"], p["N"], p["K"]) == (1024, 1024, 1024) and p["tile"] == (128, 128, 32) and p["grid"] == (8, 8)
+    assert p["threads"] == 128 and p["clear_accum"] and not p["transA"] and not p["transB"]
+    assert (p["dtype_ab"], p["dtype_acc"], p["dtype_out"]) == ("f32", "f32", "f32") and p["args"] == (0, 1, 2)
+
+
+def test_matcher_rejects_what_is_not_a_tiled_gemm():
+    module = create_gemmop()                      # the bind_test module: gemm on global memrefs inside a block op
+    with pytest.raises(ValueError, match="not a tiled GEMM"):
+        F.runtime.match(module.get_kernel("test_gemm"))
+    h = F.create_session()
+    kernel = h.tiled_gemm("g", 512, 512, 512, "fp16", tile=(256, 256, 64))
+    kernel.set_attr("frisk.target", "sm_80")      # the reference's layout inference only knows sm_80 / sm_90; this path only gfx950
+    with pytest.raises(ValueError, match="gfx950"):
+        F.runtime.match(kernel)
+    kernel.set_attr("frisk.target", "gfx950")
+    assert F.runtime.match(kernel)["target"] == "gfx950"
+
+
+def test_plan_goes_through_the_hip_library():
+    h = F.create_session()
+    kernel = h.tiled_gemm("g", 4096, 4096, 4096, "fp16", tile=(256, 256, 64), trans_b=True)
+    p = F.runtime.plan(kernel)
+    assert p["hip_tile"] == (256, 256, 64) and p["hip_grid"] == (16, 16) and p["lds_bytes"] <= 160 * 1024
+    assert p["hip_kernel"].startswith("f16_nt_256x256x64") and p["flops"] == 2.0 * 4096 ** 3

@@ -1,0 +1,62 @@
+"""End to end through the drop-in surface: build the tiled GEMM with the IR builder, let
+frisk_ffi.runtime lower it to the C ABI, run it on the GPU, compare with the CPU oracle."""
+import numpy as np
+import pytest
+
+import frisk_amd  # noqa: F401
+import frisk as F
+import oracle as O
+from helpers import from_dev, make_operand, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(kernel, A, B, M, N, out_np, **kw):
+    import torch
+    dA, dB = to_dev(A), to_dev(B)
+    dC = torch.full((M * N * np.dtype(out_np).itemsize,), 0xFF, dtype=torch.uint8, device="cuda")
+    F.runtime.launch(kernel, [dA.data_ptr(), dB.data_ptr(), dC.data_ptr()], torch.cuda.current_stream().cuda_stream, **kw)
+    torch.cuda.synchronize()
+    return from_dev(dC, out_np, (M, N))
+
+
+def test_config1_fp32_1024_built_through_the_builder(hip):
+    """fp32 C = A.B, M = N = K = 1024, uniform[-1, 1] seed 0: the matmul of the reference's design sketch"""
+    M = N = K = 1024
+    h = F.create_session()
+    kernel = h.tiled_gemm("matmul", M, N, K, "fp32", tile=(128, 128, 32), threads=256)
+    assert h.module.verify()
+    A = make_operand(O.F32, M, K, seed=0, tensor=0, kind="uniform")
+    B = make_operand(O.F32, K, N, seed=0, tensor=1, kind="uniform")
+    got = _run(kernel, A, B, M, N, np.float32)
+    r = O.compare(O.F32, got, O.gemm_f64(O.F32, A, B))
+    assert r["nonfinite"] == 0 and r["max_rel"] <= 1e-4 and r["fro_rel"] <= 1e-4, r
+    # the naive definition agrees on a window of rows
+    ref_naive = O.gemm_naive(O.F32, np.ascontiguousarray(A[:16]), B)
+    assert O.compare(O.F32, np.ascontiguousarray(got[:16]), ref_naive)["max_rel"] <= 1e-4
+
+
+@pytest.mark.parametrize("dtype,odt,np_out,trans_b", [("fp16", O.F16, np.uint16, False), ("bf16", O.BF16, np.uint16, True)])
+def test_sixteen_bit_gemm_through_the_builder(hip, dtype, odt, np_out, trans_b):
+    M, N, K = 512, 768, 256
+    h = F.create_session()
+    kernel = h.tiled_gemm("g", M, N, K, dtype, tile=(256, 256, 64), trans_b=trans_b)
+    A = make_operand(odt, M, K, seed=21, tensor=0, scale=0.25)
+    B = make_operand(odt, *((N, K) if trans_b else (K, N)), seed=21, tensor=1, scale=0.25)
+    got = _run(kernel, A, B, M, N, np_out)
+    r = O.compare(odt, got, O.gemm_f64(odt, A, B, False, trans_b))
+    assert r["nonfinite"] == 0 and r["max_rel"] <= 1e-2 and r["fro_rel"] <= 1e-2, r
+
+
+def test_int8_with_dequant_epilogue_through_the_builder(hip):
+    import torch
+    M, N, K = 512, 512, 512
+    h = F.create_session()
+    kernel = h.tiled_gemm("w8a8", M, N, K, "int8", out_dtype="fp16", tile=(256, 256, 128))
+    A = make_operand(O.I8, M, K, seed=3, tensor=0)
+    B = make_operand(O.I8, K, N, seed=3, tensor=1)
+    sA, sB = O.uniform(M, 3, 2, 0.001, 0.02), O.uniform(N, 3, 3, 0.001, 0.02)
+    dsA, dsB = to_dev(sA), to_dev(sB)
+    got = _run(kernel, A, B, M, N, np.uint16, epilogue="row_col_scale", scale_a=dsA.data_ptr(), scale_b=dsB.data_ptr())
+    assert np.array_equal(got, O.epilogue_rowcol_f16(O.gemm_i32(A, B), sA, sB))
+    del torch
