@@ -18,6 +18,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "i8": 5033.2, "e4m3": 5033.2, "f32": 157.3}
+# L2-miss bytes of one fp16 4096^3 launch from rocprofv3 counters: FETCH_SIZE 98 358.6 KiB x 2.00 (the factor a 1 GiB
+# copy shows for this counter) + WRITE_SIZE 32 768 KiB x 1.00; see profiles/gemm_f16_nn_4096_and_i8_4096_bench.md
+TRAFFIC_BYTES_F16_4096 = int((98358.6 * 2.0 + 32768.0) * 1024)
 
 
 def gpu_time_gemm(R, torch, desc, ptrs, steps, warmup):
@@ -61,6 +64,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-mib", type=int, default=0,
+                    help="also run 3 plain device copies of this many MiB first: a kernel of known traffic to scale profiler byte counters by")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: the GEMM path has no multi-GPU leg (run with --gpus 1)")
@@ -71,6 +76,13 @@ def main():
     R.lib()
     assert torch.cuda.is_available(), "bench.py needs an MI355X"
     dev = torch.device("cuda:0")
+    if a.copy_mib:
+        src = torch.empty(a.copy_mib << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     M = N = K = 4096
     g = torch.Generator(device=dev)
     g.manual_seed(1)
@@ -105,7 +117,7 @@ def main():
                    "kernel": R.kernel_names()[plan.kernel_id], "grid": [plan.grid_x, plan.grid_y],
                    "lds_bytes": plan.lds_bytes},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS["f16"], 4), "traffic": None,
+                     "frac": round(achieved / PEAK_TFLOPS["f16"], 4), "traffic": TRAFFIC_BYTES_F16_4096, "traffic_unit": "bytes per launch",
                      "kernel_ms": round(kern_ms, 5)},
         "int8_4096": {"value": round(i8_tops, 2), "unit": "TOPS", "peak": PEAK_TFLOPS["i8"],
                       "frac": round(i8_tops / PEAK_TFLOPS["i8"], 4), "kernel_ms": round(i8_ms, 5),
