@@ -80,11 +80,29 @@ def build_ffi(verbose=True):
     return out
 
 
+def build_tools(verbose=True):
+    """the hardware probe behind the LDS cost model (frisk_amd/csrc/tools/lds_probe.hip) -> lib/lds_probe"""
+    out = os.path.join(LIBDIR, "lds_probe")
+    os.makedirs(LIBDIR, exist_ok=True)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-Wno-unused-value", os.path.join(CSRC, "tools", "lds_probe.hip"), "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building lds_probe failed:\n" + r.stderr)
+    if verbose:
+        print("built", out)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--if-missing", action="store_true")
     ap.add_argument("-j", type=int, default=None)
+    ap.add_argument("--tools", action="store_true", help="build only the hardware probe")
     a = ap.parse_args()
+    if a.tools:
+        build_tools()
+        return
     if a.if_missing and os.path.exists(LIB):
         print("present", LIB)
         return
