@@ -114,9 +114,6 @@ static int validate(const frisk_gemm_desc* d) {
   if (d->lda < std::max<int64_t>(1, a_cols)) return fail(FRISK_ERR_SHAPE, "lda=%lld smaller than the stored row length %lld", (long long)d->lda, (long long)a_cols);
   if (d->ldb < std::max<int64_t>(1, b_cols)) return fail(FRISK_ERR_SHAPE, "ldb=%lld smaller than the stored row length %lld", (long long)d->ldb, (long long)b_cols);
   if (d->ldc < std::max<int64_t>(1, d->N)) return fail(FRISK_ERR_SHAPE, "ldc=%lld smaller than N=%lld", (long long)d->ldc, (long long)d->N);
-  const int es = elem_size(ab), os = elem_size(out);
-  if ((d->lda * es) % 16 || (d->ldb * es) % 16) return fail(FRISK_ERR_ALIGNMENT, "rows of A and B must start on 16-byte boundaries (lda, ldb in bytes multiples of 16)");
-  if ((d->ldc * os) % 16) return fail(FRISK_ERR_ALIGNMENT, "rows of C must start on 16-byte boundaries");
   return FRISK_OK;
 }
 
@@ -139,7 +136,7 @@ static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, in
   (void)nw;
 }
 
-static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_model) {
+static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_model, bool force_guard = false) {
   int st = validate(d);
   if (st != FRISK_OK) return st;
   if (!plan) return fail(FRISK_ERR_NULL, "plan is null");
@@ -152,6 +149,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   if (d->epilogue == FRISK_EPI_TENSOR_SCALE) plan->bytes += 8.0;
   plan->split_k = 1;
 
+  const bool rows_aligned = (d->lda * es) % 16 == 0 && (d->ldb * es) % 16 == 0 && (d->ldc * os) % 16 == 0;
   const auto& ks = kernels();
   int best = -1;
   int64_t best_tiles = 0;
@@ -166,13 +164,16 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
     if (d->waves_m && d->waves_m != k->wm) continue;
     if (d->waves_n && d->waves_n != k->wn) continue;
     if (d->stages && d->stages != k->stages) continue;
-    if (d->M % k->bm || d->N % k->bn || d->K % k->bk) continue;
-    int64_t tiles = (d->M / k->bm) * (d->N / k->bn);
+    // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
+    if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
+    if (k->guard && best >= 0 && !ks[best]->guard) continue;  // never prefer a guarded kernel over a fast one that fits
+    int64_t tiles = ((d->M + k->bm - 1) / k->bm) * ((d->N + k->bn - 1) / k->bn);
     // largest tile that still gives every CU a work-group; otherwise the most work-groups
     bool better;
     if (best < 0) better = true;
     else {
       const KernelEntry* b = ks[best];
+      if (b->guard && !k->guard) { best = (int)i; best_tiles = tiles; continue; }
       bool fills = tiles >= 256, bfills = best_tiles >= 256;
       if (fills != bfills) better = fills;
       else if (fills && (int64_t)k->bm * k->bn != (int64_t)b->bm * b->bn) better = (int64_t)k->bm * k->bn > (int64_t)b->bm * b->bn;
@@ -200,8 +201,9 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   plan->mfma_m = 32; plan->mfma_n = 32; plan->mfma_k = mfma_k(d->dtype_ab);
   plan->lds_bytes = k->lds_bytes;
   plan->stages = k->stages;
-  plan->grid_x = (int)(d->N / k->bn);
-  plan->grid_y = (int)(d->M / k->bm);
+  plan->grid_x = (int)((d->N + k->bn - 1) / k->bn);
+  plan->grid_y = (int)((d->M + k->bm - 1) / k->bm);
+  plan->guarded = k->guard;
   plan->xcd_remap = ((int64_t)plan->grid_x * plan->grid_y) % 8 == 0;
   fill_layout(&plan->lds_a, !d->transA, es, frag_bytes(d->dtype_ab), k->bm, k->bk, k->wm * k->wn, with_model);
   fill_layout(&plan->lds_b, d->transB != 0, es, frag_bytes(d->dtype_ab), k->bn, k->bk, k->wm * k->wn, with_model);
@@ -254,12 +256,18 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
   if (desc->M == 0 || desc->N == 0) return FRISK_OK;
   if (!A || !B || !C) return fail(FRISK_ERR_NULL, "A, B and C must be device pointers");
   if (desc->epilogue != FRISK_EPI_NONE && (!scaleA || !scaleB)) return fail(FRISK_ERR_EPILOGUE, "epilogue %d needs scaleA and scaleB", desc->epilogue);
-  if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) return fail(FRISK_ERR_ALIGNMENT, "A, B and C must be 16-byte aligned");
-  if (desc->epilogue == FRISK_EPI_ROW_COL_SCALE && ((uintptr_t)scaleB & 15)) return fail(FRISK_ERR_ALIGNMENT, "scaleB must be 16-byte aligned");
+  const uintptr_t es = (uintptr_t)elem_size(desc->dtype_ab), os = (uintptr_t)elem_size(desc->dtype_out);
+  if (((uintptr_t)A | (uintptr_t)B) & (es - 1) || (uintptr_t)C & (os - 1) || (((uintptr_t)scaleA | (uintptr_t)scaleB) & 3))
+    return fail(FRISK_ERR_ALIGNMENT, "pointers must be aligned to their element size");
+  const bool ptrs16 = ((((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) == 0) &&
+                      !(desc->epilogue == FRISK_EPI_ROW_COL_SCALE && ((uintptr_t)scaleB & 15));
+  if (!ptrs16 && !plan.guarded) {  // the fast kernels move 16-byte chunks: fall back to the guarded kernel
+    st = make_plan(desc, &plan, false, true);
+    if (st != FRISK_OK) return st;
+  }
   if (plan.workspace_bytes > 0 && (!workspace || workspace_bytes < plan.workspace_bytes))
     return fail(FRISK_ERR_WORKSPACE, "needs %zu bytes of workspace", plan.workspace_bytes);
   if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
-  if (desc->K == 0) return fail(FRISK_ERR_SHAPE, "K = 0 is not launched; fill C instead");
 
   GemmParams p;
   p.A = A; p.B = B; p.C = C; p.scaleA = scaleA; p.scaleB = scaleB;

@@ -25,6 +25,7 @@ struct KernelEntry {
   int dtype;  // frisk_dtype of A and B
   int transA, transB;
   int bm, bn, bk, wm, wn, stages;
+  int guard;  // 1: handles any shape / leading dimension (slower staging)
   int lds_bytes;
   hipError_t (*launch)(const GemmParams&, hipStream_t);
 };

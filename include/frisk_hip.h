@@ -60,7 +60,7 @@ typedef enum frisk_status {
   FRISK_ERR_EPILOGUE = 7,    /* epilogue needs scales that were not given             */
   FRISK_ERR_WORKSPACE = 8,   /* workspace missing or too small                        */
   FRISK_ERR_DEVICE = 9,      /* no gfx950 device / HIP runtime error                  */
-  FRISK_ERR_ALIGNMENT = 10   /* a pointer or leading dimension breaks 16-byte alignment */
+  FRISK_ERR_ALIGNMENT = 10   /* a pointer is not aligned to its element size */
 } frisk_status;
 
 /*
@@ -72,7 +72,9 @@ typedef enum frisk_status {
  * Supported (dtype_ab -> dtype_acc -> dtype_out):
  *   F32->F32->F32, F16->F32->{F16,F32}, BF16->F32->{BF16,F32},
  *   I8->I32->{I32, F16 with ROW_COL_SCALE}, E4M3->F32->{BF16,F32} (NONE or TENSOR_SCALE)
- * tile_* and waves_* = 0 let the planner choose.
+ * tile_* and waves_* = 0 let the planner choose.  Shapes that are whole tiles with 16-byte aligned rows and
+ * pointers run the fast kernels; anything else (ragged M, N, K, odd leading dimensions, K = 0) runs a
+ * bounds-checked kernel with the same arithmetic.
  */
 typedef struct frisk_gemm_desc {
   int32_t abi_version; /* FRISK_HIP_ABI_VERSION */
@@ -111,6 +113,7 @@ typedef struct frisk_gemm_plan {
   int32_t grid_x, grid_y;            /* work-group grid (tiles along N, tiles along M) */
   int32_t split_k;                   /* >1: partial sums go through the workspace */
   int32_t xcd_remap;                 /* 1: work-group ids are remapped so each XCD owns a compact block of tiles */
+  int32_t guarded;                   /* 1: the bounds-checked kernel runs (ragged shape, unaligned rows or pointers) */
   frisk_lds_layout lds_a, lds_b;
   size_t workspace_bytes;
   double flops;                      /* 2.M.N.K */

@@ -32,24 +32,41 @@ def from_dev(t, np_dtype, shape):
 
 
 def run_gemm(R, dtype, A, B, transA, transB, dtype_out, M, N, K, epilogue=0, sA=None, sB=None, C_init=None,
-             clear_accum=True, tile=(0, 0, 0), waves=(0, 0)):
-    """launch through the C ABI; returns the output as a numpy array in storage type"""
+             clear_accum=True, tile=(0, 0, 0), waves=(0, 0), pad=0, shift=0):
+    """launch through the C ABI; returns the output as a numpy array in storage type.
+    pad: extra elements at the end of every stored row of A, B and C (odd leading dimensions);
+    shift: the operands start `shift` elements into their allocations (pointers only element-aligned)."""
     import torch
-    dA, dB = to_dev(A), to_dev(B)
     out_np = O.NP_STORAGE[dtype_out]
-    if C_init is None:
-        dC = torch.full((M * N * np.dtype(out_np).itemsize,), 0xFF, dtype=torch.uint8, device="cuda")
-    else:
-        dC = to_dev(C_init)
+
+    def padded(x):
+        if pad == 0 and shift == 0:
+            return np.ascontiguousarray(x), x.shape[1]
+        buf = np.zeros(shift + x.shape[0] * (x.shape[1] + pad), dtype=x.dtype)
+        buf[shift:].reshape(x.shape[0], x.shape[1] + pad)[:, :x.shape[1]] = x
+        return buf, x.shape[1] + pad
+
+    hA, lda = padded(A)
+    hB, ldb = padded(B)
+    C0 = C_init if C_init is not None else np.full((M, N), 0xFF, dtype=np.uint8).repeat(np.dtype(out_np).itemsize, axis=1).view(out_np)
+    hC, ldc = padded(np.ascontiguousarray(C0).view(out_np).reshape(M, N))
+    dA, dB, dC = to_dev(hA), to_dev(hB), to_dev(hC)
+    es, osz = hA.dtype.itemsize, np.dtype(out_np).itemsize
     dsA = to_dev(np.asarray(sA, dtype=np.float32)) if sA is not None else None
     dsB = to_dev(np.asarray(sB, dtype=np.float32)) if sB is not None else None
     desc = R.make_desc(dtype, M, N, K, dtype_out=dtype_out, transA=transA, transB=transB, clear_accum=clear_accum,
-                       epilogue=epilogue, tile=tile, waves=waves)
+                       epilogue=epilogue, tile=tile, waves=waves, lda=lda, ldb=ldb, ldc=ldc)
     stream = torch.cuda.current_stream().cuda_stream
-    R.gemm(desc, dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), dsA.data_ptr() if dsA is not None else None,
-           dsB.data_ptr() if dsB is not None else None, None, 0, stream)
+    R.gemm(desc, dA.data_ptr() + shift * es, dB.data_ptr() + shift * es, dC.data_ptr() + shift * osz,
+           dsA.data_ptr() if dsA is not None else None, dsB.data_ptr() if dsB is not None else None, None, 0, stream)
     torch.cuda.synchronize()
-    return from_dev(dC, out_np, (M, N))
+    full = dC.cpu().numpy().view(out_np)
+    if M == 0 or N == 0:
+        return np.zeros((M, N), dtype=out_np)
+    got = full[shift:].reshape(M, ldc)
+    if pad:
+        assert np.all(got[:, N:] == 0), "the kernel wrote into the padding of C"
+    return np.ascontiguousarray(got[:, :N])
 
 
 def stored_shapes(M, N, K, transA, transB):

@@ -186,3 +186,66 @@ def test_config_fp8_8192(hip):
     ref = O.gemm_f64(O.E4M3, np.ascontiguousarray(A[rows]), B, False, True)
     r = check(O.E4M3, O.BF16, np.ascontiguousarray(got[rows]), O.epilogue_tensor(ref, sA, sB))
     note(f"fp8 8192^3 NT ({len(rows)} rows): {r}")
+
+
+# ------------------------------------------------------------------ ragged shapes, odd leading dimensions, K = 0
+RAGGED = [(1, 1, 1), (100, 75, 40), (257, 129, 65), (33, 500, 130), (128, 128, 1)]
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.I8, O.E4M3, O.F32])
+@pytest.mark.parametrize("transA,transB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_ragged_shapes_run_the_guarded_kernel(hip, dtype, transA, transB):
+    for (M, N, K) in RAGGED:
+        note(f"case ragged {NAMES[dtype]} tA={transA} tB={transB} M={M} N={N} K={K}")
+        sa, sb = stored_shapes(M, N, K, transA, transB)
+        A = make_operand(dtype, *sa, seed=31, tensor=0, scale=0.5)
+        B = make_operand(dtype, *sb, seed=31, tensor=1, scale=0.5)
+        out_dt = DEFAULT_OUT[dtype]
+        got = run_gemm(hip, dtype, A, B, transA, transB, out_dt, M, N, K)
+        if dtype == O.I8:
+            assert np.array_equal(got, O.gemm_i32(A, B, transA, transB))
+        else:
+            check(dtype, out_dt, got, O.gemm_f64(dtype, A, B, transA, transB))
+
+
+def test_odd_leading_dimensions_and_unaligned_pointers(hip):
+    """rows padded by 3 elements and buffers entered one element in: no 16-byte alignment anywhere"""
+    M, N, K = 256, 256, 128
+    A = make_operand(O.F16, M, K, seed=32, tensor=0, scale=0.5)
+    B = make_operand(O.F16, K, N, seed=32, tensor=1, scale=0.5)
+    ref = O.gemm_f64(O.F16, A, B)
+    for pad, shift in ((3, 0), (0, 1), (5, 3)):
+        got = run_gemm(hip, O.F16, A, B, 0, 0, O.F16, M, N, K, pad=pad, shift=shift)
+        check(O.F16, O.F16, got, ref)
+    # the aligned call of the same problem takes the fast kernel and agrees bit for bit with the guarded one
+    fast = run_gemm(hip, O.F16, A, B, 0, 0, O.F16, M, N, K)
+    slow = run_gemm(hip, O.F16, A, B, 0, 0, O.F16, M, N, K, pad=8, shift=0)  # rows still 16-byte aligned: fast kernel
+    assert np.array_equal(fast, slow)
+    assert np.array_equal(fast, run_gemm(hip, O.F16, A, B, 0, 0, O.F16, M, N, K, pad=3))
+
+
+def test_ragged_int8_dequant_and_accumulate(hip):
+    M, N, K = 70, 90, 200
+    A = make_operand(O.I8, M, K, seed=33, tensor=0)
+    B = make_operand(O.I8, K, N, seed=33, tensor=1)
+    sA, sB = O.uniform(M, 33, 2, 0.001, 0.02), O.uniform(N, 33, 3, 0.001, 0.02)
+    got = run_gemm(hip, O.I8, A, B, 0, 0, O.F16, M, N, K, epilogue=hip.EPI_ROW_COL_SCALE, sA=sA, sB=sB)
+    assert np.array_equal(got, O.epilogue_rowcol_f16(O.gemm_i32(A, B), sA, sB))
+    C0 = (np.arange(M * N, dtype=np.int64).reshape(M, N) % 77 - 30).astype(np.int32)
+    goti = run_gemm(hip, O.I8, A, B, 0, 0, O.I32, M, N, K, C_init=C0, clear_accum=False)
+    assert np.array_equal(goti, O.gemm_i32(A, B) + C0)
+
+
+def test_empty_problems(hip):
+    """K = 0: C = 0 (or C unchanged when accumulating); M = 0 or N = 0: nothing is launched"""
+    M, N = 64, 48
+    A = np.zeros((M, 0), dtype=np.uint16)
+    B = np.zeros((0, N), dtype=np.uint16)
+    got = run_gemm(hip, O.F16, np.zeros((M, 1), np.uint16), np.zeros((1, N), np.uint16), 0, 0, O.F32, M, N, 0)
+    assert np.all(got == 0.0)
+    C0 = O.uniform(M * N, 5, 0, -1.0, 1.0).reshape(M, N)
+    got = run_gemm(hip, O.F16, np.zeros((M, 1), np.uint16), np.zeros((1, N), np.uint16), 0, 0, O.F32, M, N, 0, C_init=C0, clear_accum=False)
+    assert np.array_equal(got, C0)
+    d = hip.make_desc(hip.F16, 0, 128, 64)
+    hip.gemm(d, None, None, None)
+    del A, B
