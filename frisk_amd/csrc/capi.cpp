@@ -136,7 +136,7 @@ static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, in
   (void)nw;
 }
 
-static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_model, bool force_guard = false) {
+static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_model, bool force_guard = false, bool no_split = false) {
   int st = validate(d);
   if (st != FRISK_OK) return st;
   if (!plan) return fail(FRISK_ERR_NULL, "plan is null");
@@ -197,7 +197,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   if (k->lds_bytes > 160 * 1024) return fail(FRISK_ERR_LDS, "tile needs %d bytes of LDS", k->lds_bytes);
   plan->kernel_id = best;
   plan->tile_m = k->bm; plan->tile_n = k->bn; plan->tile_k = k->bk;
-  plan->waves_m = k->wm; plan->waves_n = k->wn; plan->threads = k->wm * k->wn * 64;
+  plan->waves_m = k->wm; plan->waves_n = k->wn; plan->waves_k = k->wk; plan->threads = k->wm * k->wn * k->wk * 64;
   plan->mfma_m = 32; plan->mfma_n = 32; plan->mfma_k = mfma_k(d->dtype_ab);
   plan->lds_bytes = k->lds_bytes;
   plan->stages = k->stages;
@@ -205,9 +205,26 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   plan->grid_y = (int)((d->M + k->bm - 1) / k->bm);
   plan->guarded = k->guard;
   plan->xcd_remap = ((int64_t)plan->grid_x * plan->grid_y) % 8 == 0;
-  fill_layout(&plan->lds_a, !d->transA, es, frag_bytes(d->dtype_ab), k->bm, k->bk, k->wm * k->wn, with_model);
-  fill_layout(&plan->lds_b, d->transB != 0, es, frag_bytes(d->dtype_ab), k->bn, k->bk, k->wm * k->wn, with_model);
+  fill_layout(&plan->lds_a, !d->transA, es, frag_bytes(d->dtype_ab), k->bm, k->bk, k->wm * k->wn * k->wk, with_model);
+  fill_layout(&plan->lds_b, d->transB != 0, es, frag_bytes(d->dtype_ab), k->bn, k->bk, k->wm * k->wn * k->wk, with_model);
   plan->workspace_bytes = 0;
+  // Split K over the grid's y dimension when the tile grid alone leaves most CUs idle (skinny problems are
+  // bound by streaming the large operand, which needs many work-groups in flight).  Slices hold whole K tiles.
+  const int64_t kt = d->K / k->bk, tiles = (int64_t)plan->grid_x * plan->grid_y;
+  int split = 1;
+  if (k->splitk && !no_split && d->K % k->bk == 0) {
+    if (d->split_k > 1) {
+      if (kt % d->split_k) return fail(FRISK_ERR_TILE, "split_k=%d does not divide the %lld K tiles", d->split_k, (long long)kt);
+      split = d->split_k;
+    } else if (d->split_k == 0 && tiles < 256) {  // up to one work-group per CU, at least 4 K tiles per slice
+      for (int c = 2; c <= 64; c *= 2)
+        if (kt % c == 0 && kt / c >= 4 && tiles * c <= 256) split = c;
+    }
+  } else if (d->split_k > 1 && !no_split) {
+    return fail(FRISK_ERR_TILE, "split_k=%d: the chosen kernel %s has no split-K path", d->split_k, k->name);
+  }
+  plan->split_k = split;
+  if (split > 1) plan->workspace_bytes = (size_t)split * (size_t)d->M * (size_t)d->N * 4;
   return FRISK_OK;
 }
 
@@ -265,8 +282,13 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
     st = make_plan(desc, &plan, false, true);
     if (st != FRISK_OK) return st;
   }
-  if (plan.workspace_bytes > 0 && (!workspace || workspace_bytes < plan.workspace_bytes))
-    return fail(FRISK_ERR_WORKSPACE, "needs %zu bytes of workspace", plan.workspace_bytes);
+  if (plan.workspace_bytes > 0 && (!workspace || workspace_bytes < plan.workspace_bytes)) {
+    // an explicit split_k needs its workspace; the planner's own choice degrades to a single pass without one
+    if (desc->split_k > 1) return fail(FRISK_ERR_WORKSPACE, "split_k=%d needs %zu bytes of workspace", desc->split_k, plan.workspace_bytes);
+    st = make_plan(desc, &plan, false, plan.guarded != 0, true);
+    if (st != FRISK_OK) return st;
+  }
+  if (plan.split_k > 1 && ((uintptr_t)workspace & 15)) return fail(FRISK_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
   if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
 
   GemmParams p;
@@ -277,8 +299,16 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
   p.group_m = group_rows(p.tiles_m, p.tiles_n);
   p.xcd_remap = plan.xcd_remap;
   p.epilogue = desc->epilogue; p.dtype_out = desc->dtype_out; p.accumulate = desc->clear_accum ? 0 : 1;
-  hipError_t e = kernels()[plan.kernel_id]->launch(p, (hipStream_t)stream);
-  if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "launch of %s failed: %s", kernels()[plan.kernel_id]->name, hipGetErrorString(e));
+  const KernelEntry* k = kernels()[plan.kernel_id];
+  p.split_k = plan.split_k;
+  p.kt_per_slice = (int)((desc->K + k->bk - 1) / k->bk) / plan.split_k;
+  p.partial = plan.split_k > 1 ? workspace : nullptr;
+  hipError_t e = k->launch(p, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "launch of %s failed: %s", k->name, hipGetErrorString(e));
+  if (plan.split_k > 1) {
+    e = launch_splitk_reduce(p, desc->dtype_acc == FRISK_I32, (hipStream_t)stream);
+    if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "launch of the split-K reduction failed: %s", hipGetErrorString(e));
+  }
   return FRISK_OK;
 }
 

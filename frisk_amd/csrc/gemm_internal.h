@@ -17,6 +17,10 @@ struct GemmParams {
   int tiles_m, tiles_n;
   int group_m, xcd_remap;
   int epilogue, dtype_out, accumulate;
+  // K range of a work-group: blockIdx.y walks `split_k` slices of `kt_per_slice` K tiles each.  With more than one
+  // slice the kernel writes raw 32-bit accumulators to partial[slice][M][N] and a second kernel sums the slices.
+  int split_k, kt_per_slice;
+  void* partial;
 };
 
 // One compiled kernel variant.
@@ -25,10 +29,15 @@ struct KernelEntry {
   int dtype;  // frisk_dtype of A and B
   int transA, transB;
   int bm, bn, bk, wm, wn, stages;
+  int wk;  // waves splitting the K steps of a tile (1 = none)
   int guard;  // 1: handles any shape / leading dimension (slower staging)
+  int splitk;  // 1: compiled with the split-K store path
   int lds_bytes;
   hipError_t (*launch)(const GemmParams&, hipStream_t);
 };
+
+// sums the split-K slices and applies the epilogue (splitk_reduce.hip)
+hipError_t launch_splitk_reduce(const GemmParams& p, int acc_is_int, hipStream_t stream);
 
 // defined in kernels_*.hip
 extern const KernelEntry kKernelsF16[];

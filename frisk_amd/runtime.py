@@ -29,7 +29,7 @@ class GemmDesc(ctypes.Structure):
                 ("dtype_out", ctypes.c_int32), ("M", ctypes.c_int64), ("N", ctypes.c_int64), ("K", ctypes.c_int64),
                 ("lda", ctypes.c_int64), ("ldb", ctypes.c_int64), ("ldc", ctypes.c_int64),
                 ("transA", ctypes.c_uint8), ("transB", ctypes.c_uint8), ("clear_accum", ctypes.c_uint8),
-                ("reserved0", ctypes.c_uint8), ("epilogue", ctypes.c_int32), ("policy", ctypes.c_int32),
+                ("split_k", ctypes.c_uint8), ("epilogue", ctypes.c_int32), ("policy", ctypes.c_int32),
                 ("tile_m", ctypes.c_int32), ("tile_n", ctypes.c_int32), ("tile_k", ctypes.c_int32),
                 ("waves_m", ctypes.c_int32), ("waves_n", ctypes.c_int32), ("stages", ctypes.c_int32)]
 
@@ -43,11 +43,14 @@ class LdsLayout(ctypes.Structure):
 class GemmPlan(ctypes.Structure):
     _fields_ = [("kernel_id", ctypes.c_int32), ("tile_m", ctypes.c_int32), ("tile_n", ctypes.c_int32),
                 ("tile_k", ctypes.c_int32), ("waves_m", ctypes.c_int32), ("waves_n", ctypes.c_int32),
-                ("threads", ctypes.c_int32), ("mfma_m", ctypes.c_int32), ("mfma_n", ctypes.c_int32),
+                ("threads", ctypes.c_int32), ("waves_k", ctypes.c_int32), ("mfma_m", ctypes.c_int32), ("mfma_n", ctypes.c_int32),
                 ("mfma_k", ctypes.c_int32), ("stages", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
                 ("grid_x", ctypes.c_int32), ("grid_y", ctypes.c_int32), ("split_k", ctypes.c_int32),
                 ("xcd_remap", ctypes.c_int32), ("guarded", ctypes.c_int32), ("lds_a", LdsLayout), ("lds_b", LdsLayout),
                 ("workspace_bytes", ctypes.c_size_t), ("flops", ctypes.c_double), ("bytes", ctypes.c_double)]
+
+
+globals().update({name: code for code, name in STATUS_NAMES.items()})  # OK, ERR_NULL, ... as module constants
 
 
 class FriskHipError(RuntimeError):
@@ -101,7 +104,7 @@ def _check(status):
 
 
 def make_desc(dtype_ab, M, N, K, dtype_out=None, transA=False, transB=False, lda=None, ldb=None, ldc=None,
-              clear_accum=True, epilogue=EPI_NONE, policy=POLICY_SQUARE, tile=(0, 0, 0), waves=(0, 0), stages=0):
+              clear_accum=True, epilogue=EPI_NONE, policy=POLICY_SQUARE, tile=(0, 0, 0), waves=(0, 0), stages=0, split_k=0):
     d = GemmDesc()
     d.abi_version = ABI_VERSION
     d.dtype_ab = dtype_ab
@@ -116,6 +119,7 @@ def make_desc(dtype_ab, M, N, K, dtype_out=None, transA=False, transB=False, lda
     d.tile_m, d.tile_n, d.tile_k = tile
     d.waves_m, d.waves_n = waves
     d.stages = stages
+    d.split_k = split_k
     return d
 
 
@@ -123,6 +127,11 @@ def plan(desc):
     p = GemmPlan()
     _check(lib().frisk_hip_plan(ctypes.byref(desc), ctypes.byref(p)))
     return p
+
+
+def workspace_bytes(desc):
+    """device workspace a launch of `desc` wants (split-K partial sums); 0 for most shapes"""
+    return int(lib().frisk_hip_workspace_bytes(ctypes.byref(desc)))
 
 
 def gemm(desc, A_ptr, B_ptr, C_ptr, scaleA_ptr=None, scaleB_ptr=None, workspace_ptr=None, workspace_bytes=0, stream=None):

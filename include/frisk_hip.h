@@ -81,7 +81,9 @@ typedef struct frisk_gemm_desc {
   int32_t dtype_ab, dtype_acc, dtype_out;
   int64_t M, N, K;
   int64_t lda, ldb, ldc;
-  uint8_t transA, transB, clear_accum, reserved0;
+  uint8_t transA, transB, clear_accum;
+  uint8_t split_k; /* slices of K computed by separate work-groups and summed through the workspace:
+                      0 = planner's choice (splits only skinny problems, and only if a workspace is passed), 1 = never */
   int32_t epilogue;
   int32_t policy;                 /* frisk_wave_policy */
   int32_t tile_m, tile_n, tile_k; /* block tile = the M,N,K attrs of the tile-level frisk.gemm */
@@ -107,6 +109,7 @@ typedef struct frisk_gemm_plan {
   int32_t kernel_id;                 /* index into the compiled kernel table, -1 if none */
   int32_t tile_m, tile_n, tile_k;
   int32_t waves_m, waves_n, threads; /* result of the wave partition (reference: computeWarpPartition, FriskOps.cpp:825-888) */
+  int32_t waves_k;                   /* >1: that many waves split the K steps of each tile (threads = waves_m*waves_n*waves_k*64) */
   int32_t mfma_m, mfma_n, mfma_k;    /* MFMA atom */
   int32_t stages;
   int32_t lds_bytes;                 /* total, <= 163840 */
@@ -128,7 +131,8 @@ const char* frisk_hip_last_error(void);
 /* Pure host: validate the descriptor and fill the plan.  Needs no GPU. */
 int frisk_hip_plan(const frisk_gemm_desc* desc, frisk_gemm_plan* plan);
 
-/* Pure host: bytes of device workspace `frisk_hip_gemm` needs for this descriptor (0 for most). */
+/* Pure host: bytes of device workspace `frisk_hip_gemm` wants for this descriptor: split_k * M * N * 4 when the
+ * plan splits K, else 0.  With split_k = 0 in the descriptor a launch without workspace still runs, unsplit. */
 size_t frisk_hip_workspace_bytes(const frisk_gemm_desc* desc);
 
 /* Launch on `stream` (a hipStream_t, may be NULL for the default stream).

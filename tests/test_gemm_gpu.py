@@ -249,3 +249,89 @@ def test_empty_problems(hip):
     d = hip.make_desc(hip.F16, 0, 128, 64)
     hip.gemm(d, None, None, None)
     del A, B
+
+
+# ------------------------------------------------------------------ skinny problems: 32-row tiles, K split over work-groups
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.I8, O.E4M3])
+@pytest.mark.parametrize("transB", [0, 1])
+def test_skinny_split_k(hip, dtype, transB):
+    """M = 32 and 64: a 32-row kernel runs (B stored [N][K]: 32x32 tile whose 4 waves split the K steps; B stored
+    [K][N]: 32x128 tile); every split factor gives the oracle's result (int8: the same bits)"""
+    for M in (32, 64):
+        N, K = 384, 32 * BK[dtype]
+        sa, sb = stored_shapes(M, N, K, 0, transB)
+        A = make_operand(dtype, *sa, seed=41, tensor=0, scale=0.5)
+        B = make_operand(dtype, *sb, seed=41, tensor=1, scale=0.5)
+        out_dt = DEFAULT_OUT[dtype]
+        ref = O.gemm_i32(A, B, 0, transB) if dtype == O.I8 else O.gemm_f64(dtype, A, B, 0, transB)
+        d = hip.make_desc(dtype, M, N, K, dtype_out=out_dt, transB=bool(transB))
+        p = hip.plan(d)
+        assert p.tile_m == 32 and p.split_k > 1 and p.workspace_bytes == p.split_k * M * N * 4, (p.tile_m, p.split_k, p.workspace_bytes)
+        for split in (0, 1, 2, 4, 8):
+            note(f"case skinny {NAMES[dtype]} tB={transB} M={M} N={N} K={K} split_k={split}")
+            got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, split_k=split)
+            if dtype == O.I8:
+                assert np.array_equal(got, ref)
+            else:
+                check(dtype, out_dt, got, ref)
+        # the planner's own split needs no workspace to be correct: without one the launch runs unsplit
+        got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, workspace=False)
+        if dtype == O.I8:
+            assert np.array_equal(got, ref)
+        else:
+            check(dtype, out_dt, got, ref)
+
+
+def test_split_k_epilogues_and_accumulate(hip):
+    M, N, K = 32, 256, 2048
+    A = make_operand(O.I8, M, K, seed=42, tensor=0)
+    B = make_operand(O.I8, K, N, seed=42, tensor=1)
+    sA, sB = O.uniform(M, 42, 2, 0.001, 0.02), O.uniform(N, 42, 3, 0.001, 0.02)
+    acc = O.gemm_i32(A, B)
+    got = run_gemm(hip, O.I8, A, B, 0, 0, O.F16, M, N, K, epilogue=hip.EPI_ROW_COL_SCALE, sA=sA, sB=sB, split_k=4)
+    assert np.array_equal(got, O.epilogue_rowcol_f16(acc, sA, sB))
+    C0 = (np.arange(M * N, dtype=np.int64).reshape(M, N) % 91 - 45).astype(np.int32)
+    goti = run_gemm(hip, O.I8, A, B, 0, 0, O.I32, M, N, K, C_init=C0, clear_accum=False, split_k=8)
+    assert np.array_equal(goti, acc + C0)
+    # fp16 with fp32 output, accumulating into C, ldc padded
+    Ah = make_operand(O.F16, M, K, seed=43, tensor=0, scale=0.5)
+    Bh = make_operand(O.F16, N, K, seed=43, tensor=1, scale=0.5)
+    C0f = O.uniform(M * N, 43, 2, -1.0, 1.0).reshape(M, N).astype(np.float32)
+    gotf = run_gemm(hip, O.F16, Ah, Bh, 0, 1, O.F32, M, N, K, C_init=C0f, clear_accum=False, split_k=4, pad=8)
+    check(O.F16, O.F32, gotf, O.gemm_f64(O.F16, Ah, Bh, False, True) + C0f.astype(np.float64))
+
+
+def test_split_k_status_codes(hip):
+    import torch
+    M, N, K = 32, 256, 2048
+    d = hip.make_desc(O.F16, M, N, K, split_k=3)
+    with pytest.raises(hip.FriskHipError) as e:
+        hip.plan(d)
+    assert e.value.status == hip.ERR_TILE
+    d = hip.make_desc(O.F16, M, N, K, split_k=4)
+    buf = torch.zeros(M * K + K * N + M * N, dtype=torch.float16, device="cuda")
+    with pytest.raises(hip.FriskHipError) as e:
+        hip.gemm(d, buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), None, None, None, 0, None)
+    assert e.value.status == hip.ERR_WORKSPACE
+    # a kernel without the split path refuses an explicit split
+    d = hip.make_desc(O.F16, 256, 256, 2048, transA=True, split_k=4)
+    with pytest.raises(hip.FriskHipError) as e:
+        hip.plan(d)
+    assert e.value.status == hip.ERR_TILE
+
+
+def test_config_fp8_skinny_decode(hip):
+    """M = 32, N = K = 8192, e4m3 with per-tensor scales, bf16 output: every row checked"""
+    M, N, K = 32, 8192, 8192
+    xa, xb = O.normal(M * K, 4, 0, 1.0), O.normal(N * K, 4, 1, 1.0)
+    sA, sB = np.float32(np.abs(xa).max() / 448.0), np.float32(np.abs(xb).max() / 448.0)
+    A = O.encode(O.E4M3, xa / sA).reshape(M, K)
+    B = O.encode(O.E4M3, xb / sB).reshape(N, K)
+    del xa, xb
+    d = hip.make_desc(O.E4M3, M, N, K, dtype_out=O.BF16, transB=True, epilogue=hip.EPI_TENSOR_SCALE)
+    p = hip.plan(d)
+    assert p.tile_m == 32 and p.grid_x * p.grid_y * p.split_k >= 256
+    got = run_gemm(hip, O.E4M3, A, B, 0, 1, O.BF16, M, N, K, epilogue=hip.EPI_TENSOR_SCALE, sA=[sA], sB=[sB])
+    ref = O.epilogue_tensor(O.gemm_f64(O.E4M3, A, B, False, True), sA, sB)
+    r = check(O.E4M3, O.BF16, got, ref)
+    note(f"fp8 skinny 32x8192x8192 NT split_k={p.split_k}: {r}")
