@@ -18,15 +18,35 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "i8": 5033.2, "e4m3": 5033.2, "f32": 157.3}
-# L2-miss bytes of one fp16 4096^3 launch from rocprofv3 counters: FETCH_SIZE 98 358.6 KiB x 2.00 (the factor a 1 GiB
-# copy shows for this counter) + WRITE_SIZE 32 768 KiB x 1.00; see profiles/gemm_f16_nn_4096_and_i8_4096_bench.md
-TRAFFIC_BYTES_F16_4096 = int((98358.6 * 2.0 + 32768.0) * 1024)
+# L2-miss bytes of one fp16 4096^3 launch from rocprofv3 counters: FETCH_SIZE 98 405.1 KiB x 2.00 (the factor a 1 GiB
+# copy shows for this counter) + WRITE_SIZE 32 768 KiB x 1.00; see profiles/bench_kernels_f16_4096_i8_4096_fp8_skinny.md
+TRAFFIC_BYTES_F16_4096 = int((98405.1 * 2.0 + 32768.0) * 1024)
+
+
+SETTLE_MS = 100.0
+
+
+def settle(torch, launch, stream):
+    """Untimed launches until SETTLE_MS of GPU time have passed.  After an idle period the part's power management
+    first overshoots and then takes about 50 ms of continuous load to reach its steady clocks (launch time goes
+    122 -> 145 -> 116 us over the first 400 launches of the fp16 4096^3 kernel; the vendor library shows the same
+    curve), so a short warm-up would time the transient, not the kernel."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    spent = 0.0
+    while spent < SETTLE_MS:
+        e0.record(stream)
+        for _ in range(50):
+            launch()
+        e1.record(stream)
+        e1.synchronize()
+        spent += e0.elapsed_time(e1)
 
 
 def gpu_time_gemm(R, torch, desc, ptrs, steps, warmup):
     """returns (wall seconds for `steps` launches, mean kernel ms from HIP events on the launch stream)"""
     stream = torch.cuda.current_stream()
     s = stream.cuda_stream
+    settle(torch, lambda: R.gemm(desc, *ptrs, None, 0, s), stream)
     for _ in range(warmup):
         R.gemm(desc, *ptrs, None, 0, s)
     torch.cuda.synchronize()
@@ -108,11 +128,41 @@ def main():
                              a.steps, a.warmup)
     i8_tops = flops / (i8_ms * 1e-3) / 1e12
 
+    # HBM-bound shape of the configuration list: fp8 e4m3 M=32, N=K=8192 (B stored [N][K]), per-tensor scales, bf16 out.
+    # B rotates over 6 buffers (384 MiB > the 256 MiB last-level cache) so every launch streams it from HBM.
+    Ms, Ns, Ks = 32, 8192, 8192
+    Af = torch.randn(Ms, Ks, device=dev, generator=g).to(torch.float8_e4m3fn)
+    Bf = [torch.randn(Ns, Ks, device=dev, generator=g).to(torch.float8_e4m3fn) for _ in range(6)]
+    Cf = torch.empty(Ms, Ns, device=dev, dtype=torch.bfloat16)
+    one = torch.ones(1, device=dev)
+    df = R.make_desc(R.E4M3, Ms, Ns, Ks, dtype_out=R.BF16, transB=True, epilogue=R.EPI_TENSOR_SCALE)
+    pf = R.plan(df)
+    ws_bytes = R.workspace_bytes(df)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream()
+
+    def skinny(n):
+        for i in range(n):
+            R.gemm(df, Af.data_ptr(), Bf[i % len(Bf)].data_ptr(), Cf.data_ptr(), one.data_ptr(), one.data_ptr(),
+                   ws.data_ptr() if ws_bytes else None, ws_bytes, stream.cuda_stream)
+    settle(torch, lambda: skinny(1), stream)
+    skinny(a.warmup)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    skinny(a.steps)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    sk_ms = e0.elapsed_time(e1) / a.steps
+    sk_bytes = Ms * Ks + Ns * Ks + 2 * Ms * Ns + 8
+    sk_gbs = sk_bytes / (sk_ms * 1e-3) / 1e9
+    del Bf
+
     line = {
         "metric": "GEMM TFLOP/s at 4096^3 fp16 (fp32 accumulate), 1 GPU",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(wall / a.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic", "settle_ms": SETTLE_MS,
         "config": {"workload": "fp16 GEMM M=N=K=4096 NN row-major, N(0,1)/sqrt(K) seed 1, fp32 accumulate, fp16 out",
                    "kernel": R.kernel_names()[plan.kernel_id], "grid": [plan.grid_x, plan.grid_y],
                    "lds_bytes": plan.lds_bytes},
@@ -122,6 +172,11 @@ def main():
         "int8_4096": {"value": round(i8_tops, 2), "unit": "TOPS", "peak": PEAK_TFLOPS["i8"],
                       "frac": round(i8_tops / PEAK_TFLOPS["i8"], 4), "kernel_ms": round(i8_ms, 5),
                       "workload": "W8A8 int8 4096^3 NN, int32 accumulate, per-row/per-column fp32 scales, fp16 out"},
+        "fp8_skinny_32x8192x8192": {"bound": "hbm", "achieved": round(sk_gbs, 1), "peak": 8000.0, "unit": "GB/s",
+                                    "frac": round(sk_gbs / 8000.0, 4), "kernel_ms": round(sk_ms, 5),
+                                    "kernel": R.kernel_names()[pf.kernel_id], "split_k": pf.split_k,
+                                    "workload": "fp8 e4m3 M=32 N=K=8192 NT, per-tensor scales, bf16 out; algorithmic bytes "
+                                                "|A|+|B|+|C|+scales per launch, B rotating over 6 buffers"},
     }
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(M, N, K)
