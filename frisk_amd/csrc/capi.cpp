@@ -163,7 +163,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
     if (d->tile_k && d->tile_k != k->bk) continue;
     if (d->waves_m && d->waves_m != k->wm) continue;
     if (d->waves_n && d->waves_n != k->wn) continue;
-    if (d->stages && d->stages != k->stages) continue;
+    if (d->stages && d->stages != k->stages_b) continue;  // the deeper ring names the variant
     // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
     if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
     if (k->guard && best >= 0 && !ks[best]->guard) continue;  // never prefer a guarded kernel over a fast one that fits
@@ -201,6 +201,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   plan->mfma_m = 32; plan->mfma_n = 32; plan->mfma_k = mfma_k(d->dtype_ab);
   plan->lds_bytes = k->lds_bytes;
   plan->stages = k->stages;
+  plan->stages_b = k->stages_b;
   plan->grid_x = (int)((d->N + k->bn - 1) / k->bn);
   plan->grid_y = (int)((d->M + k->bm - 1) / k->bm);
   plan->guarded = k->guard;

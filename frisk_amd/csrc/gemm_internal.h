@@ -28,7 +28,8 @@ struct KernelEntry {
   const char* name;
   int dtype;  // frisk_dtype of A and B
   int transA, transB;
-  int bm, bn, bk, wm, wn, stages;
+  int bm, bn, bk, wm, wn;
+  int stages, stages_b;  // LDS ring depth for A and for B (stages_b >= stages)
   int wk;  // waves splitting the K steps of a tile (1 = none)
   int guard;  // 1: handles any shape / leading dimension (slower staging)
   int splitk;  // 1: compiled with the split-K store path

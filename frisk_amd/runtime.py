@@ -44,7 +44,7 @@ class GemmPlan(ctypes.Structure):
     _fields_ = [("kernel_id", ctypes.c_int32), ("tile_m", ctypes.c_int32), ("tile_n", ctypes.c_int32),
                 ("tile_k", ctypes.c_int32), ("waves_m", ctypes.c_int32), ("waves_n", ctypes.c_int32),
                 ("threads", ctypes.c_int32), ("waves_k", ctypes.c_int32), ("mfma_m", ctypes.c_int32), ("mfma_n", ctypes.c_int32),
-                ("mfma_k", ctypes.c_int32), ("stages", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
+                ("mfma_k", ctypes.c_int32), ("stages", ctypes.c_int32), ("stages_b", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
                 ("grid_x", ctypes.c_int32), ("grid_y", ctypes.c_int32), ("split_k", ctypes.c_int32),
                 ("xcd_remap", ctypes.c_int32), ("guarded", ctypes.c_int32), ("lds_a", LdsLayout), ("lds_b", LdsLayout),
                 ("workspace_bytes", ctypes.c_size_t), ("flops", ctypes.c_double), ("bytes", ctypes.c_double)]

@@ -88,7 +88,7 @@ typedef struct frisk_gemm_desc {
   int32_t policy;                 /* frisk_wave_policy */
   int32_t tile_m, tile_n, tile_k; /* block tile = the M,N,K attrs of the tile-level frisk.gemm */
   int32_t waves_m, waves_n;       /* wave grid inside the work-group */
-  int32_t stages;                 /* LDS stages of the global->LDS pipeline, 0 = planner's choice */
+  int32_t stages;                 /* LDS stages of the global->LDS pipeline (of B when A and B differ), 0 = planner's choice */
 } frisk_gemm_desc;
 
 /* XOR swizzle of an LDS tile: 16-byte chunk index c of row r is stored at
@@ -111,7 +111,7 @@ typedef struct frisk_gemm_plan {
   int32_t waves_m, waves_n, threads; /* result of the wave partition (reference: computeWarpPartition, FriskOps.cpp:825-888) */
   int32_t waves_k;                   /* >1: that many waves split the K steps of each tile (threads = waves_m*waves_n*waves_k*64) */
   int32_t mfma_m, mfma_n, mfma_k;    /* MFMA atom */
-  int32_t stages;
+  int32_t stages, stages_b;          /* LDS ring depth for tiles of A and of B */
   int32_t lds_bytes;                 /* total, <= 163840 */
   int32_t grid_x, grid_y;            /* work-group grid (tiles along N, tiles along M) */
   int32_t split_k;                   /* >1: partial sums go through the workspace */

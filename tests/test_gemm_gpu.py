@@ -51,6 +51,26 @@ def test_layouts_small_shapes(hip, dtype, transA, transB, which):
         check(dtype, out_dt, got, O.gemm_f64(dtype, A, B, transA, transB))
 
 
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
+@pytest.mark.parametrize("transA,transB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_deeper_ring_for_b(hip, dtype, transA, transB):
+    """the variant with 2 LDS tiles of A and 3 of B: K of 1, 2, 3, 4 and 7 tiles walks every phase of its pipeline
+    (fewer tiles than stages, A-only tail, steady state) and must give the bits of the 2 + 2 variant"""
+    for ktiles in (1, 2, 3, 4, 7):
+        M, N, K = 256, 512, ktiles * 64
+        note(f"case deep-B {NAMES[dtype]} tA={transA} tB={transB} K={K}")
+        sa, sb = stored_shapes(M, N, K, transA, transB)
+        A = make_operand(dtype, *sa, seed=12, tensor=0, scale=0.5)
+        B = make_operand(dtype, *sb, seed=12, tensor=1, scale=0.5)
+        d = hip.make_desc(dtype, M, N, K, transA=bool(transA), transB=bool(transB), tile=(256, 256, 64), stages=3)
+        p = hip.plan(d)
+        assert (p.stages, p.stages_b, p.lds_bytes) == (2, 3, 160 * 1024)
+        got = run_gemm(hip, dtype, A, B, transA, transB, dtype, M, N, K, tile=(256, 256, 64), stages=3)
+        check(dtype, dtype, got, O.gemm_f64(dtype, A, B, transA, transB))
+        same = run_gemm(hip, dtype, A, B, transA, transB, dtype, M, N, K, tile=(256, 256, 64), stages=2)
+        assert np.array_equal(got, same)
+
+
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.E4M3, O.F32])
 def test_identity_is_exact(hip, dtype):
     """A = I  =>  C == B bit for bit (every product is exact, every sum has one non-zero term)"""
