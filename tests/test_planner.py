@@ -5,6 +5,7 @@ import json
 import os
 import re
 
+import numpy as np
 import pytest
 
 from frisk_amd import runtime as R
@@ -169,3 +170,30 @@ def test_gemm_rejects_bad_arguments_before_touching_the_device():
         R.gemm(d8, 0x1000, 0x2000, 0x3000)                      # scales missing
     assert e.value.status == 7
     R.gemm(R.make_desc(R.F16, 0, 512, 512), None, None, None)   # nothing to do: OK without pointers
+
+
+def test_wave_partition_equals_the_restated_reference_rule_everywhere():
+    """product (C ABI) against the oracle's restatement of computeWarpPartition (FriskOps.cpp:825-888) with the gfx950
+    parameters: 64-wide waves, 32 x 32 atoms; the same restatement reproduces the reference's golden layouts with the
+    NVIDIA parameters (tests/test_layout_oracle.py)"""
+    from oracle import layouts as L
+    for policy in (L.SQUARE, L.FULL_ROW, L.FULL_COL):
+        for tm in (32, 64, 96, 128, 256, 512):
+            for tn in (32, 64, 128, 160, 256):
+                for waves in (1, 2, 4, 8, 16):
+                    assert R.wave_partition(policy, tm, tn, waves) == L.warp_partition(policy, tm, tn, waves * 64, 64, 32, 32), (policy, tm, tn, waves)
+
+
+def test_lds_swizzle_representation_contains_the_reference_bank_swizzles():
+    """chunk ^ (((row >> sh) & mk) << cs) with (0,7,0) / (1,3,0) / (2,1,0) is the reference's full / half / quarter bank
+    swizzle (FriskOps.cpp:500-558) on rows of 128 / 64 / 32 bytes: same byte offset for every element of a 16-bit tile"""
+    from oracle import layouts as L
+    for cols, (sh, mk, cs), ref in ((64, (0, 7, 0), L.full_bank_swizzle), (32, (1, 3, 0), L.half_bank_swizzle), (16, (2, 1, 0), L.quarter_bank_swizzle)):
+        rows = 32
+        lay = R.LdsLayout(rows=rows, row_bytes=cols * 2, k_contiguous=1, row_shift=sh, row_mask=mk, chunk_shift=cs)
+        i, j = L.grid(rows, cols)
+        tc, ts, idx = ref(rows, cols, 16)(i, j)
+        assert int(np.max(tc)) == 0
+        want = (np.broadcast_to(ts, idx.shape) * 8 * cols + idx) * 2  # atoms of 8 rows follow each other
+        got = np.array([[R.lds_offset(lay, r, c * 2) for c in range(cols)] for r in range(rows)])
+        assert np.array_equal(got, want), (cols, sh, mk, cs)
