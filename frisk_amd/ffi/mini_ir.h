@@ -131,8 +131,8 @@ struct AffineExpr {
     }
     AffineExpr l(impl->lhs), r(impl->rhs);
     std::string out;
-    // binding strength as in MLIR's printer: operands of * mod floordiv ceildiv are parenthesised when
-    // they are sums; operands of a sum never are
+    // binding strength as in MLIR's printer: operands of * mod floordiv ceildiv are parenthesised whenever
+    // they are binary expressions themselves; operands of a sum never are
     if (kind() == ExprKind::Add) {
       // a + (-1) * b and a + (-c) print as subtractions
       if (r.kind() == ExprKind::Mul && AffineExpr(r.impl->rhs).is_constant() && AffineExpr(r.impl->rhs).constant_value() == -1)
@@ -144,10 +144,8 @@ struct AffineExpr {
       return nested ? "(" + out + ")" : out;
     }
     const char* op = kind() == ExprKind::Mul ? " * " : kind() == ExprKind::Mod ? " mod " : kind() == ExprKind::FloorDiv ? " floordiv " : " ceildiv ";
-    if (kind() == ExprKind::Mul && r.is_constant() && r.constant_value() == -1) return "-" + l.str(names, num_dims, true);
-    return l.str(names, num_dims, true) + op + r.str(names, num_dims, true);
-  }
-  std::string unused_tail_(bool nested, const std::string& out) const {
+    if (kind() == ExprKind::Mul && r.is_constant() && r.constant_value() == -1) out = "-" + l.str(names, num_dims, true);
+    else out = l.str(names, num_dims, true) + op + r.str(names, num_dims, true);
     return nested ? "(" + out + ")" : out;
   }
 };

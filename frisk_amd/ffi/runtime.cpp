@@ -96,6 +96,32 @@ GemmProgram program_of(py::object kernel, py::object module) {
   return match_tiled_gemm(k, m);
 }
 
+// Index map of an LDS tile in the form the reference prints its LayoutAttr (printLayoutDebug,
+// lib/Dialect/Frisk/IR/FriskAttributes.cpp:38-56): Layout(shape=[rows, cols], index=affine_map<(d0, d1) -> (...)>),
+// element (d0, d1) of the tile as stored -> element offset in LDS.  The XOR of the 16-byte chunk index with row bits is
+// written with sums and floordiv, bit by bit, as the reference writes its bank swizzles (FriskOps.cpp:123-143, 500-558).
+std::string lds_layout_debug(const frisk_lds_layout& L, int elem_bytes) {
+  const int64_t vec = 16 / elem_bytes, cols = L.row_bytes / elem_bytes;
+  AffineExpr i = AffineExpr::dim(0), j = AffineExpr::dim(1);
+  AffineExpr chunk = j.floor_div(AffineExpr::constant(vec));
+  AffineExpr stored = chunk;
+  if (L.row_mask) {
+    const int64_t lo = (int64_t)1 << L.chunk_shift, span = (int64_t)L.row_mask + 1;
+    AffineExpr field = chunk.floor_div(AffineExpr::constant(lo)).mod(AffineExpr::constant(span));  // the chunk bits the swizzle touches
+    AffineExpr key = i.floor_div(AffineExpr::constant((int64_t)1 << L.row_shift)).mod(AffineExpr::constant(span));
+    AffineExpr x = AffineExpr::constant(0);
+    for (int64_t b = 1; b < span; b *= 2) {
+      AffineExpr fb = field.floor_div(AffineExpr::constant(b)).mod(AffineExpr::constant(2));
+      AffineExpr kb = key.floor_div(AffineExpr::constant(b)).mod(AffineExpr::constant(2));
+      x = x + (fb + kb).mod(AffineExpr::constant(2)) * b;
+    }
+    stored = chunk + (x - field) * lo;
+  }
+  AffineExpr index = i * cols + stored * vec + j.mod(AffineExpr::constant(vec));
+  AffineMap map(2, 0, {index});
+  return "Layout(shape=[" + std::to_string(L.rows) + ", " + std::to_string(cols) + "], index=affine_map<" + map.str() + ">)";
+}
+
 py::dict program_dict(const GemmProgram& g) {
   py::dict d;
   d["kernel"] = g.kernel_name;
@@ -135,7 +161,12 @@ void init_ffi_runtime(py::module_&& m) {
     out["hip_waves"] = py::make_tuple(p.waves_m, p.waves_n);
     out["hip_grid"] = py::make_tuple(p.grid_y, p.grid_x);
     out["lds_bytes"] = p.lds_bytes;
-    out["stages"] = p.stages;
+    out["stages"] = py::make_tuple(p.stages, p.stages_b);
+    const int es = (int)(g.elem_ab.bit_width() / 8);
+    out["lds_a"] = lds_layout_debug(p.lds_a, es);
+    out["lds_b"] = lds_layout_debug(p.lds_b, es);
+    out["lds_swizzle"] = py::make_tuple(py::make_tuple(p.lds_a.row_shift, p.lds_a.row_mask, p.lds_a.chunk_shift),
+                                        py::make_tuple(p.lds_b.row_shift, p.lds_b.row_mask, p.lds_b.chunk_shift));
     out["flops"] = p.flops;
     out["bytes"] = p.bytes;
     return out;

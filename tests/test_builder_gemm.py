@@ -182,3 +182,34 @@ def test_plan_goes_through_the_hip_library():
     p = F.runtime.plan(kernel)
     assert p["hip_tile"] == (256, 256, 64) and p["hip_grid"] == (16, 16) and p["lds_bytes"] <= 160 * 1024
     assert p["hip_kernel"].startswith("f16_nt_256x256x64") and p["flops"] == 2.0 * 4096 ** 3
+
+
+@pytest.mark.parametrize("dtype,tile,trans_a,trans_b", [("fp16", (256, 256, 64), False, False), ("fp16", (256, 256, 64), False, True),
+                                                        ("bf16", (128, 128, 64), True, False),
+                                                        ("fp32", (128, 128, 32), False, False)])
+def test_plan_prints_lds_layouts_in_the_reference_debug_form(dtype, tile, trans_a, trans_b):
+    """Layout(shape=[...], index=affine_map<...>) as printLayoutDebug writes it; evaluating the printed map with the
+    oracle's affine evaluator gives, element by element, the offsets frisk_hip_lds_offset computes"""
+    import re
+
+    import numpy as np
+
+    from frisk_amd import runtime as R
+    from oracle import layouts as L
+    es = {"fp16": 2, "bf16": 2, "fp32": 4}[dtype]
+    h = F.create_session()
+    n = 4 * max(tile)
+    kernel = h.tiled_gemm("g", n, n, n, dtype, tile=tile, trans_a=trans_a, trans_b=trans_b)
+    p = F.runtime.plan(kernel)
+    for text, (sh, mk, cs) in zip((p["lds_a"], p["lds_b"]), p["lds_swizzle"]):
+        m = re.fullmatch(r"Layout\(shape=\[(\d+), (\d+)\], index=(affine_map<.*>)\)", text)
+        assert m, text
+        rows, cols = int(m.group(1)), int(m.group(2))
+        i, j = L.grid(rows, cols)
+        (idx,) = L.eval_affine_map(m.group(3), i, j)
+        lay = R.LdsLayout(rows=rows, row_bytes=cols * es, k_contiguous=1, row_shift=sh, row_mask=mk, chunk_shift=cs)
+        rr = np.random.default_rng(0).integers(0, rows, 300)
+        cc = np.random.default_rng(1).integers(0, cols, 300)
+        for r, c in zip(rr, cc):
+            assert R.lds_offset(lay, int(r), int(c) * es) == int(idx[r, c]) * es
+        assert len(np.unique(idx)) == rows * cols and idx.max() == rows * cols - 1  # a permutation of the tile
