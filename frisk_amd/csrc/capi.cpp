@@ -12,6 +12,7 @@
 #include "frisk_hip.h"
 #include "gemm_internal.h"
 #include "lds_model.h"
+#include "tile_ops.h"
 
 namespace frisk {
 
@@ -248,6 +249,19 @@ static int device_ok() {
   return cached;
 }
 
+// a rank-2 view handed to the tile ops: element type, extents, leading dimension, pointer
+static int check_view(const char* what, int dtype, const void* p, int64_t rows, int64_t cols, int64_t ld) {
+  if (dtype != FRISK_F32 && dtype != FRISK_F16 && dtype != FRISK_BF16) return fail(FRISK_ERR_DTYPE, "%s: element type %d is not f32, f16 or bf16", what, dtype);
+  if (rows < 0 || cols < 0) return fail(FRISK_ERR_SHAPE, "%s: negative extent %lld x %lld", what, (long long)rows, (long long)cols);
+  if (rows > INT32_MAX || cols > INT32_MAX) return fail(FRISK_ERR_SHAPE, "%s: extent exceeds 2^31-1", what);
+  if (ld < cols) return fail(FRISK_ERR_SHAPE, "%s: leading dimension %lld smaller than the row length %lld", what, (long long)ld, (long long)cols);
+  if (rows * cols > 0 && !p) return fail(FRISK_ERR_NULL, "%s: pointer is null", what);
+  if ((uintptr_t)p & (uintptr_t)(elem_size(dtype) - 1)) return fail(FRISK_ERR_ALIGNMENT, "%s: pointer is not aligned to its element size", what);
+  return FRISK_OK;
+}
+
+static bool rows_on_16_bytes(int dtype, const void* p, int64_t ld) { return ((uintptr_t)p & 15) == 0 && (ld * elem_size(dtype)) % 16 == 0; }
+
 }  // namespace frisk
 
 using namespace frisk;
@@ -354,6 +368,54 @@ int frisk_hip_wave_partition(int policy, int tile_m, int tile_n, int num_waves, 
   if (!waves_m || !waves_n) return fail(FRISK_ERR_NULL, "output pointers are null");
   if (policy < FRISK_POLICY_SQUARE || policy > FRISK_POLICY_FULL_COL) return fail(FRISK_ERR_TILE, "unknown wave policy %d", policy);
   wave_partition(policy, tile_m, tile_n, num_waves, 32, 32, waves_m, waves_n);
+  return FRISK_OK;
+}
+
+int frisk_hip_fill(int dtype, void* dst, int64_t rows, int64_t cols, int64_t ld, double value, void* stream) {
+  if (int st = check_view("fill destination", dtype, dst, rows, cols, ld)) return st;
+  if (rows == 0 || cols == 0) return FRISK_OK;
+  if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
+  if (ld == cols) { cols *= rows; rows = 1; ld = cols; }  // a dense view is one long row
+  hipError_t e = launch_fill(dtype, dst, rows, cols, ld, value, rows_on_16_bytes(dtype, dst, ld), (hipStream_t)stream);
+  if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "fill launch failed: %s", hipGetErrorString(e));
+  return FRISK_OK;
+}
+
+int frisk_hip_copy(int src_dtype, const void* src, int64_t src_ld, int dst_dtype, void* dst, int64_t dst_ld, int64_t rows, int64_t cols,
+                   void* stream) {
+  if (int st = check_view("copy source", src_dtype, src, rows, cols, src_ld)) return st;
+  if (int st = check_view("copy destination", dst_dtype, dst, rows, cols, dst_ld)) return st;
+  if (rows == 0 || cols == 0) return FRISK_OK;
+  if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
+  if (src_ld == cols && dst_ld == cols) { cols *= rows; rows = 1; src_ld = dst_ld = cols; }
+  const int vec = rows_on_16_bytes(src_dtype, src, src_ld) && rows_on_16_bytes(dst_dtype, dst, dst_ld);
+  hipError_t e = launch_copy(src_dtype, src, src_ld, dst_dtype, dst, dst_ld, rows, cols, vec, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "copy launch failed: %s", hipGetErrorString(e));
+  return FRISK_OK;
+}
+
+size_t frisk_hip_reduce_workspace_bytes(int dtype, int64_t rows, int64_t cols, int dim) {
+  if ((dtype != FRISK_F32 && dtype != FRISK_F16 && dtype != FRISK_BF16) || rows <= 0 || cols <= 0 || (dim != 0 && dim != 1)) return 0;
+  const int slices = reduce_slices(dtype, rows, cols, dim);
+  return slices > 1 ? (size_t)slices * (size_t)(dim == 1 ? rows : cols) * 4 : 0;
+}
+
+int frisk_hip_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int64_t ld, int dim, int kind, int clear, void* dst, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+  if (int st = check_view("reduce source", dtype, src, rows, cols, ld)) return st;
+  if (dim != 0 && dim != 1) return fail(FRISK_ERR_ARGUMENT, "reduce dim %d is out of range for a source of rank 2", dim);
+  if (kind < FRISK_REDUCE_ADD || kind > FRISK_REDUCE_MAX) return fail(FRISK_ERR_ARGUMENT, "unsupported reduce kind %d (add, mul, min, max)", kind);
+  const int64_t kept = dim == 1 ? rows : cols;
+  if (kept == 0) return FRISK_OK;
+  if (!dst) return fail(FRISK_ERR_NULL, "reduce destination: pointer is null");
+  if ((uintptr_t)dst & (uintptr_t)(elem_size(dtype) - 1)) return fail(FRISK_ERR_ALIGNMENT, "reduce destination: pointer is not aligned to its element size");
+  if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
+  int slices = (rows > 0 && cols > 0) ? reduce_slices(dtype, rows, cols, dim) : 1;
+  // without a (large enough, 4-byte aligned) workspace the reduction runs unsplit: same result, fewer work-groups
+  if (slices > 1 && (!workspace || workspace_bytes < (size_t)slices * (size_t)kept * 4 || ((uintptr_t)workspace & 3))) slices = 1;
+  hipError_t e = launch_reduce(dtype, src, rows, cols, ld, dim, kind, clear ? 1 : 0, dst, (float*)workspace, slices, rows_on_16_bytes(dtype, src, ld),
+                               (hipStream_t)stream);
+  if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "reduce launch failed: %s", hipGetErrorString(e));
   return FRISK_OK;
 }
 

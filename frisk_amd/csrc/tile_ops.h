@@ -1,0 +1,17 @@
+// Launch helpers of tile_ops.hip, called by the C ABI after argument validation.
+#pragma once
+#include <hip/hip_runtime_api.h>
+#include <stdint.h>
+#include "frisk_hip.h"
+
+namespace frisk {
+// vec_ok: every row of every view starts on a 16-byte boundary (pointers and leading dimensions), so whole
+// 16-byte groups may be moved with one access
+hipError_t launch_fill(int dtype, void* dst, int64_t rows, int64_t cols, int64_t ld, double value, int vec_ok, hipStream_t s);
+hipError_t launch_copy(int src_dtype, const void* src, int64_t src_ld, int dst_dtype, void* dst, int64_t dst_ld, int64_t rows, int64_t cols, int vec_ok,
+                       hipStream_t s);
+// slices > 1: the reduced extent is split over that many work-groups through `partial` (slices x kept-extent floats)
+int reduce_slices(int dtype, int64_t rows, int64_t cols, int dim);
+hipError_t launch_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int64_t ld, int dim, int kind, int clear, void* dst, float* partial, int slices,
+                         int vec_ok, hipStream_t s);
+}  // namespace frisk

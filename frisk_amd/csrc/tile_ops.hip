@@ -1,0 +1,264 @@
+// frisk.fill, frisk.copy and frisk.reduce on rank-2 views of device memory.  All three are bound by
+// HBM traffic: a lane moves 16 bytes at a time wherever the view allows it (row start and row length
+// multiples of 16 bytes), falls back to single elements otherwise, and a launch covers the view with
+// many more work-groups than the 256 CUs.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "tile_ops.h"
+
+namespace frisk {
+namespace {
+
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+template <int DT> struct Elem;
+template <> struct Elem<FRISK_F32> { typedef float T; static __device__ float load(const T& x) { return x; } static __device__ T store(float x) { return x; } };
+template <> struct Elem<FRISK_F16> { typedef _Float16 T; static __device__ float load(const T& x) { return (float)x; } static __device__ T store(float x) { return (_Float16)x; } };
+template <> struct Elem<FRISK_BF16> { typedef __bf16 T; static __device__ float load(const T& x) { return (float)x; } static __device__ T store(float x) { return (__bf16)x; } };
+
+// a rows x cols view is walked as (row, group of G columns); G columns of the narrower type fill 16 bytes
+__device__ __forceinline__ bool group_of(int64_t id, int64_t groups_per_row, int64_t rows, int64_t& r, int64_t& c0, int G) {
+  if (id >= groups_per_row * rows) return false;
+  r = id / groups_per_row;
+  c0 = (id % groups_per_row) * G;
+  return true;
+}
+
+template <int DT> __global__ void __launch_bounds__(256) fill_kernel(typename Elem<DT>::T* dst, int64_t rows, int64_t cols, int64_t ld, float value, int vec_ok) {
+  typedef typename Elem<DT>::T T;
+  constexpr int G = 16 / sizeof(T);
+  const int64_t gpr = (cols + G - 1) / G;
+  const T v = Elem<DT>::store(value);
+  for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;; id += (int64_t)gridDim.x * 256) {
+    int64_t r, c0;
+    if (!group_of(id, gpr, rows, r, c0, G)) break;
+    T* p = dst + r * ld + c0;
+    if (vec_ok && c0 + G <= cols) {
+      T tmp[G];
+#pragma unroll
+      for (int e = 0; e < G; ++e) tmp[e] = v;
+      *(v4u*)p = *(const v4u*)tmp;
+    } else {
+      for (int e = 0; e < G && c0 + e < cols; ++e) p[e] = v;
+    }
+  }
+}
+
+template <int SDT, int DDT> __global__ void __launch_bounds__(256)
+copy_kernel(const typename Elem<SDT>::T* src, int64_t sld, typename Elem<DDT>::T* dst, int64_t dld, int64_t rows, int64_t cols, int vec_ok) {
+  typedef typename Elem<SDT>::T S;
+  typedef typename Elem<DDT>::T D;
+  constexpr int G = 16 / (sizeof(S) < sizeof(D) ? sizeof(S) : sizeof(D));  // 16 bytes of the narrower side, 32 of the wider
+  const int64_t gpr = (cols + G - 1) / G;
+  for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;; id += (int64_t)gridDim.x * 256) {
+    int64_t r, c0;
+    if (!group_of(id, gpr, rows, r, c0, G)) break;
+    const S* sp = src + r * sld + c0;
+    D* dp = dst + r * dld + c0;
+    if (vec_ok && c0 + G <= cols) {
+      S in[G];
+      D out[G];
+#pragma unroll
+      for (int q = 0; q < (int)(G * sizeof(S) / 16); ++q) ((v4u*)in)[q] = ((const v4u*)sp)[q];
+#pragma unroll
+      for (int e = 0; e < G; ++e) {
+        if constexpr (SDT == DDT) out[e] = in[e]; else out[e] = Elem<DDT>::store(Elem<SDT>::load(in[e]));
+      }
+#pragma unroll
+      for (int q = 0; q < (int)(G * sizeof(D) / 16); ++q) ((v4u*)dp)[q] = ((const v4u*)out)[q];
+    } else {
+      for (int e = 0; e < G && c0 + e < cols; ++e) {
+        if constexpr (SDT == DDT) dp[e] = sp[e]; else dp[e] = Elem<DDT>::store(Elem<SDT>::load(sp[e]));
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------ reduce
+template <int KIND> struct Op;
+template <> struct Op<FRISK_REDUCE_ADD> { static __device__ float id() { return 0.f; } static __device__ float f(float a, float b) { return a + b; } };
+template <> struct Op<FRISK_REDUCE_MUL> { static __device__ float id() { return 1.f; } static __device__ float f(float a, float b) { return a * b; } };
+template <> struct Op<FRISK_REDUCE_MIN> { static __device__ float id() { return __builtin_inff(); } static __device__ float f(float a, float b) { return __builtin_fminf(a, b); } };
+template <> struct Op<FRISK_REDUCE_MAX> { static __device__ float id() { return -__builtin_inff(); } static __device__ float f(float a, float b) { return __builtin_fmaxf(a, b); } };
+
+template <int KIND> __device__ __forceinline__ float wave_reduce(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = Op<KIND>::f(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// along dim 1: work-group (x = row, y = column slice) reduces its slice of one row; lanes stride over 16-byte groups.
+// With gridDim.y == 1 the result goes to dst (combined with the old value unless clear), else to partial[y][row].
+template <int DT, int KIND> __global__ void __launch_bounds__(256)
+reduce_rows_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, int64_t ld, int clear, typename Elem<DT>::T* dst, float* partial, int vec_ok) {
+  typedef typename Elem<DT>::T T;
+  constexpr int G = 16 / sizeof(T);
+  const int64_t r = blockIdx.x;
+  const int64_t gpr = (cols + G - 1) / G;
+  const int64_t per = (gpr + gridDim.y - 1) / gridDim.y;
+  const int64_t g0 = (int64_t)blockIdx.y * per, g1 = g0 + per < gpr ? g0 + per : gpr;
+  float acc = Op<KIND>::id();
+  const T* row = src + r * ld;
+  for (int64_t g = g0 + threadIdx.x; g < g1; g += 256) {
+    const int64_t c0 = g * G;
+    if (vec_ok && c0 + G <= cols) {
+      T in[G];
+      *(v4u*)in = *(const v4u*)(row + c0);
+#pragma unroll
+      for (int e = 0; e < G; ++e) acc = Op<KIND>::f(acc, Elem<DT>::load(in[e]));
+    } else {
+      for (int e = 0; e < G && c0 + e < cols; ++e) acc = Op<KIND>::f(acc, Elem<DT>::load(row[c0 + e]));
+    }
+  }
+  __shared__ float wsum[4];
+  acc = wave_reduce<KIND>(acc);
+  if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float v = Op<KIND>::f(Op<KIND>::f(wsum[0], wsum[1]), Op<KIND>::f(wsum[2], wsum[3]));
+    if (gridDim.y > 1) partial[(int64_t)blockIdx.y * rows + r] = v;
+    else dst[r] = Elem<DT>::store(clear ? v : Op<KIND>::f(Elem<DT>::load(dst[r]), v));
+  }
+}
+
+// along dim 0: a work-group owns a strip of 32 x G columns and a slice of the rows; 32 column lanes x 8 row lanes
+template <int DT, int KIND> __global__ void __launch_bounds__(256)
+reduce_cols_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, int64_t ld, int clear, typename Elem<DT>::T* dst, float* partial, int vec_ok) {
+  typedef typename Elem<DT>::T T;
+  constexpr int G = 16 / sizeof(T);
+  const int cl = threadIdx.x & 31, rl = threadIdx.x >> 5;
+  const int64_t c0 = ((int64_t)blockIdx.x * 32 + cl) * G;
+  const int64_t per = (rows + gridDim.y - 1) / gridDim.y;
+  const int64_t r0 = (int64_t)blockIdx.y * per, r1 = r0 + per < rows ? r0 + per : rows;
+  float acc[G];
+#pragma unroll
+  for (int e = 0; e < G; ++e) acc[e] = Op<KIND>::id();
+  if (c0 < cols) {
+    for (int64_t r = r0 + rl; r < r1; r += 8) {
+      const T* p = src + r * ld + c0;
+      if (vec_ok && c0 + G <= cols) {
+        T in[G];
+        *(v4u*)in = *(const v4u*)p;
+#pragma unroll
+        for (int e = 0; e < G; ++e) acc[e] = Op<KIND>::f(acc[e], Elem<DT>::load(in[e]));
+      } else {
+        for (int e = 0; e < G && c0 + e < cols; ++e) acc[e] = Op<KIND>::f(acc[e], Elem<DT>::load(p[e]));
+      }
+    }
+  }
+  __shared__ float red[8][32][G + 1];
+#pragma unroll
+  for (int e = 0; e < G; ++e) red[rl][cl][e] = acc[e];
+  __syncthreads();
+  if (rl == 0 && c0 < cols) {
+#pragma unroll
+    for (int e = 0; e < G; ++e) {
+      float v = red[0][cl][e];
+#pragma unroll
+      for (int k = 1; k < 8; ++k) v = Op<KIND>::f(v, red[k][cl][e]);
+      if (c0 + e < cols) {
+        if (gridDim.y > 1) partial[(int64_t)blockIdx.y * cols + c0 + e] = v;
+        else dst[c0 + e] = Elem<DT>::store(clear ? v : Op<KIND>::f(Elem<DT>::load(dst[c0 + e]), v));
+      }
+    }
+  }
+}
+
+// second pass of a split reduction: out[i] = kind over s of partial[s][i] (combined with dst unless clear)
+template <int DT, int KIND> __global__ void __launch_bounds__(256)
+reduce_finish_kernel(const float* partial, int slices, int64_t n, int clear, typename Elem<DT>::T* dst) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float v = partial[i];
+  for (int s = 1; s < slices; ++s) v = Op<KIND>::f(v, partial[(int64_t)s * n + i]);
+  dst[i] = Elem<DT>::store(clear ? v : Op<KIND>::f(Elem<DT>::load(dst[i]), v));
+}
+
+unsigned blocks_for(int64_t work_items) {
+  int64_t b = (work_items + 255) / 256;
+  const int64_t cap = 256 * 16;  // 16 work-groups per CU keep every CU streaming; beyond that lanes loop
+  return (unsigned)(b < 1 ? 1 : (b > cap ? cap : b));
+}
+
+template <int DT> hipError_t fill_t(void* dst, int64_t rows, int64_t cols, int64_t ld, double value, int vec_ok, hipStream_t s) {
+  typedef typename Elem<DT>::T T;
+  constexpr int G = 16 / sizeof(T);
+  hipLaunchKernelGGL(fill_kernel<DT>, dim3(blocks_for(rows * ((cols + G - 1) / G))), dim3(256), 0, s, (T*)dst, rows, cols, ld, (float)value, vec_ok);
+  return hipGetLastError();
+}
+
+template <int SDT, int DDT> hipError_t copy_t(const void* src, int64_t sld, void* dst, int64_t dld, int64_t rows, int64_t cols, int vec_ok, hipStream_t s) {
+  typedef typename Elem<SDT>::T S;
+  typedef typename Elem<DDT>::T D;
+  constexpr int G = 16 / (sizeof(S) < sizeof(D) ? sizeof(S) : sizeof(D));
+  hipLaunchKernelGGL((copy_kernel<SDT, DDT>), dim3(blocks_for(rows * ((cols + G - 1) / G))), dim3(256), 0, s, (const S*)src, sld, (D*)dst, dld, rows, cols, vec_ok);
+  return hipGetLastError();
+}
+
+template <int DT, int KIND> hipError_t reduce_t(const void* src, int64_t rows, int64_t cols, int64_t ld, int dim, int clear, void* dst, float* partial,
+                                                int slices, int vec_ok, hipStream_t s) {
+  typedef typename Elem<DT>::T T;
+  constexpr int G = 16 / sizeof(T);
+  if (dim == 1) {
+    hipLaunchKernelGGL((reduce_rows_kernel<DT, KIND>), dim3((unsigned)rows, (unsigned)slices), dim3(256), 0, s, (const T*)src, rows, cols, ld, clear, (T*)dst, partial, vec_ok);
+  } else {
+    const unsigned strips = (unsigned)((cols + 32 * G - 1) / (32 * G));
+    hipLaunchKernelGGL((reduce_cols_kernel<DT, KIND>), dim3(strips, (unsigned)slices), dim3(256), 0, s, (const T*)src, rows, cols, ld, clear, (T*)dst, partial, vec_ok);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || slices == 1) return e;
+  const int64_t n = dim == 1 ? rows : cols;
+  hipLaunchKernelGGL((reduce_finish_kernel<DT, KIND>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, partial, slices, n, clear, (T*)dst);
+  return hipGetLastError();
+}
+
+template <int DT> hipError_t reduce_k(int kind, const void* src, int64_t rows, int64_t cols, int64_t ld, int dim, int clear, void* dst, float* partial, int slices,
+                                      int vec_ok, hipStream_t s) {
+  switch (kind) {
+    case FRISK_REDUCE_ADD: return reduce_t<DT, FRISK_REDUCE_ADD>(src, rows, cols, ld, dim, clear, dst, partial, slices, vec_ok, s);
+    case FRISK_REDUCE_MUL: return reduce_t<DT, FRISK_REDUCE_MUL>(src, rows, cols, ld, dim, clear, dst, partial, slices, vec_ok, s);
+    case FRISK_REDUCE_MIN: return reduce_t<DT, FRISK_REDUCE_MIN>(src, rows, cols, ld, dim, clear, dst, partial, slices, vec_ok, s);
+    default: return reduce_t<DT, FRISK_REDUCE_MAX>(src, rows, cols, ld, dim, clear, dst, partial, slices, vec_ok, s);
+  }
+}
+
+}  // namespace
+
+int reduce_slices(int dtype, int64_t rows, int64_t cols, int dim) {
+  // Split the reduced extent so that about 1024 work-groups exist, each still reducing at least 16 KiB.
+  const int es = dtype == FRISK_F32 ? 4 : 2;
+  const int G = 16 / es;
+  const int64_t groups = dim == 1 ? rows : (cols + 32 * G - 1) / (32 * G);
+  const int64_t extent_bytes = dim == 1 ? cols * es : rows * 32 * 16;  // bytes one work-group would walk unsplit
+  int slices = 1;
+  while (groups * slices < 1024 && extent_bytes / (slices * 2) >= 16384 && slices < 256) slices *= 2;
+  return slices;
+}
+
+hipError_t launch_fill(int dtype, void* dst, int64_t rows, int64_t cols, int64_t ld, double value, int vec_ok, hipStream_t s) {
+  switch (dtype) {
+    case FRISK_F32: return fill_t<FRISK_F32>(dst, rows, cols, ld, value, vec_ok, s);
+    case FRISK_F16: return fill_t<FRISK_F16>(dst, rows, cols, ld, value, vec_ok, s);
+    default: return fill_t<FRISK_BF16>(dst, rows, cols, ld, value, vec_ok, s);
+  }
+}
+
+hipError_t launch_copy(int sdt, const void* src, int64_t sld, int ddt, void* dst, int64_t dld, int64_t rows, int64_t cols, int vec_ok, hipStream_t s) {
+#define FRISK_COPY_CASE(S, D) if (sdt == S && ddt == D) return copy_t<S, D>(src, sld, dst, dld, rows, cols, vec_ok, s);
+  FRISK_COPY_CASE(FRISK_F32, FRISK_F32) FRISK_COPY_CASE(FRISK_F32, FRISK_F16) FRISK_COPY_CASE(FRISK_F32, FRISK_BF16)
+  FRISK_COPY_CASE(FRISK_F16, FRISK_F32) FRISK_COPY_CASE(FRISK_F16, FRISK_F16) FRISK_COPY_CASE(FRISK_F16, FRISK_BF16)
+  FRISK_COPY_CASE(FRISK_BF16, FRISK_F32) FRISK_COPY_CASE(FRISK_BF16, FRISK_F16) FRISK_COPY_CASE(FRISK_BF16, FRISK_BF16)
+#undef FRISK_COPY_CASE
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int64_t ld, int dim, int kind, int clear, void* dst, float* partial, int slices,
+                         int vec_ok, hipStream_t s) {
+  switch (dtype) {
+    case FRISK_F32: return reduce_k<FRISK_F32>(kind, src, rows, cols, ld, dim, clear, dst, partial, slices, vec_ok, s);
+    case FRISK_F16: return reduce_k<FRISK_F16>(kind, src, rows, cols, ld, dim, clear, dst, partial, slices, vec_ok, s);
+    default: return reduce_k<FRISK_BF16>(kind, src, rows, cols, ld, dim, clear, dst, partial, slices, vec_ok, s);
+  }
+}
+
+}  // namespace frisk

@@ -21,7 +21,7 @@ DTYPE_NAMES = {"fp32": F32, "f32": F32, "fp16": F16, "f16": F16, "bf16": BF16, "
 ACC_OF = {F32: F32, F16: F32, BF16: F32, I8: I32, E4M3: F32}
 
 STATUS_NAMES = {0: "OK", 1: "ERR_NULL", 2: "ERR_ABI", 3: "ERR_DTYPE", 4: "ERR_SHAPE", 5: "ERR_TILE", 6: "ERR_LDS",
-                7: "ERR_EPILOGUE", 8: "ERR_WORKSPACE", 9: "ERR_DEVICE", 10: "ERR_ALIGNMENT"}
+                7: "ERR_EPILOGUE", 8: "ERR_WORKSPACE", 9: "ERR_DEVICE", 10: "ERR_ALIGNMENT", 11: "ERR_ARGUMENT"}
 
 
 class GemmDesc(ctypes.Structure):
@@ -63,7 +63,8 @@ _lib = None
 
 EXPORTS = ["frisk_hip_abi_version", "frisk_hip_last_error", "frisk_hip_plan", "frisk_hip_workspace_bytes",
            "frisk_hip_gemm", "frisk_hip_lds_access_cycles", "frisk_hip_lds_search", "frisk_hip_lds_offset", "frisk_hip_wave_partition",
-           "frisk_hip_kernel_count", "frisk_hip_kernel_name"]
+           "frisk_hip_kernel_count", "frisk_hip_kernel_name", "frisk_hip_fill", "frisk_hip_copy", "frisk_hip_reduce",
+           "frisk_hip_reduce_workspace_bytes"]
 
 
 def lib():
@@ -92,6 +93,12 @@ def lib():
     L.frisk_hip_kernel_count.restype = ctypes.c_int
     L.frisk_hip_kernel_name.restype = ctypes.c_char_p
     L.frisk_hip_kernel_name.argtypes = [ctypes.c_int]
+    i64, vp = ctypes.c_int64, ctypes.c_void_p
+    L.frisk_hip_fill.argtypes = [ctypes.c_int, vp, i64, i64, i64, ctypes.c_double, vp]
+    L.frisk_hip_copy.argtypes = [ctypes.c_int, vp, i64, ctypes.c_int, vp, i64, i64, i64, vp]
+    L.frisk_hip_reduce_workspace_bytes.restype = ctypes.c_size_t
+    L.frisk_hip_reduce_workspace_bytes.argtypes = [ctypes.c_int, i64, i64, ctypes.c_int]
+    L.frisk_hip_reduce.argtypes = [ctypes.c_int, vp, i64, i64, i64, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, ctypes.c_size_t, vp]
     if L.frisk_hip_abi_version() != ABI_VERSION:
         raise ImportError("libfrisk_hip.so has ABI %d, binding expects %d" % (L.frisk_hip_abi_version(), ABI_VERSION))
     _lib = L
@@ -138,6 +145,29 @@ def gemm(desc, A_ptr, B_ptr, C_ptr, scaleA_ptr=None, scaleB_ptr=None, workspace_
     """Asynchronous launch on `stream` (a raw hipStream_t value or None). Pointers are raw device addresses."""
     _check(lib().frisk_hip_gemm(ctypes.byref(desc), A_ptr, B_ptr, C_ptr, scaleA_ptr, scaleB_ptr, workspace_ptr,
                                 workspace_bytes, stream))
+
+
+REDUCE_KINDS = {"add": 0, "sum": 0, "mul": 1, "min": 2, "max": 3}
+
+
+def fill(dtype, dst_ptr, rows, cols, ld, value, stream=None):
+    """frisk.fill on a rank-2 view of device memory (asynchronous on `stream`)"""
+    _check(lib().frisk_hip_fill(dtype, dst_ptr, rows, cols, ld, float(value), stream))
+
+
+def copy(src_dtype, src_ptr, src_ld, dst_dtype, dst_ptr, dst_ld, rows, cols, stream=None):
+    """frisk.copy of a rows x cols window, converting between f32 / f16 / bf16 when the types differ"""
+    _check(lib().frisk_hip_copy(src_dtype, src_ptr, src_ld, dst_dtype, dst_ptr, dst_ld, rows, cols, stream))
+
+
+def reduce_workspace_bytes(dtype, rows, cols, dim):
+    return int(lib().frisk_hip_reduce_workspace_bytes(dtype, rows, cols, dim))
+
+
+def reduce(dtype, src_ptr, rows, cols, ld, dim, kind, clear, dst_ptr, workspace_ptr=None, workspace_bytes=0, stream=None):
+    """frisk.reduce along `dim` with kind "add" | "mul" | "min" | "max" (or its enum value)"""
+    k = REDUCE_KINDS[kind] if isinstance(kind, str) else kind
+    _check(lib().frisk_hip_reduce(dtype, src_ptr, rows, cols, ld, dim, k, int(bool(clear)), dst_ptr, workspace_ptr, workspace_bytes, stream))
 
 
 def wave_partition(policy, tile_m, tile_n, num_waves):

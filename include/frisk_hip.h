@@ -60,7 +60,8 @@ typedef enum frisk_status {
   FRISK_ERR_EPILOGUE = 7,    /* epilogue needs scales that were not given             */
   FRISK_ERR_WORKSPACE = 8,   /* workspace missing or too small                        */
   FRISK_ERR_DEVICE = 9,      /* no gfx950 device / HIP runtime error                  */
-  FRISK_ERR_ALIGNMENT = 10   /* a pointer is not aligned to its element size */
+  FRISK_ERR_ALIGNMENT = 10,  /* a pointer is not aligned to its element size */
+  FRISK_ERR_ARGUMENT = 11    /* an enumerated argument (reduce kind, dim) is out of range */
 } frisk_status;
 
 /*
@@ -166,6 +167,39 @@ int frisk_hip_wave_partition(int policy, int tile_m, int tile_n, int num_waves, 
 /* Number of kernels compiled into the library and a printable name for each. */
 int frisk_hip_kernel_count(void);
 const char* frisk_hip_kernel_name(int kernel_id);
+
+/* ------------------------------------------------------------------------------------------------
+ * The dialect's data-movement ops on rank-2 views of device memory (row-major, leading dimension in
+ * elements; a rank-1 view is rows = 1).  Element types F32, F16, BF16.  All launches are asynchronous
+ * on `stream`; nothing is allocated.  Index maps and indices of the ops are applied by the caller as
+ * pointer offsets: a view is (pointer to its first element, rows, cols, ld).
+ * ------------------------------------------------------------------------------------------------ */
+typedef enum frisk_reduce_kind {
+  FRISK_REDUCE_ADD = 0,
+  FRISK_REDUCE_MUL = 1,
+  FRISK_REDUCE_MIN = 2,
+  FRISK_REDUCE_MAX = 3
+} frisk_reduce_kind;
+
+/* frisk.fill (include/Dialect/Frisk/IR/FriskOps.td:392-410; the value is a float attribute of the element
+ * type, lib/Dialect/Frisk/IR/FriskOps.cpp:1686-1701): every element of the view := value rounded to dtype. */
+int frisk_hip_fill(int dtype, void* dst, int64_t rows, int64_t cols, int64_t ld, double value, void* stream);
+
+/* frisk.copy (FriskOps.td:348-389; the window is src_extents / dst_extents, by default the destination
+ * shape, FriskOps.cpp:1564-1591): the rows x cols window at `src` goes to the window at `dst`.  Element
+ * types may differ (the fragment -> shared f32 -> f16 casts of tmp/ir.mlir:121,129): values are converted
+ * through fp32 with round-to-nearest-even.  The windows must not overlap. */
+int frisk_hip_copy(int src_dtype, const void* src, int64_t src_ld, int dst_dtype, void* dst, int64_t dst_ld, int64_t rows,
+                   int64_t cols, void* stream);
+
+/* frisk.reduce (FriskOps.td:412-441, verifier FriskOps.cpp:1733-1767): reduces the rows x cols view along
+ * `dim` (0: over rows, dst has cols entries; 1: over columns, dst has rows entries) with `kind`.  Arithmetic
+ * in fp32, result rounded to dtype.  clear = 1: dst := reduction; clear = 0: dst := kind(dst, reduction).
+ * min / max ignore NaN operands (maxnum / minnum).  Long reductions are split over work-groups through
+ * `workspace` (frisk_hip_reduce_workspace_bytes; 0 for most shapes). */
+size_t frisk_hip_reduce_workspace_bytes(int dtype, int64_t rows, int64_t cols, int dim);
+int frisk_hip_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int64_t ld, int dim, int kind, int clear, void* dst,
+                     void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

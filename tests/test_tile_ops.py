@@ -1,0 +1,181 @@
+"""frisk.fill / frisk.copy / frisk.reduce: the oracle against closed forms (CPU), the C ABI's argument checks (CPU),
+and the HIP kernels against the oracle through the C ABI (GPU).
+
+Bars: fill and same-type copy bit-exact; converting copies bit-exact (one rounding, the oracle's codec); min / max
+bit-exact; add / mul within 1e-3 (f16, bf16: the result's own rounding dominates) or 1e-5 (f32) of the float64 value,
+relative to max(|r|, rms(R))."""
+import numpy as np
+import pytest
+
+import oracle as O
+from oracle import tile_ops as T
+
+FLOATS = [O.F32, O.F16, O.BF16]
+NAMES = {O.F32: "f32", O.F16: "f16", O.BF16: "bf16"}
+
+
+# ------------------------------------------------------------------ oracle (CPU)
+def test_oracle_fill_and_copy_closed_forms():
+    for dt in FLOATS:
+        a = T.fill(dt, 3, 5, 1.25)
+        assert a.shape == (3, 5) and np.all(O.decode(dt, a) == 1.25)
+        assert np.all(O.decode(dt, T.fill(dt, 2, 2, -np.inf)) == -np.inf)
+    # 1/3 is not representable: the fill value is the type's nearest
+    assert O.decode(O.F16, T.fill(O.F16, 1, 1, 1.0 / 3.0))[0, 0] == np.float32(np.float16(1.0 / 3.0))
+    x = O.encode(O.F32, O.normal(77, 9, 0, 3.0)).reshape(7, 11)
+    assert np.array_equal(T.copy(O.F32, x, O.F32), x)
+    h = T.copy(O.F32, x, O.F16)
+    assert np.array_equal(h.view(np.float16), x.astype(np.float16))          # numpy's own RNE conversion
+    assert np.array_equal(T.copy(O.F16, h, O.F32), h.view(np.float16).astype(np.float32))   # widening is exact
+    assert np.array_equal(T.copy(O.F32, T.copy(O.F16, h, O.F32), O.F16), h)  # so the round trip is the identity
+
+
+def test_oracle_reduce_closed_forms_and_shape_rule():
+    n = 64
+    ramp = O.encode(O.F32, np.arange(1, n + 1, dtype=np.float32)).reshape(1, n)
+    assert O.decode(O.F32, T.reduce(O.F32, ramp, 1, "add"))[0] == n * (n + 1) / 2
+    assert O.decode(O.F32, T.reduce(O.F32, ramp, 1, "max"))[0] == n and O.decode(O.F32, T.reduce(O.F32, ramp, 1, "min"))[0] == 1
+    pw = O.encode(O.F32, np.array([[2.0, 0.5, 4.0, 0.25, 8.0]], dtype=np.float32))
+    assert O.decode(O.F32, T.reduce(O.F32, pw, 1, "mul"))[0] == 8.0           # powers of two: exact
+    x = O.encode(O.F16, O.normal(6 * 9, 10, 0, 1.0)).reshape(6, 9)
+    assert T.reduce(O.F16, x, 0, "add").shape == (9,) and T.reduce(O.F16, x, 1, "add").shape == (6,)   # rank - 1, other extent kept
+    xf = O.decode(O.F16, x).astype(np.float64).reshape(6, 9)
+    assert np.array_equal(T.reduce_f64(O.F16, x, 0, "max"), xf.max(axis=0)) and np.array_equal(T.reduce_f64(O.F16, x, 1, "min"), xf.min(axis=1))
+    # clear = False combines with the old destination
+    old = O.encode(O.F16, np.full(6, 100.0, dtype=np.float32))
+    assert np.all(O.decode(O.F16, T.reduce(O.F16, x, 1, "max", old)) == 100.0)
+    assert np.allclose(T.reduce_f64(O.F16, x, 1, "add", old), 100.0 + xf.sum(axis=1))
+    with pytest.raises(ValueError):
+        T.reduce(O.F16, x, 2, "add")
+    with pytest.raises(ValueError):
+        T.reduce(O.F16, x, 0, "xor")
+
+
+# ------------------------------------------------------------------ C ABI argument checks (no device needed)
+def test_tile_op_status_codes_before_any_launch():
+    from frisk_amd import runtime as R
+
+    def status(fn, *a):
+        with pytest.raises(R.FriskHipError) as e:
+            fn(*a)
+        return e.value.status
+    assert status(R.fill, R.I8, 0x1000, 4, 4, 4, 0.0) == R.ERR_DTYPE
+    assert status(R.fill, R.F16, 0x1000, -1, 4, 4, 0.0) == R.ERR_SHAPE
+    assert status(R.fill, R.F16, 0x1000, 4, 8, 4, 0.0) == R.ERR_SHAPE          # ld < cols
+    assert status(R.fill, R.F16, None, 4, 4, 4, 0.0) == R.ERR_NULL
+    assert status(R.fill, R.F32, 0x1002, 4, 4, 4, 0.0) == R.ERR_ALIGNMENT
+    assert status(R.copy, R.F32, 0x1000, 4, R.E4M3, 0x2000, 4, 4, 4) == R.ERR_DTYPE
+    assert status(R.copy, R.F32, 0x1000, 2, R.F16, 0x2000, 4, 4, 4) == R.ERR_SHAPE
+    assert status(R.reduce, R.F32, 0x1000, 4, 4, 4, 2, "add", True, 0x2000) == R.ERR_ARGUMENT   # dim out of range for rank 2
+    assert status(R.reduce, R.F32, 0x1000, 4, 4, 4, 0, 9, True, 0x2000) == R.ERR_ARGUMENT       # kind
+    assert status(R.reduce, R.F32, 0x1000, 4, 4, 4, 0, "add", True, None) == R.ERR_NULL
+    # empty views are legal and touch nothing
+    R.fill(R.F16, None, 0, 4, 4, 1.0)
+    R.copy(R.F16, None, 8, R.F32, None, 8, 4, 0)
+    R.reduce(R.F16, None, 0, 0, 0, 1, "add", True, None)
+    # the workspace request: nothing for short reductions, slices x kept extent x 4 bytes for long ones
+    assert R.reduce_workspace_bytes(R.F16, 8192, 8192, 1) == 0
+    w = R.reduce_workspace_bytes(R.F16, 8192, 8192, 0)
+    assert w > 0 and w % (8192 * 4) == 0
+    assert R.reduce_workspace_bytes(R.F16, 4, 1 << 22, 1) % (4 * 4) == 0 and R.reduce_workspace_bytes(R.F16, 4, 1 << 22, 1) > 0
+
+
+# ------------------------------------------------------------------ HIP kernels against the oracle (GPU)
+def _dev(arr):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(arr).view(np.uint8).reshape(-1).copy()).cuda()
+
+
+def _host(t, np_dtype):
+    return t.cpu().numpy().view(np_dtype)
+
+
+VIEWS = [(1, 1, 0, 0), (1, 1000, 0, 0), (37, 53, 0, 0), (64, 256, 0, 0), (64, 256, 8, 0), (33, 100, 3, 1), (300, 7, 1, 0), (5, 4096, 0, 0)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", FLOATS, ids=[NAMES[d] for d in FLOATS])
+def test_fill_gpu(hip, dt):
+    import torch
+    st = O.NP_STORAGE[dt]
+    es = np.dtype(st).itemsize
+    for rows, cols, pad, shift in VIEWS:
+        ld = cols + pad
+        buf = np.full(shift + rows * ld, 0x5A5A5A5A if es == 4 else 0x5A5A, dtype=st)
+        d = _dev(buf)
+        hip.fill(dt, d.data_ptr() + shift * es, rows, cols, ld, -2.71828, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        got = _host(d, st)
+        view = got[shift:shift + rows * ld].reshape(rows, ld)
+        assert np.array_equal(view[:, :cols], T.fill(dt, rows, cols, -2.71828)), (rows, cols, pad, shift)
+        assert np.array_equal(view[:, cols:], buf[shift:].reshape(rows, ld)[:, cols:]) and np.array_equal(got[:shift], buf[:shift])   # nothing outside the view
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sdt", FLOATS, ids=[NAMES[d] for d in FLOATS])
+@pytest.mark.parametrize("ddt", FLOATS, ids=[NAMES[d] for d in FLOATS])
+def test_copy_gpu(hip, sdt, ddt):
+    import torch
+    sst, dst_t = O.NP_STORAGE[sdt], O.NP_STORAGE[ddt]
+    ses, des = np.dtype(sst).itemsize, np.dtype(dst_t).itemsize
+    for rows, cols, pad, shift in VIEWS:
+        sld, dld = cols + pad, cols + 2 * pad
+        src = np.zeros(shift + rows * sld, dtype=sst)
+        vals = O.encode(sdt, O.normal(rows * cols, 21, 0, 50.0)).reshape(rows, cols)
+        src[shift:].reshape(rows, sld)[:, :cols] = vals
+        dst0 = np.full(shift + rows * dld, 0x7B7B7B7B if des == 4 else 0x7B7B, dtype=dst_t)
+        dS, dD = _dev(src), _dev(dst0)
+        hip.copy(sdt, dS.data_ptr() + shift * ses, sld, ddt, dD.data_ptr() + shift * des, dld, rows, cols, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        got = _host(dD, dst_t)
+        view = got[shift:].reshape(rows, dld)
+        assert np.array_equal(view[:, :cols], T.copy(sdt, vals, ddt)), (rows, cols, pad, shift)
+        assert np.array_equal(view[:, cols:], dst0[shift:].reshape(rows, dld)[:, cols:]) and np.array_equal(got[:shift], dst0[:shift])
+
+
+def _close(dt, got, ref64):
+    g = O.decode(dt, got).astype(np.float64).reshape(-1)
+    r = np.asarray(ref64, dtype=np.float64).reshape(-1)
+    tol = 1e-5 if dt == O.F32 else (1e-3 if dt == O.F16 else 8e-3)   # bf16 keeps 8 bits: half an ulp is 2^-9
+    scale = np.maximum(np.abs(r), np.sqrt(np.mean(r * r)) if r.size else 0.0)
+    assert np.all(np.isfinite(g)) and np.all(np.abs(g - r) <= tol * np.maximum(scale, 1e-30)), float(np.max(np.abs(g - r) / np.maximum(scale, 1e-30)))
+
+
+REDUCE_VIEWS = [(1, 1, 0), (7, 5, 0), (64, 256, 0), (33, 1000, 3), (300, 9, 1), (4, 70000, 0), (70000, 4, 0), (2048, 2048, 0), (16, 1 << 18, 0), (1 << 16, 40, 8)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", FLOATS, ids=[NAMES[d] for d in FLOATS])
+@pytest.mark.parametrize("dim", [0, 1])
+def test_reduce_gpu(hip, dt, dim):
+    import torch
+    st = O.NP_STORAGE[dt]
+    stream = torch.cuda.current_stream().cuda_stream
+    for rows, cols, pad in REDUCE_VIEWS:
+        ld = cols + pad
+        for kind in T.KINDS:
+            # products need factors near 1 and few of them to stay finite
+            if kind == "mul":
+                if (cols if dim == 1 else rows) > 300:
+                    continue
+                f = 1.0 + 0.01 * O.normal(rows * cols, 31, 0, 1.0)
+            else:
+                f = O.normal(rows * cols, 31, 1, 1.0)
+            vals = O.encode(dt, f.astype(np.float32)).reshape(rows, cols)
+            src = np.zeros(rows * ld, dtype=st)
+            src.reshape(rows, ld)[:, :cols] = vals
+            kept = rows if dim == 1 else cols
+            old = O.encode(dt, O.normal(kept, 32, 2, 0.5))
+            ws_bytes = hip.reduce_workspace_bytes(dt, rows, cols, dim)
+            ws = torch.full((max(ws_bytes, 4),), 0xFF, dtype=torch.uint8, device="cuda")
+            dS = _dev(src)
+            for clear, use_ws in ((True, True), (False, True), (True, False)):
+                dD = _dev(old)
+                hip.reduce(dt, dS.data_ptr(), rows, cols, ld, dim, kind, clear, dD.data_ptr(), ws.data_ptr() if use_ws and ws_bytes else None,
+                           ws_bytes if use_ws else 0, stream)
+                torch.cuda.synchronize()
+                got = _host(dD, st)
+                if kind in ("min", "max"):
+                    assert np.array_equal(got, T.reduce(dt, vals, dim, kind, None if clear else old)), (rows, cols, pad, kind, clear, use_ws)
+                else:
+                    _close(dt, got, T.reduce_f64(dt, vals, dim, kind, None if clear else old))
