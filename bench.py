@@ -158,6 +158,35 @@ def main():
     sk_gbs = sk_bytes / (sk_ms * 1e-3) / 1e9
     del Bf
 
+    # the dialect's data-movement ops on a 32768 x 8192 f16 view (512 MiB per array: twice the last-level cache)
+    def time_op(fn):
+        settle(torch, fn, stream)
+        e0.record(stream)
+        for _ in range(20):
+            fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / 20
+
+    orows, ocols = 32768, 8192
+    src16 = torch.randn(orows, ocols, device=dev, generator=g).half()
+    dst16 = torch.empty_like(src16)
+    red = torch.empty(orows, device=dev, dtype=torch.float16)
+    rws_bytes = R.reduce_workspace_bytes(R.F16, orows, ocols, 0)
+    rws = torch.empty(max(rws_bytes, 16), dtype=torch.uint8, device=dev)
+    cs = stream.cuda_stream
+    nbytes = orows * ocols * 2
+    ops = {}
+    for name, moved, fn in (
+            ("fill", nbytes, lambda: R.fill(R.F16, dst16.data_ptr(), orows, ocols, ocols, 1.5, cs)),
+            ("copy", 2 * nbytes, lambda: R.copy(R.F16, src16.data_ptr(), ocols, R.F16, dst16.data_ptr(), ocols, orows, ocols, cs)),
+            ("reduce_dim1_add", nbytes, lambda: R.reduce(R.F16, src16.data_ptr(), orows, ocols, ocols, 1, "add", True, red.data_ptr(), None, 0, cs)),
+            ("reduce_dim0_max", nbytes, lambda: R.reduce(R.F16, src16.data_ptr(), orows, ocols, ocols, 0, "max", True, red.data_ptr(), rws.data_ptr(),
+                                                         rws_bytes, cs))):
+        ms = time_op(fn)
+        ops[name] = {"GB/s": round(moved / (ms * 1e-3) / 1e9, 1), "frac_of_8TB/s": round(moved / (ms * 1e-3) / 8e12, 4), "kernel_ms": round(ms, 5)}
+    del src16, dst16
+
     line = {
         "metric": "GEMM TFLOP/s at 4096^3 fp16 (fp32 accumulate), 1 GPU",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -177,6 +206,7 @@ def main():
                                     "kernel": R.kernel_names()[pf.kernel_id], "split_k": pf.split_k,
                                     "workload": "fp8 e4m3 M=32 N=K=8192 NT, per-tensor scales, bf16 out; algorithmic bytes "
                                                 "|A|+|B|+|C|+scales per launch, B rotating over 6 buffers"},
+        "tile_ops_32768x8192_f16": ops,
     }
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(M, N, K)
