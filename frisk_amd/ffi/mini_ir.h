@@ -810,4 +810,98 @@ inline GemmProgram match_tiled_gemm(Operation* kernel, Operation* module = nullp
   return g;
 }
 
+// ------------------------------------------------------------------ data-movement programs
+// What the runtime extracts from a kernel whose entry block is a straight line of
+//   frisk.fill %arg            frisk.copy %arg[const map], %arg[const map] {src_extents, dst_extents}
+//   frisk.reduce %arg, %arg {kind, dim, clear}
+// on kernel arguments of rank 1 or 2 (global memrefs): one entry per op, in program order.  Window origins come from
+// index maps without inputs (constant results); extents follow the op (default: the destination shape left-padded
+// with 1s, FriskOps.cpp:1564-1591).
+struct TileOpDesc {
+  enum Kind { Fill, Copy, Reduce } kind = Fill;
+  int arg_src = -1, arg_dst = -1;          // kernel argument positions (fill: arg_dst only)
+  Type elem_src, elem_dst;
+  int64_t src_offset = 0, dst_offset = 0;  // elements from the start of the argument
+  int64_t rows = 0, cols = 0, src_ld = 0, dst_ld = 0;
+  double value = 0.0;                      // fill
+  std::string reduce_kind;                 // add | mul | min | max
+  int64_t dim = 0;
+  bool clear = true;
+};
+
+inline std::vector<TileOpDesc> match_data_movement(Operation* kernel) {
+  auto bad = [](const std::string& m) -> std::vector<TileOpDesc> { throw std::invalid_argument("not a data-movement kernel: " + m); };
+  if (!kernel || kernel->name != "frisk.kernel") return bad("expected a frisk.kernel");
+  if (kernel->regions.empty() || kernel->regions[0]->blocks.empty()) return bad("kernel has no entry block");
+  Block* entry = kernel->regions[0]->blocks[0];
+  struct View { int arg; Type elem; int64_t rows, cols; };
+  auto view_of = [&](Value v, const char* what) -> View {
+    int a = kernel_arg_index(kernel, v);
+    if (a < 0 || !v.type().is_memref()) throw std::invalid_argument(std::string("not a data-movement kernel: ") + what + " is not a kernel argument memref");
+    const auto& sh = v.type().impl->shape;
+    if (sh.empty() || sh.size() > 2) throw std::invalid_argument(std::string("not a data-movement kernel: ") + what + " must have rank 1 or 2");
+    for (int64_t d : sh) if (d < 0) throw std::invalid_argument(std::string("not a data-movement kernel: ") + what + " has a dynamic extent");
+    return View{a, v.type().element(), sh.size() == 2 ? sh[0] : 1, sh.back()};
+  };
+  // window (origin, extents) of a copy operand -> (element offset, rows, cols) inside its view
+  auto window_of = [&](const View& v, size_t rank, const AffineMap& map, const std::vector<int64_t>& ext, const char* what, int64_t& off, int64_t& r, int64_t& c) {
+    if (map.num_inputs() != 0) throw std::invalid_argument(std::string("not a data-movement kernel: the ") + what + " map of a copy must have constant results (no index operands)");
+    if ((size_t)map.num_results() != rank) throw std::invalid_argument(std::string("not a data-movement kernel: the ") + what + " map must give one origin per dimension");
+    std::vector<int64_t> org;
+    for (int i = 0; i < map.num_results(); ++i) {
+      const AffineExpr& e = map.impl->results[(size_t)i];
+      if (!e.is_constant()) throw std::invalid_argument(std::string("not a data-movement kernel: the ") + what + " origin is not constant");
+      org.push_back(e.constant_value());
+    }
+    // extents may carry leading 1s (source rank > destination rank): the window is their last `rank` entries
+    if (ext.size() < rank) throw std::invalid_argument(std::string("not a data-movement kernel: too few ") + what + " extents");
+    for (size_t i = 0; i + rank < ext.size(); ++i) if (ext[i] != 1) throw std::invalid_argument(std::string("not a data-movement kernel: leading ") + what + " extents must be 1");
+    std::vector<int64_t> e(ext.end() - (long)rank, ext.end());
+    int64_t r0 = rank == 2 ? org[0] : 0, c0 = org.back();
+    r = rank == 2 ? e[0] : 1;
+    c = e.back();
+    if (r0 < 0 || c0 < 0 || r < 0 || c < 0 || r0 + r > v.rows || c0 + c > v.cols) throw std::invalid_argument(std::string("not a data-movement kernel: the ") + what + " window leaves the memref");
+    off = r0 * v.cols + c0;
+  };
+  std::vector<TileOpDesc> out;
+  for (Operation* op : entry->ops) {
+    TileOpDesc d;
+    if (op->name == "frisk.end") continue;
+    if (op->name == "frisk.fill") {
+      View v = view_of(op->operands[0], "the fill target");
+      d.kind = TileOpDesc::Fill;
+      d.arg_dst = v.arg; d.elem_dst = v.elem; d.rows = v.rows; d.cols = v.cols; d.dst_ld = v.cols;
+      d.value = op->attr("value")->f;
+    } else if (op->name == "frisk.copy") {
+      View s = view_of(op->operands[0], "the copy source"), t = view_of(op->operands[1], "the copy destination");
+      d.kind = TileOpDesc::Copy;
+      d.arg_src = s.arg; d.arg_dst = t.arg; d.elem_src = s.elem; d.elem_dst = t.elem; d.src_ld = s.cols; d.dst_ld = t.cols;
+      int64_t sr, sc, tr, tc;
+      window_of(s, op->operands[0].type().impl->shape.size(), op->attr("srcMap")->map, op->attr("srcExtents")->ints, "source", d.src_offset, sr, sc);
+      window_of(t, op->operands[1].type().impl->shape.size(), op->attr("dstMap")->map, op->attr("dstExtents")->ints, "destination", d.dst_offset, tr, tc);
+      if (sr * sc != tr * tc) return bad("source and destination windows of a copy hold different numbers of elements");
+      if (sr == tr && sc == tc) { d.rows = sr; d.cols = sc; }
+      else if (sr == 1 && tr == 1) { d.rows = 1; d.cols = sc; }
+      else if ((sr == 1 || tr == 1) && (sc == s.cols || sr == 1) && (tc == t.cols || tr == 1)) { d.rows = 1; d.cols = sr * sc; d.src_ld = d.dst_ld = d.cols; }  // a dense window against a row
+      else return bad("source and destination windows of a copy have different shapes");
+    } else if (op->name == "frisk.reduce") {
+      View s = view_of(op->operands[0], "the reduce source"), t = view_of(op->operands[1], "the reduce destination");
+      if (op->operands[0].type().impl->shape.size() != 2) return bad("the reduce source must have rank 2");
+      d.kind = TileOpDesc::Reduce;
+      d.arg_src = s.arg; d.arg_dst = t.arg; d.elem_src = s.elem; d.elem_dst = t.elem; d.rows = s.rows; d.cols = s.cols; d.src_ld = s.cols;
+      d.dim = op->int_attr("dim");
+      d.reduce_kind = op->attr("kind")->s == "sum" ? "add" : op->attr("kind")->s;
+      d.clear = op->attr("clear")->b;
+      if (d.dim != 0 && d.dim != 1) return bad("reduce dimension out of range");
+      if (t.rows * t.cols != (d.dim == 1 ? s.rows : s.cols)) return bad("the reduce destination does not hold one element per kept index");
+      if (!s.elem.equals(t.elem)) return bad("reduce source and destination element types differ");
+    } else {
+      return bad("operation " + op->name + " is not fill, copy or reduce");
+    }
+    out.push_back(d);
+  }
+  if (out.empty()) return bad("the kernel holds no fill, copy or reduce");
+  return out;
+}
+
 }  // namespace frisk_ir

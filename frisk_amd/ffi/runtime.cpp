@@ -1,5 +1,6 @@
 // `frisk_ffi.runtime`: lowers a tiled-GEMM kernel built with the IR builder to a
-// frisk_gemm_desc and launches it through the C ABI of libfrisk_hip.so
+// frisk_gemm_desc, or a straight line of fill / copy / reduce ops to the tile-op
+// entry points, and launches it through the C ABI of libfrisk_hip.so
 // (include/frisk_hip.h).  This fills the slot the reference reserves for
 // `init_ffi_passes` (ffi/ffi.h:14, ffi/ffi.cpp:6): the reference has nothing
 // below its builder, so what it would lower to is the library's entry points.
@@ -27,6 +28,10 @@ struct HipLibrary {
   decltype(&frisk_hip_last_error) last_error = nullptr;
   decltype(&frisk_hip_abi_version) abi_version = nullptr;
   decltype(&frisk_hip_kernel_name) kernel_name = nullptr;
+  decltype(&frisk_hip_fill) fill = nullptr;
+  decltype(&frisk_hip_copy) copy = nullptr;
+  decltype(&frisk_hip_reduce) reduce = nullptr;
+  decltype(&frisk_hip_reduce_workspace_bytes) reduce_workspace_bytes = nullptr;
 };
 
 HipLibrary g_lib;
@@ -47,7 +52,11 @@ HipLibrary& library() {
   lib.last_error = (decltype(lib.last_error))dlsym(h, "frisk_hip_last_error");
   lib.abi_version = (decltype(lib.abi_version))dlsym(h, "frisk_hip_abi_version");
   lib.kernel_name = (decltype(lib.kernel_name))dlsym(h, "frisk_hip_kernel_name");
-  if (!lib.plan || !lib.gemm || !lib.last_error || !lib.abi_version || !lib.kernel_name)
+  lib.fill = (decltype(lib.fill))dlsym(h, "frisk_hip_fill");
+  lib.copy = (decltype(lib.copy))dlsym(h, "frisk_hip_copy");
+  lib.reduce = (decltype(lib.reduce))dlsym(h, "frisk_hip_reduce");
+  lib.reduce_workspace_bytes = (decltype(lib.reduce_workspace_bytes))dlsym(h, "frisk_hip_reduce_workspace_bytes");
+  if (!lib.plan || !lib.gemm || !lib.last_error || !lib.abi_version || !lib.kernel_name || !lib.fill || !lib.copy || !lib.reduce || !lib.reduce_workspace_bytes)
     throw std::runtime_error("frisk runtime: " + g_lib_path + " does not export the frisk_hip entry points");
   if (lib.abi_version() != FRISK_HIP_ABI_VERSION) throw std::runtime_error("frisk runtime: libfrisk_hip.so ABI version mismatch");
   g_lib = lib;
@@ -136,6 +145,26 @@ py::dict program_dict(const GemmProgram& g) {
   return d;
 }
 
+int reduce_kind_of(const std::string& k) {
+  if (k == "add") return FRISK_REDUCE_ADD;
+  if (k == "mul") return FRISK_REDUCE_MUL;
+  if (k == "min") return FRISK_REDUCE_MIN;
+  if (k == "max") return FRISK_REDUCE_MAX;
+  throw std::invalid_argument("unsupported reduce kind: " + k + ". Supported: add, mul, min, max");
+}
+
+py::dict tile_op_dict(const TileOpDesc& d) {
+  py::dict o;
+  o["op"] = d.kind == TileOpDesc::Fill ? "fill" : d.kind == TileOpDesc::Copy ? "copy" : "reduce";
+  o["rows"] = d.rows; o["cols"] = d.cols;
+  if (d.kind != TileOpDesc::Fill) { o["src"] = d.arg_src; o["src_offset"] = d.src_offset; o["src_ld"] = d.src_ld; o["src_dtype"] = d.elem_src.str(); }
+  o["dst"] = d.arg_dst; o["dst_offset"] = d.dst_offset; o["dst_dtype"] = d.elem_dst.str();
+  if (d.kind != TileOpDesc::Reduce) o["dst_ld"] = d.dst_ld;
+  if (d.kind == TileOpDesc::Fill) o["value"] = d.value;
+  if (d.kind == TileOpDesc::Reduce) { o["kind"] = d.reduce_kind; o["dim"] = d.dim; o["clear"] = d.clear; }
+  return o;
+}
+
 }  // namespace
 
 void init_ffi_runtime(py::module_&& m) {
@@ -171,6 +200,46 @@ void init_ffi_runtime(py::module_&& m) {
     out["bytes"] = p.bytes;
     return out;
   }, py::arg("kernel"), py::arg("module") = py::none(), py::arg("epilogue") = "none");
+
+  m.def("match_ops", [](py::object kernel) {
+    py::list out;
+    for (const TileOpDesc& d : match_data_movement(op_of_handle(kernel))) out.append(tile_op_dict(d));
+    return out;
+  }, py::arg("kernel"), "recognise a kernel whose body is a straight line of fill / copy / reduce on its arguments; pure host");
+
+  m.def("ops_workspace_bytes", [](py::object kernel) {
+    HipLibrary& lib = library();
+    size_t need = 0;
+    for (const TileOpDesc& d : match_data_movement(op_of_handle(kernel)))
+      if (d.kind == TileOpDesc::Reduce) need = std::max(need, lib.reduce_workspace_bytes(dtype_of(d.elem_src), d.rows, d.cols, (int)d.dim));
+    return need;
+  }, py::arg("kernel"), "device workspace launch_ops can use for the kernel's longest reduction (0 if none needs one)");
+
+  m.def("launch_ops", [](py::object kernel, std::vector<uint64_t> args, uint64_t stream, uint64_t workspace, size_t workspace_bytes) {
+    std::vector<TileOpDesc> ops = match_data_movement(op_of_handle(kernel));
+    HipLibrary& lib = library();
+    auto ptr = [&](int arg, int64_t offset, const Type& elem) -> void* {
+      if (arg < 0 || (size_t)arg >= args.size()) throw std::invalid_argument("launch_ops needs one device pointer per kernel argument");
+      return (void*)(args[(size_t)arg] + (uint64_t)offset * (uint64_t)(elem.bit_width() / 8));
+    };
+    py::gil_scoped_release release;
+    for (const TileOpDesc& d : ops) {  // program order on one stream: each op sees the results of the ones before it
+      int st = 0;
+      if (d.kind == TileOpDesc::Fill)
+        st = lib.fill(dtype_of(d.elem_dst), ptr(d.arg_dst, d.dst_offset, d.elem_dst), d.rows, d.cols, d.dst_ld, d.value, (void*)stream);
+      else if (d.kind == TileOpDesc::Copy)
+        st = lib.copy(dtype_of(d.elem_src), ptr(d.arg_src, d.src_offset, d.elem_src), d.src_ld, dtype_of(d.elem_dst), ptr(d.arg_dst, d.dst_offset, d.elem_dst),
+                      d.dst_ld, d.rows, d.cols, (void*)stream);
+      else
+        st = lib.reduce(dtype_of(d.elem_src), ptr(d.arg_src, d.src_offset, d.elem_src), d.rows, d.cols, d.src_ld, (int)d.dim, reduce_kind_of(d.reduce_kind),
+                        d.clear ? 1 : 0, ptr(d.arg_dst, d.dst_offset, d.elem_dst), (void*)workspace, workspace_bytes, (void*)stream);
+      if (st) {
+        py::gil_scoped_acquire acquire;
+        throw std::runtime_error(std::string("frisk_hip tile op: ") + lib.last_error() + " (status " + std::to_string(st) + ")");
+      }
+    }
+  }, py::arg("kernel"), py::arg("args"), py::arg("stream") = 0, py::arg("workspace") = 0, py::arg("workspace_bytes") = 0,
+     "asynchronous launch, in program order on `stream`, of a kernel made of fill / copy / reduce on its arguments");
 
   m.def("launch", [](py::object kernel, std::vector<uint64_t> args, uint64_t stream, py::object module, const std::string& epilogue,
                      uint64_t scale_a, uint64_t scale_b) {

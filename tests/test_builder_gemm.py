@@ -213,3 +213,41 @@ def test_plan_prints_lds_layouts_in_the_reference_debug_form(dtype, tile, trans_
         for r, c in zip(rr, cc):
             assert R.lds_offset(lay, int(r), int(c) * es) == int(idx[r, c]) * es
         assert len(np.unique(idx)) == rows * cols and idx.max() == rows * cols - 1  # a permutation of the tile
+
+
+def _data_movement_kernel(h):
+    """kernel(x: 64x96 f32, y: 64x96 f16, v: 64 f16): y := 0.5; y[8:40, 16:80] := f16(x[0:32, 32:96]); v := max over columns of y"""
+    b = h.builder
+    x_t, y_t, v_t = h.memref_type((64, 96), "fp32"), h.memref_type((64, 96), "fp16"), h.memref_type((64,), "fp16")
+    kernel, entry = h.new_kernel("prep", [x_t, y_t, v_t])
+    x, y, v = (entry.get_argument(i) for i in range(3))
+    c = b.get_affine_constant_expr
+    b.create_fill_op(y, 0.5, "fp16")
+    b.create_copy_op(x, y, [], [], srcMap=F.AffineMap.get(0, 0, [c(0), c(32)]), dstMap=F.AffineMap.get(0, 0, [c(8), c(16)]),
+                     srcExtents=[32, 64], dstExtents=[32, 64])
+    b.create_reduce_op(y, v, "max", 1, True)
+    return kernel
+
+
+def test_data_movement_kernel_is_recognised_op_by_op():
+    h = F.create_session()
+    kernel = _data_movement_kernel(h)
+    assert h.module.verify()
+    ops = F.runtime.match_ops(kernel)
+    assert [o["op"] for o in ops] == ["fill", "copy", "reduce"]
+    assert ops[0] == {"op": "fill", "rows": 64, "cols": 96, "dst": 1, "dst_offset": 0, "dst_dtype": "f16", "dst_ld": 96, "value": 0.5}
+    assert ops[1]["src"] == 0 and ops[1]["src_offset"] == 32 and ops[1]["dst_offset"] == 8 * 96 + 16 and (ops[1]["rows"], ops[1]["cols"]) == (32, 64)
+    assert (ops[1]["src_ld"], ops[1]["dst_ld"], ops[1]["src_dtype"], ops[1]["dst_dtype"]) == (96, 96, "f32", "f16")
+    assert ops[2]["kind"] == "max" and ops[2]["dim"] == 1 and ops[2]["clear"] is True and (ops[2]["src"], ops[2]["dst"]) == (1, 2)
+    # a tiled GEMM is not a data-movement kernel, and a window that leaves its memref is refused
+    with pytest.raises(ValueError):
+        F.runtime.match_ops(h.tiled_gemm("g", 256, 256, 64, "fp16", tile=(128, 128, 32)))
+    h2 = F.create_session()
+    t = h2.memref_type((8, 8), "fp32")
+    k2, e2 = h2.new_kernel("bad", [t, t])
+    c = h2.builder.get_affine_constant_expr
+    h2.builder.create_copy_op(e2.get_argument(0), e2.get_argument(1), [], [], srcMap=F.AffineMap.get(0, 0, [c(4), c(0)]),
+                              dstMap=F.AffineMap.get(0, 0, [c(0), c(0)]), srcExtents=[8, 8], dstExtents=[8, 8])
+    with pytest.raises(ValueError) as e:
+        F.runtime.match_ops(k2)
+    assert "window leaves the memref" in str(e.value)

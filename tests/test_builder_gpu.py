@@ -60,3 +60,24 @@ def test_int8_with_dequant_epilogue_through_the_builder(hip):
     got = _run(kernel, A, B, M, N, np.uint16, epilogue="row_col_scale", scale_a=dsA.data_ptr(), scale_b=dsB.data_ptr())
     assert np.array_equal(got, O.epilogue_rowcol_f16(O.gemm_i32(A, B), sA, sB))
     del torch
+
+
+def test_data_movement_kernel_through_the_builder(hip):
+    """fill, converting window copy and row-wise max built with the IR builder, run op by op on the device, against the oracle"""
+    import torch
+    from oracle import tile_ops as T
+    from test_builder_gemm import _data_movement_kernel
+    h = F.create_session()
+    kernel = _data_movement_kernel(h)
+    x = O.encode(O.F32, O.normal(64 * 96, 51, 0, 2.0)).reshape(64, 96)
+    dx = to_dev(x)
+    dy = torch.full((64 * 96 * 2,), 0xEE, dtype=torch.uint8, device="cuda")
+    dv = torch.full((64 * 2,), 0xEE, dtype=torch.uint8, device="cuda")
+    ws_bytes = F.runtime.ops_workspace_bytes(kernel)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device="cuda")
+    F.runtime.launch_ops(kernel, [dx.data_ptr(), dy.data_ptr(), dv.data_ptr()], torch.cuda.current_stream().cuda_stream, ws.data_ptr(), ws_bytes)
+    torch.cuda.synchronize()
+    want_y = T.fill(O.F16, 64, 96, 0.5)
+    want_y[8:40, 16:80] = T.copy(O.F32, np.ascontiguousarray(x[0:32, 32:96]), O.F16)
+    assert np.array_equal(from_dev(dy, np.uint16, (64, 96)), want_y)
+    assert np.array_equal(from_dev(dv, np.uint16, (64,)), T.reduce(O.F16, want_y, 1, "max"))
