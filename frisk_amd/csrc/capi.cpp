@@ -2,6 +2,7 @@
 // grid / LDS layout choice) and kernel dispatch.  Host code only.
 #include <hip/hip_runtime_api.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -240,13 +241,15 @@ static int group_rows(int tiles_m, int tiles_n) {
 }
 
 static int device_ok() {
-  static int cached = -1;
-  if (cached >= 0) return cached;
+  static std::atomic<int> cached{-1};  // the answer for the process's GPU; racing threads compute the same value
+  int c = cached.load(std::memory_order_relaxed);
+  if (c >= 0) return c;
   int dev = 0;
   hipDeviceProp_t prop;
   if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
-  cached = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
-  return cached;
+  c = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
+  cached.store(c, std::memory_order_relaxed);
+  return c;
 }
 
 // a rank-2 view handed to the tile ops: element type, extents, leading dimension, pointer

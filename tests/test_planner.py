@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_plans_of_the_benchmark_configurations():
     cases = [
-        (R.F32, 1024, 1024, 1024, 0, 0, R.F32, (64, 64, 32)),
+        (R.F32, 1024, 1024, 1024, 0, 0, R.F32, (64, 64, 64)),
         (R.F16, 4096, 4096, 4096, 0, 0, R.F16, (256, 256, 64)),
         (R.BF16, 8192, 8192, 8192, 0, 1, R.BF16, (256, 256, 64)),
         (R.I8, 4096, 4096, 4096, 0, 0, R.F16, (256, 256, 128)),
@@ -61,6 +61,7 @@ SHAPES = [  # rows, row_bytes, k_contiguous, elem_bytes, frag_bytes, tile_mn, ti
     (256, 128, 1, 1, 16, 256, 128), (128, 256, 0, 1, 16, 256, 128), (128, 128, 1, 1, 16, 128, 128), (128, 128, 0, 1, 16, 128, 128),
     (256, 128, 1, 1, 32, 256, 128), (128, 256, 0, 1, 32, 256, 128), (128, 128, 1, 1, 32, 128, 128), (128, 128, 0, 1, 32, 128, 128),
     (128, 128, 1, 4, 4, 128, 32), (32, 512, 0, 4, 4, 128, 32), (64, 128, 1, 4, 4, 64, 32), (32, 256, 0, 4, 4, 64, 32),
+    (64, 256, 1, 4, 4, 64, 64), (64, 256, 0, 4, 4, 64, 64),
 ]
 
 
