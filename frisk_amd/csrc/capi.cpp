@@ -275,6 +275,13 @@ int frisk_hip_abi_version(void) { return FRISK_HIP_ABI_VERSION; }
 
 const char* frisk_hip_last_error(void) { return g_last_error.c_str(); }
 
+int frisk_hip_init(void) {
+  if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
+  for (const KernelEntry* k : kernels())
+    if (hipError_t e = k->prepare(); e != hipSuccess) return fail(FRISK_ERR_DEVICE, "preparing %s failed: %s", k->name, hipGetErrorString(e));
+  return FRISK_OK;
+}
+
 int frisk_hip_plan(const frisk_gemm_desc* desc, frisk_gemm_plan* plan) { return make_plan(desc, plan, true); }
 
 size_t frisk_hip_workspace_bytes(const frisk_gemm_desc* desc) {

@@ -35,6 +35,7 @@ struct KernelEntry {
   int splitk;  // 1: compiled with the split-K store path
   int lds_bytes;
   hipError_t (*launch)(const GemmParams&, hipStream_t);
+  hipError_t (*prepare)();  // one-time, non-stream set-up of the kernel function (dynamic LDS limit)
 };
 
 // sums the split-K slices and applies the epilogue (splitk_reduce.hip)

@@ -61,7 +61,7 @@ class FriskHipError(RuntimeError):
 
 _lib = None
 
-EXPORTS = ["frisk_hip_abi_version", "frisk_hip_last_error", "frisk_hip_plan", "frisk_hip_workspace_bytes",
+EXPORTS = ["frisk_hip_init", "frisk_hip_abi_version", "frisk_hip_last_error", "frisk_hip_plan", "frisk_hip_workspace_bytes",
            "frisk_hip_gemm", "frisk_hip_lds_access_cycles", "frisk_hip_lds_search", "frisk_hip_lds_offset", "frisk_hip_wave_partition",
            "frisk_hip_kernel_count", "frisk_hip_kernel_name", "frisk_hip_fill", "frisk_hip_copy", "frisk_hip_reduce",
            "frisk_hip_reduce_workspace_bytes"]
@@ -134,6 +134,11 @@ def plan(desc):
     p = GemmPlan()
     _check(lib().frisk_hip_plan(ctypes.byref(desc), ctypes.byref(p)))
     return p
+
+
+def init():
+    """one-time set-up on the current device; needed only before launches are captured into a HIP graph"""
+    _check(lib().frisk_hip_init())
 
 
 def workspace_bytes(desc):

@@ -126,6 +126,11 @@ typedef struct frisk_gemm_plan {
 
 int frisk_hip_abi_version(void);
 
+/* Optional one-time set-up on the current device: everything that is not a stream operation (the kernels' dynamic
+ * LDS limits).  Launches do this lazily for the kernel they pick, so the call is only needed before launches are
+ * captured into a HIP graph, where such set-up is not allowed.  The reference has no counterpart (it launches nothing). */
+int frisk_hip_init(void);
+
 /* thread-local text of the last non-OK status returned on this thread */
 const char* frisk_hip_last_error(void);
 

@@ -1,0 +1,67 @@
+"""Launches through the C ABI recorded into a HIP graph (stream capture) and replayed: every replay must give the bits
+of the same launches made eagerly.  The entry points allocate nothing and synchronise nothing, and frisk_hip_init does
+the one piece of non-stream set-up (the kernels' LDS limits) ahead of the capture."""
+import numpy as np
+import pytest
+
+import oracle as O
+from helpers import make_operand, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def test_gemm_split_k_and_reduce_replay_from_a_graph(hip):
+    import torch
+    hip.init()
+    M, N, K = 512, 512, 256
+    Ms = 32
+    dA = to_dev(make_operand(O.F16, M, K, seed=61, tensor=0, scale=0.25))
+    dB = to_dev(make_operand(O.F16, K, N, seed=61, tensor=1, scale=0.25))
+    dAs = to_dev(make_operand(O.F16, Ms, 2048, seed=61, tensor=2, scale=0.25))
+    dBs = to_dev(make_operand(O.F16, 2048, N, seed=61, tensor=3, scale=0.25))
+    dC = torch.zeros(M * N * 2, dtype=torch.uint8, device="cuda")
+    dCs = torch.zeros(Ms * N * 2, dtype=torch.uint8, device="cuda")
+    dV = torch.zeros(M * 2, dtype=torch.uint8, device="cuda")
+    d1 = hip.make_desc(O.F16, M, N, K)
+    d2 = hip.make_desc(O.F16, Ms, N, 2048, split_k=4)
+    p2 = hip.plan(d2)
+    assert p2.split_k == 4 and p2.workspace_bytes > 0
+    ws = torch.empty(p2.workspace_bytes, dtype=torch.uint8, device="cuda")
+
+    def launches(stream):
+        hip.gemm(d1, dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), None, None, None, 0, stream)
+        hip.gemm(d2, dAs.data_ptr(), dBs.data_ptr(), dCs.data_ptr(), None, None, ws.data_ptr(), ws.numel(), stream)
+        hip.reduce(O.F16, dC.data_ptr(), M, N, N, 1, "max", True, dV.data_ptr(), None, 0, stream)
+
+    def snapshot():
+        torch.cuda.synchronize()
+        return dC.cpu().numpy().copy(), dCs.cpu().numpy().copy(), dV.cpu().numpy().copy()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on the capture stream, as captures want
+        launches(side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launches(torch.cuda.current_stream().cuda_stream)
+
+    for rep in range(3):
+        # new operand contents in the same buffers, then the eager result, then scrub the outputs and replay
+        dA.copy_(to_dev(make_operand(O.F16, M, K, seed=70 + rep, tensor=0, scale=0.25)))
+        dAs.copy_(to_dev(make_operand(O.F16, Ms, 2048, seed=70 + rep, tensor=2, scale=0.25)))
+        launches(torch.cuda.current_stream().cuda_stream)
+        want = snapshot()
+        for t in (dC, dCs, dV, ws):
+            t.fill_(0xA5)
+        torch.cuda.synchronize()
+        graph.replay()
+        got = snapshot()
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w), "replay %d differs from the eager launches" % rep
+    # and the eager result is the oracle's
+    A = dA.cpu().numpy().view(np.uint16).reshape(M, K)
+    B = dB.cpu().numpy().view(np.uint16).reshape(K, N)
+    r = O.compare(O.F16, want[0].view(np.uint16).reshape(M, N), O.gemm_f64(O.F16, A, B))
+    assert r["max_rel"] <= 1e-2 and r["fro_rel"] <= 1e-2, r
