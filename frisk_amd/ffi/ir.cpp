@@ -108,6 +108,12 @@ static void print_diagnostics(const Diagnostics& d) {
 
 template <class OpClass> static void def_common(py::class_<OpClass, OpState>&) {}
 
+// an affine expression typed by its kind, as the reference's dyn_casts return (ffi/ir.cpp:811-858)
+struct AffineBinaryOpExpr : AffineExpr { explicit AffineBinaryOpExpr(const AffineExpr& e) : AffineExpr(e) {} };
+struct AffineDimExpr : AffineExpr { explicit AffineDimExpr(const AffineExpr& e) : AffineExpr(e) {} };
+struct AffineSymbolExpr : AffineExpr { explicit AffineSymbolExpr(const AffineExpr& e) : AffineExpr(e) {} };
+struct AffineConstantExpr : AffineExpr { explicit AffineConstantExpr(const AffineExpr& e) : AffineExpr(e) {} };
+
 void init_ffi_ir(py::module_&& m) {
   // ---------------------------------------------------------------- context, types, values (ffi/ir.cpp:883-1078)
   py::class_<PyContext>(m, "context", py::module_local())
@@ -120,21 +126,61 @@ void init_ffi_ir(py::module_&& m) {
       .value("LOCAL", MemorySpace::Local)
       .export_values();
 
-  py::class_<AffineExpr>(m, "AffineExpr", py::module_local())  // ffi/ir.cpp:700-810, the arithmetic subset
+  // ---------------------------------------------------------------- affine expressions and maps (ffi/ir.cpp:646-881)
+  py::enum_<ExprKind>(m, "AffineExprKind", py::module_local())  // values and order of mlir::AffineExprKind
+      .value("Add", ExprKind::Add)
+      .value("Mul", ExprKind::Mul)
+      .value("Mod", ExprKind::Mod)
+      .value("FloorDiv", ExprKind::FloorDiv)
+      .value("CeilDiv", ExprKind::CeilDiv)
+      .value("LAST_AFFINE_BINARY_OP", ExprKind::CeilDiv)
+      .value("Constant", ExprKind::Constant)
+      .value("DimId", ExprKind::DimId)
+      .value("SymbolId", ExprKind::SymbolId)
+      .export_values();
+
+  auto require_binary_kind = [](ExprKind k) {
+    if ((int)k < 0 || (int)k > (int)ExprKind::CeilDiv) throw std::invalid_argument("not a binary affine expression kind");
+  };
+
+  py::class_<AffineExpr>(m, "AffineExpr", py::module_local())  // ffi/ir.cpp:760-858
       .def(py::init<>())
       .def("__eq__", [](const AffineExpr& a, const AffineExpr& b) { return a.equals(b); })
       .def("__eq__", [](const AffineExpr& a, int64_t v) { return a.is_constant() && a.constant_value() == v; })
       .def("__ne__", [](const AffineExpr& a, const AffineExpr& b) { return !a.equals(b); })
+      .def("__ne__", [](const AffineExpr& a, int64_t v) { return !(a.is_constant() && a.constant_value() == v); })
       .def("__bool__", [](const AffineExpr& a) { return (bool)a; })
+      .def("__nonzero__", [](const AffineExpr& a) { return (bool)a; })
+      .def("__hash__", [](const AffineExpr& a) { return std::hash<std::string>()(a.str()); })
       .def("__str__", [](const AffineExpr& a) { return a.str(); })
-      .def("__repr__", [](const AffineExpr& a) { return a.str(); })
-      .def("get_kind", [](const AffineExpr& a) { return (int)a.kind(); })
+      .def("__repr__", [](const AffineExpr& a) { return "AffineExpr(" + a.str() + ")"; })
+      .def("get_kind", [](const AffineExpr& a) { return a.kind(); })
+      .def("is_symbolic_or_constant", &AffineExpr::is_symbolic_or_constant)
+      .def("is_pure_affine", &AffineExpr::is_pure_affine)
+      .def("get_largest_known_divisor", &AffineExpr::largest_known_divisor)
+      .def("is_multiple_of", &AffineExpr::is_multiple_of)
+      .def("is_function_of_dim", [](const AffineExpr& a, unsigned p) { return a.is_function_of(ExprKind::DimId, p); })
+      .def("is_function_of_symbol", [](const AffineExpr& a, unsigned p) { return a.is_function_of(ExprKind::SymbolId, p); })
+      .def("replace_dims_and_symbols", &AffineExpr::replace_dims_and_symbols)
+      .def("replace_dims", [](const AffineExpr& a, std::vector<AffineExpr> dims) { return a.replace_dims_and_symbols(dims, {}); })
+      .def("replace_symbols", [](const AffineExpr& a, std::vector<AffineExpr> syms) { return a.replace_dims_and_symbols({}, syms); })
+      .def("replace", &AffineExpr::replace)
+      .def("replace_with_map", [](const AffineExpr& a, std::vector<std::pair<AffineExpr, AffineExpr>> pairs) {
+        AffineExpr out = a;
+        for (auto& p : pairs) out = out.replace(p.first, p.second);
+        return out;
+      })
+      .def("shift_dims", [](const AffineExpr& a, unsigned, unsigned shift, unsigned offset) { return a.shift(ExprKind::DimId, shift, offset); },
+           py::arg("num_dims"), py::arg("shift"), py::arg("offset") = 0)
+      .def("shift_symbols", [](const AffineExpr& a, unsigned, unsigned shift, unsigned offset) { return a.shift(ExprKind::SymbolId, shift, offset); },
+           py::arg("num_symbols"), py::arg("shift"), py::arg("offset") = 0)
       .def("__add__", [](const AffineExpr& a, int64_t v) { return a + v; })
       .def("__add__", [](const AffineExpr& a, const AffineExpr& b) { return a + b; })
       .def("__radd__", [](const AffineExpr& a, int64_t v) { return a + v; })
       .def("__neg__", [](const AffineExpr& a) { return -a; })
       .def("__sub__", [](const AffineExpr& a, int64_t v) { return a - v; })
       .def("__sub__", [](const AffineExpr& a, const AffineExpr& b) { return a - b; })
+      .def("__rsub__", [](const AffineExpr& a, int64_t v) { return AffineExpr::constant(v) - a; })
       .def("__mul__", [](const AffineExpr& a, int64_t v) { return a * v; })
       .def("__mul__", [](const AffineExpr& a, const AffineExpr& b) { return a * b; })
       .def("__rmul__", [](const AffineExpr& a, int64_t v) { return a * v; })
@@ -144,28 +190,136 @@ void init_ffi_ir(py::module_&& m) {
       .def("ceil_div", [](const AffineExpr& a, const AffineExpr& b) { return a.ceil_div(b); })
       .def("__mod__", [](const AffineExpr& a, int64_t v) { return a.mod(AffineExpr::constant(v)); })
       .def("__mod__", [](const AffineExpr& a, const AffineExpr& b) { return a.mod(b); })
+      .def("__floordiv__", [](const AffineExpr& a, int64_t v) { return a.floor_div(AffineExpr::constant(v)); })  // not in the reference: `//` for floor_div
+      .def("__floordiv__", [](const AffineExpr& a, const AffineExpr& b) { return a.floor_div(b); })
+      .def("compose", [](const AffineExpr& a, const AffineMap& map) {  // dims of the expression := results of the map
+        return a.replace_dims_and_symbols(map.impl ? map.impl->results : std::vector<AffineExpr>(), {});
+      })
+      // the dyn_casts of the reference: the same expression typed by its kind, or None
+      .def("as_binary", [](const AffineExpr& a) -> py::object { return a.is_binary() ? py::cast(AffineBinaryOpExpr(a)) : py::none(); })
+      .def("as_dim", [](const AffineExpr& a) -> py::object { return a.kind() == ExprKind::DimId ? py::cast(AffineDimExpr(a)) : py::none(); })
+      .def("as_symbol", [](const AffineExpr& a) -> py::object { return a.kind() == ExprKind::SymbolId ? py::cast(AffineSymbolExpr(a)) : py::none(); })
+      .def("as_constant", [](const AffineExpr& a) -> py::object { return a.is_constant() ? py::cast(AffineConstantExpr(a)) : py::none(); })
       .def("evaluate", [](const AffineExpr& a, std::vector<int64_t> dims, std::vector<int64_t> syms) { return a.eval(dims, syms); },
            py::arg("dims"), py::arg("symbols") = std::vector<int64_t>());
 
-  py::class_<AffineMap>(m, "AffineMap", py::module_local())  // ffi/ir.cpp:646-699
+  py::class_<AffineBinaryOpExpr, AffineExpr>(m, "AffineBinaryOpExpr", py::module_local())
+      .def("get_lhs", [](const AffineBinaryOpExpr& a) { return a.lhs(); })
+      .def("get_rhs", [](const AffineBinaryOpExpr& a) { return a.rhs(); });
+  py::class_<AffineDimExpr, AffineExpr>(m, "AffineDimExpr", py::module_local()).def("get_position", [](const AffineDimExpr& a) { return a.impl->value; });
+  py::class_<AffineSymbolExpr, AffineExpr>(m, "AffineSymbolExpr", py::module_local()).def("get_position", [](const AffineSymbolExpr& a) { return a.impl->value; });
+  py::class_<AffineConstantExpr, AffineExpr>(m, "AffineConstantExpr", py::module_local()).def("get_value", [](const AffineConstantExpr& a) { return a.impl->value; });
+
+  m.def("get_affine_dim_expr", [](unsigned p, PyContext*) { return AffineExpr::dim(p); }, py::arg("position"), py::arg("context") = nullptr);
+  m.def("get_affine_symbol_expr", [](unsigned p, PyContext*) { return AffineExpr::symbol(p); }, py::arg("position"), py::arg("context") = nullptr);
+  m.def("get_affine_constant_expr", [](int64_t v, PyContext*) { return AffineExpr::constant(v); }, py::arg("constant"), py::arg("context") = nullptr);
+  m.def("get_affine_constant_exprs", [](std::vector<int64_t> vs, PyContext*) {
+    std::vector<AffineExpr> out;
+    for (int64_t v : vs) out.push_back(AffineExpr::constant(v));
+    return out;
+  }, py::arg("constants"), py::arg("context") = nullptr);
+  m.def("get_affine_binary_op_expr", [require_binary_kind](ExprKind k, AffineExpr l, AffineExpr r) { require_binary_kind(k); return AffineExpr::binary(k, l, r); });
+  // sum over dims, then symbols, of coefficient * variable, plus the trailing constant (local expressions are not supported)
+  m.def("get_affine_expr_from_flat_form", [](std::vector<int64_t> flat, unsigned num_dims, unsigned num_symbols, std::vector<AffineExpr> locals, PyContext*) {
+    if (flat.size() != (size_t)num_dims + num_symbols + locals.size() + 1) throw std::invalid_argument("flat form must hold one coefficient per dim, symbol and local, and a constant");
+    AffineExpr e = AffineExpr::constant(0);
+    for (unsigned i = 0; i < num_dims + num_symbols + locals.size(); ++i) {
+      if (flat[i] == 0) continue;
+      AffineExpr v = i < num_dims ? AffineExpr::dim(i) : (i < num_dims + num_symbols ? AffineExpr::symbol(i - num_dims) : locals[i - num_dims - num_symbols]);
+      e = e + v * flat[i];
+    }
+    return e + flat.back();
+  }, py::arg("flat_exprs"), py::arg("num_dims"), py::arg("num_symbols"), py::arg("local_exprs") = std::vector<AffineExpr>(), py::arg("context") = nullptr);
+  m.def("simplify_affine_expr", [](const AffineExpr& e, unsigned, unsigned) { return e.simplified(); }, py::arg("expr"), py::arg("num_dims") = 0,
+        py::arg("num_symbols") = 0);
+
+  py::class_<AffineMap>(m, "AffineMap", py::module_local())  // ffi/ir.cpp:646-757
       .def(py::init<>())
+      .def_static("get", [](PyContext*) { return AffineMap(0, 0, {}); })
+      .def_static("get", [](unsigned dims, unsigned syms, PyContext*) { return AffineMap((int)dims, (int)syms, {}); })
       .def_static("get", [](unsigned dims, unsigned syms, AffineExpr result) { return AffineMap((int)dims, (int)syms, {result}); })
       .def_static("get", [](unsigned dims, unsigned syms, std::vector<AffineExpr> results, PyContext*) { return AffineMap((int)dims, (int)syms, results); },
                   py::arg("dim_count"), py::arg("symbol_count"), py::arg("results"), py::arg("context") = nullptr)
+      .def_static("get_constant_map", [](int64_t v, PyContext*) { return AffineMap(0, 0, {AffineExpr::constant(v)}); }, py::arg("value"),
+                  py::arg("context") = nullptr)
       .def_static("get_multi_dim_identity_map", [](unsigned n, PyContext*) { return AffineMap::identity((int)n); }, py::arg("num_dims"),
                   py::arg("context") = nullptr)
+      .def_static("get_multi_dim_map_with_targets", [](unsigned n, PyContext*) { return AffineMap::identity((int)n); }, py::arg("num_dims"),
+                  py::arg("context") = nullptr)
+      .def_static("get_minor_identity_map", [](unsigned dims, unsigned results, PyContext*) {
+        if (results > dims) throw std::invalid_argument("a minor identity map cannot have more results than dims");
+        std::vector<AffineExpr> r;
+        for (unsigned i = dims - results; i < dims; ++i) r.push_back(AffineExpr::dim(i));
+        return AffineMap((int)dims, 0, r);
+      }, py::arg("dims"), py::arg("results"), py::arg("context") = nullptr)
+      .def_static("get_permutation_map", [](std::vector<int64_t> perm, PyContext*) {
+        std::vector<bool> seen(perm.size(), false);
+        std::vector<AffineExpr> r;
+        for (int64_t p : perm) {
+          if (p < 0 || (size_t)p >= perm.size() || seen[(size_t)p]) throw std::invalid_argument("not a permutation");
+          seen[(size_t)p] = true;
+          r.push_back(AffineExpr::dim(p));
+        }
+        return AffineMap((int)perm.size(), 0, r);
+      }, py::arg("permutation"), py::arg("context") = nullptr)
       .def("__eq__", [](const AffineMap& a, const AffineMap& b) { return a.equals(b); })
       .def("__ne__", [](const AffineMap& a, const AffineMap& b) { return !a.equals(b); })
       .def("__bool__", [](const AffineMap& a) { return (bool)a; })
+      .def("__nonzero__", [](const AffineMap& a) { return (bool)a; })
       .def("__str__", [](const AffineMap& a) { return a.str(); })
-      .def("__repr__", [](const AffineMap& a) { return a.str(); })
+      .def("__repr__", [](const AffineMap& a) { return "AffineMap(" + a.str() + ")"; })
       .def("get_num_dims", &AffineMap::num_dims)
       .def("get_num_symbols", &AffineMap::num_symbols)
       .def("get_num_results", &AffineMap::num_results)
       .def("get_num_inputs", &AffineMap::num_inputs)
       .def("get_results", [](const AffineMap& a) { return a.impl ? a.impl->results : std::vector<AffineExpr>(); })
       .def("get_result", [](const AffineMap& a, unsigned i) { return a.impl->results.at(i); })
-      .def("is_identity", &AffineMap::is_identity);
+      .def("is_identity", &AffineMap::is_identity)
+      .def("is_symbol_identity", [](const AffineMap& a) {
+        if (!a.impl || a.num_symbols() != a.num_results()) return false;
+        for (int i = 0; i < a.num_results(); ++i)
+          if (a.impl->results[(size_t)i].kind() != ExprKind::SymbolId || a.impl->results[(size_t)i].impl->value != i) return false;
+        return true;
+      })
+      .def("is_minor_identity", [](const AffineMap& a) {
+        if (!a.impl || a.num_symbols() || a.num_results() > a.num_dims()) return false;
+        int first = a.num_dims() - a.num_results();
+        for (int i = 0; i < a.num_results(); ++i)
+          if (a.impl->results[(size_t)i].kind() != ExprKind::DimId || a.impl->results[(size_t)i].impl->value != first + i) return false;
+        return true;
+      })
+      .def("is_empty", [](const AffineMap& a) { return a.num_dims() == 0 && a.num_symbols() == 0 && a.num_results() == 0; })
+      .def("is_single_constant", [](const AffineMap& a) { return a.num_results() == 1 && a.impl->results[0].is_constant(); })
+      .def("is_constant", [](const AffineMap& a) {
+        if (!a.impl) return false;
+        for (auto& e : a.impl->results) if (!e.is_constant()) return false;
+        return true;
+      })
+      .def("is_permutation", [](const AffineMap& a) { return a.num_dims() == a.num_results() && a.is_projected_permutation(false); })
+      .def("is_projected_permutation", &AffineMap::is_projected_permutation, py::arg("allow_zero_in_results") = false)
+      .def("get_single_constant_result", [](const AffineMap& a) {
+        if (a.num_results() != 1 || !a.impl->results[0].is_constant()) throw std::invalid_argument("map does not have a single constant result");
+        return a.impl->results[0].constant_value();
+      })
+      .def("get_constant_results", [](const AffineMap& a) {
+        std::vector<int64_t> out;
+        if (a.impl) for (auto& e : a.impl->results) {
+          if (!e.is_constant()) throw std::invalid_argument("map has a non-constant result");
+          out.push_back(e.constant_value());
+        }
+        return out;
+      })
+      .def("get_dim_position", [](const AffineMap& a, unsigned idx) {
+        const AffineExpr& e = a.impl->results.at(idx);
+        if (e.kind() != ExprKind::DimId) throw std::invalid_argument("result is not a dimension");
+        return e.impl->value;
+      }, py::arg("idx"))
+      .def("get_result_position", [](const AffineMap& a, const AffineExpr& input) -> py::object {
+        if (input.kind() != ExprKind::DimId || !a.impl) return py::none();
+        for (size_t i = 0; i < a.impl->results.size(); ++i)
+          if (a.impl->results[i].equals(input)) return py::cast((unsigned)i);
+        return py::none();
+      }, py::arg("input"));
 
   py::class_<Type>(m, "type", py::module_local())  // ffi/ir.cpp:888-937
       .def("__str__", [](const Type& t) { return t.str(); })

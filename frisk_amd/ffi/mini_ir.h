@@ -67,6 +67,14 @@ struct AffineExpr {
     return AffineExpr(impl->lhs).equals(AffineExpr(o.impl->lhs)) && AffineExpr(impl->rhs).equals(AffineExpr(o.impl->rhs));
   }
   static int64_t floordiv(int64_t a, int64_t b) { int64_t q = a / b; return (a % b != 0 && ((a < 0) != (b < 0))) ? q - 1 : q; }
+  static AffineExpr raw(ExprKind k, const AffineExpr& l, const AffineExpr& r) {
+    return AffineExpr(std::make_shared<AffineExprImpl>(AffineExprImpl{k, 0, l.impl, r.impl}));
+  }
+  bool is_kind_with_const_rhs(ExprKind k) const { return kind() == k && AffineExpr(impl->rhs).is_constant(); }
+  // The folding constructor: the simplifications MLIR applies when an affine expression is built (constant folding,
+  // constants and symbolic operands to the right, merged constants and coefficients, "e - q * (e floordiv q)" = "e mod q",
+  // divisions and remainders of known multiples), so that expressions built the way the reference builds its layouts
+  // print the way the reference's logs show them.
   static AffineExpr binary(ExprKind k, AffineExpr l, AffineExpr r) {
     if (!l || !r) throw std::invalid_argument("affine expression operand is null");
     if (l.is_constant() && r.is_constant()) {
@@ -80,17 +88,79 @@ struct AffineExpr {
         default: break;
       }
     }
-    // canonical position of the constant: right-hand side (as MLIR does)
-    if ((k == ExprKind::Add || k == ExprKind::Mul) && l.is_constant()) std::swap(l, r);
-    if (r.is_constant()) {
-      int64_t c = r.constant_value();
-      if (k == ExprKind::Add && c == 0) return l;
-      if (k == ExprKind::Mul && c == 1) return l;
-      if (k == ExprKind::Mul && c == 0) return constant(0);
-      if ((k == ExprKind::FloorDiv || k == ExprKind::CeilDiv) && c == 1) return l;
-      if (k == ExprKind::Mod && c == 1) return constant(0);
+    switch (k) {
+      case ExprKind::Add: return make_add(l, r);
+      case ExprKind::Mul: return make_mul(l, r);
+      case ExprKind::Mod: return make_mod(l, r);
+      case ExprKind::FloorDiv: return make_div(ExprKind::FloorDiv, l, r);
+      case ExprKind::CeilDiv: return make_div(ExprKind::CeilDiv, l, r);
+      default: throw std::invalid_argument("not a binary affine expression kind");
     }
-    return AffineExpr(std::make_shared<AffineExprImpl>(AffineExprImpl{k, 0, l.impl, r.impl}));
+  }
+  static AffineExpr make_add(AffineExpr l, AffineExpr r) {
+    // constants, then symbolic expressions, go to the right
+    if (l.is_constant() || (l.is_symbolic_or_constant() && !r.is_symbolic_or_constant())) return binary(ExprKind::Add, r, l);
+    if (r.is_constant()) {
+      if (r.constant_value() == 0) return l;
+      if (l.is_kind_with_const_rhs(ExprKind::Add)) return binary(ExprKind::Add, l.lhs(), constant(l.rhs().constant_value() + r.constant_value()));
+    }
+    // c1 * e + c2 * e = (c1 + c2) * e
+    {
+      int64_t cl = 1, cr = 1;
+      AffineExpr bl = l, br = r;
+      if (l.is_kind_with_const_rhs(ExprKind::Mul)) { cl = l.rhs().constant_value(); bl = l.lhs(); }
+      if (r.is_kind_with_const_rhs(ExprKind::Mul)) { cr = r.rhs().constant_value(); br = r.lhs(); }
+      if (bl.equals(br)) return binary(ExprKind::Mul, bl, constant(cl + cr));
+    }
+    // (e + c) + f = (e + f) + c
+    if (l.is_kind_with_const_rhs(ExprKind::Add)) return binary(ExprKind::Add, binary(ExprKind::Add, l.lhs(), r), l.rhs());
+    // e + (e floordiv q) * -q = e mod q, also in the form e + (q * (e floordiv q)) * -1
+    if (r.is_kind_with_const_rhs(ExprKind::Mul)) {
+      AffineExpr inner = r.lhs();
+      int64_t c = r.rhs().constant_value();
+      if (c == -1 && inner.is_kind_with_const_rhs(ExprKind::Mul)) { c = -inner.rhs().constant_value(); inner = inner.lhs(); }
+      if (c < 0 && inner.is_kind_with_const_rhs(ExprKind::FloorDiv) && inner.rhs().constant_value() == -c && inner.lhs().equals(l))
+        return binary(ExprKind::Mod, l, constant(-c));
+    }
+    return raw(ExprKind::Add, l, r);
+  }
+  static AffineExpr make_mul(AffineExpr l, AffineExpr r) {
+    // the constant or symbolic factor goes to the right
+    if (l.is_constant() || (!r.is_symbolic_or_constant() && l.is_symbolic_or_constant())) return binary(ExprKind::Mul, r, l);
+    if (r.is_constant()) {
+      if (r.constant_value() == 1) return l;
+      if (r.constant_value() == 0) return constant(0);
+      if (l.is_kind_with_const_rhs(ExprKind::Mul)) return binary(ExprKind::Mul, l.lhs(), constant(l.rhs().constant_value() * r.constant_value()));
+    }
+    // (e * c) * f = (e * f) * c
+    if (l.is_kind_with_const_rhs(ExprKind::Mul)) return binary(ExprKind::Mul, binary(ExprKind::Mul, l.lhs(), r), l.rhs());
+    return raw(ExprKind::Mul, l, r);
+  }
+  static AffineExpr make_div(ExprKind k, const AffineExpr& l, const AffineExpr& r) {
+    if (r.is_constant() && r.constant_value() >= 1) {
+      const int64_t q = r.constant_value();
+      if (q == 1) return l;
+      // (e * c) div q with q | c
+      if (l.is_kind_with_const_rhs(ExprKind::Mul) && l.rhs().constant_value() % q == 0) return binary(ExprKind::Mul, l.lhs(), constant(l.rhs().constant_value() / q));
+      // (a + b) floordiv q with q | a or q | b splits
+      if (k == ExprKind::FloorDiv && l.kind() == ExprKind::Add &&
+          (l.lhs().largest_known_divisor() % q == 0 || l.rhs().largest_known_divisor() % q == 0))
+        return binary(ExprKind::Add, binary(k, l.lhs(), r), binary(k, l.rhs(), r));
+    }
+    return raw(k, l, r);
+  }
+  static AffineExpr make_mod(const AffineExpr& l, const AffineExpr& r) {
+    if (r.is_constant() && r.constant_value() >= 1) {
+      const int64_t q = r.constant_value();
+      if (l.largest_known_divisor() % q == 0) return constant(0);
+      if (l.kind() == ExprKind::Add) {
+        if (l.lhs().largest_known_divisor() % q == 0) return binary(ExprKind::Mod, l.rhs(), r);
+        if (l.rhs().largest_known_divisor() % q == 0) return binary(ExprKind::Mod, l.lhs(), r);
+      }
+      // (e mod c) mod q with q | c
+      if (l.is_kind_with_const_rhs(ExprKind::Mod) && l.rhs().constant_value() >= 1 && l.rhs().constant_value() % q == 0) return binary(ExprKind::Mod, l.lhs(), r);
+    }
+    return raw(ExprKind::Mod, l, r);
   }
   AffineExpr operator+(const AffineExpr& o) const { return binary(ExprKind::Add, *this, o); }
   AffineExpr operator+(int64_t v) const { return *this + constant(v); }
@@ -120,6 +190,84 @@ struct AffineExpr {
       default: throw std::invalid_argument("cannot evaluate a null affine expression");
     }
   }
+  // ---- analysis and rewriting, following the documented behaviour of mlir::AffineExpr
+  AffineExpr lhs() const { return AffineExpr(impl->lhs); }
+  AffineExpr rhs() const { return AffineExpr(impl->rhs); }
+  bool is_binary() const { return impl && (int)impl->kind <= (int)ExprKind::CeilDiv && (int)impl->kind >= 0; }
+  bool is_symbolic_or_constant() const {
+    switch (kind()) {
+      case ExprKind::Constant: case ExprKind::SymbolId: return true;
+      case ExprKind::DimId: case ExprKind::Null: return false;
+      default: return lhs().is_symbolic_or_constant() && rhs().is_symbolic_or_constant();
+    }
+  }
+  bool is_pure_affine() const {
+    switch (kind()) {
+      case ExprKind::Constant: case ExprKind::SymbolId: case ExprKind::DimId: return true;
+      case ExprKind::Null: return false;
+      case ExprKind::Add: return lhs().is_pure_affine() && rhs().is_pure_affine();
+      case ExprKind::Mul: return lhs().is_pure_affine() && rhs().is_pure_affine() && (lhs().is_constant() || rhs().is_constant());
+      default: return lhs().is_pure_affine() && rhs().is_constant();  // mod, floordiv, ceildiv by a constant
+    }
+  }
+  static int64_t gcd(int64_t a, int64_t b) { a = a < 0 ? -a : a; b = b < 0 ? -b : b; while (b) { int64_t t = a % b; a = b; b = t; } return a; }
+  int64_t largest_known_divisor() const {
+    switch (kind()) {
+      case ExprKind::Constant: return impl->value < 0 ? -impl->value : impl->value;
+      case ExprKind::DimId: case ExprKind::SymbolId: case ExprKind::Null: return 1;
+      case ExprKind::Mul: return lhs().largest_known_divisor() * rhs().largest_known_divisor();
+      case ExprKind::Add: case ExprKind::Mod: return gcd(lhs().largest_known_divisor(), rhs().largest_known_divisor());
+      default: {  // floordiv, ceildiv: exact only when the constant divisor divides what is known of the dividend
+        if (rhs().is_constant() && rhs().constant_value() != 0) {
+          int64_t l = lhs().largest_known_divisor(), r = rhs().constant_value();
+          if (l % r == 0) return l / r < 0 ? -(l / r) : l / r;
+        }
+        return 1;
+      }
+    }
+  }
+  bool is_multiple_of(int64_t factor) const {
+    if (factor == 0) return false;
+    switch (kind()) {
+      case ExprKind::Constant: return impl->value % factor == 0;
+      case ExprKind::DimId: case ExprKind::SymbolId: return factor * factor == 1;
+      case ExprKind::Null: return false;
+      case ExprKind::Mul: {
+        int64_t l = lhs().largest_known_divisor();
+        return l % factor == 0 || rhs().largest_known_divisor() % factor == 0 || (l * rhs().largest_known_divisor()) % factor == 0;
+      }
+      default: return largest_known_divisor() % factor == 0;
+    }
+  }
+  bool is_function_of(ExprKind leaf, int64_t position) const {
+    if (kind() == leaf) return impl->value == position;
+    if (!is_binary()) return false;
+    return lhs().is_function_of(leaf, position) || rhs().is_function_of(leaf, position);
+  }
+  // dims / symbols with a replacement in the lists are substituted; the others stay
+  AffineExpr replace_dims_and_symbols(const std::vector<AffineExpr>& dims, const std::vector<AffineExpr>& syms) const {
+    switch (kind()) {
+      case ExprKind::Constant: case ExprKind::Null: return *this;
+      case ExprKind::DimId: return (size_t)impl->value < dims.size() ? dims[(size_t)impl->value] : *this;
+      case ExprKind::SymbolId: return (size_t)impl->value < syms.size() ? syms[(size_t)impl->value] : *this;
+      default: return binary(kind(), lhs().replace_dims_and_symbols(dims, syms), rhs().replace_dims_and_symbols(dims, syms));
+    }
+  }
+  AffineExpr replace(const AffineExpr& target, const AffineExpr& with) const {
+    if (equals(target)) return with;
+    if (!is_binary()) return *this;
+    return binary(kind(), lhs().replace(target, with), rhs().replace(target, with));
+  }
+  AffineExpr shift(ExprKind leaf, int64_t shift_by, int64_t offset) const {
+    if (kind() == leaf) return impl->value >= offset ? (leaf == ExprKind::DimId ? dim(impl->value + shift_by) : symbol(impl->value + shift_by)) : *this;
+    if (!is_binary()) return *this;
+    return binary(kind(), lhs().shift(leaf, shift_by, offset), rhs().shift(leaf, shift_by, offset));
+  }
+  AffineExpr simplified() const {  // rebuild bottom-up through the folding constructor
+    if (!is_binary()) return *this;
+    return binary(kind(), lhs().simplified(), rhs().simplified());
+  }
+
   // MLIR's spelling; `names` substitutes SSA names for dims (then symbols) when given
   std::string str(const std::vector<std::string>* names = nullptr, int num_dims = 0, bool nested = false) const {
     switch (kind()) {
@@ -174,6 +322,21 @@ struct AffineMap {
     if (!impl || impl->num_symbols || num_results() != num_dims()) return false;
     for (int i = 0; i < num_results(); ++i)
       if (impl->results[i].kind() != ExprKind::DimId || impl->results[i].impl->value != i) return false;
+    return true;
+  }
+  // every result a distinct dim (or, if allowed, the constant 0), no symbols
+  bool is_projected_permutation(bool allow_zero_in_results) const {
+    if (!impl || impl->num_symbols) return false;
+    if (num_results() > num_dims() && !allow_zero_in_results) return false;
+    std::vector<bool> seen((size_t)num_dims(), false);
+    for (const AffineExpr& e : impl->results) {
+      if (e.kind() == ExprKind::DimId) {
+        if (e.impl->value >= num_dims() || seen[(size_t)e.impl->value]) return false;
+        seen[(size_t)e.impl->value] = true;
+      } else if (!(allow_zero_in_results && e.is_constant() && e.constant_value() == 0)) {
+        return false;
+      }
+    }
     return true;
   }
   bool equals(const AffineMap& o) const {
