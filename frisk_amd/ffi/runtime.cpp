@@ -131,6 +131,24 @@ std::string lds_layout_debug(const frisk_lds_layout& L, int elem_bytes) {
   return "Layout(shape=[" + std::to_string(L.rows) + ", " + std::to_string(cols) + "], index=affine_map<" + map.str() + ">)";
 }
 
+// Accumulator fragment of a work-group tile in the same debug form: Fragment(shape, index, thread, replicate).
+// A wave owns a (BM / WM) x (BN / WN) block as 32x32 MFMA atoms kept transposed: inside an atom, element (m, n)
+// lives in lane (m mod 32) + 32 * ((n mod 8) floordiv 4), accumulator register (n mod 4) + 4 * ((n mod 32) floordiv 8).
+std::string accumulator_layout_debug(int64_t bm, int64_t bn, int64_t wm, int64_t wn) {
+  if (wm <= 0 || wn <= 0 || bm % (wm * 32) || bn % (wn * 32)) throw std::invalid_argument("the wave grid must split the tile into whole 32x32 atoms");
+  const int64_t wtm = bm / wm, wtn = bn / wn, an = wtn / 32;
+  auto c = [](int64_t v) { return AffineExpr::constant(v); };
+  AffineExpr i = AffineExpr::dim(0), j = AffineExpr::dim(1);
+  AffineExpr lane = i.mod(c(32)) + j.mod(c(8)).floor_div(c(4)) * 32;
+  AffineExpr wave = i.floor_div(c(wtm)) * wn + j.floor_div(c(wtn));
+  AffineExpr thread = lane + wave * 64;
+  AffineExpr reg = j.mod(c(4)) + j.mod(c(32)).floor_div(c(8)) * 4;
+  AffineExpr atom = i.mod(c(wtm)).floor_div(c(32)) * an + j.mod(c(wtn)).floor_div(c(32));
+  AffineExpr index = reg + atom * 16;
+  return "Fragment(shape=[" + std::to_string(bm) + ", " + std::to_string(bn) + "], index=affine_map<" + AffineMap(2, 0, {index}).str() +
+         ">, thread=affine_map<" + AffineMap(2, 0, {thread}).str() + ">, replicate=1)";
+}
+
 py::dict program_dict(const GemmProgram& g) {
   py::dict d;
   d["kernel"] = g.kernel_name;
@@ -200,6 +218,16 @@ void init_ffi_runtime(py::module_&& m) {
     out["bytes"] = p.bytes;
     return out;
   }, py::arg("kernel"), py::arg("module") = py::none(), py::arg("epilogue") = "none");
+
+  m.def("lds_layout_string", [](int rows, int row_bytes, int elem_bytes, int row_shift, int row_mask, int chunk_shift) {
+    frisk_lds_layout L{};
+    L.rows = rows; L.row_bytes = row_bytes; L.row_shift = row_shift; L.row_mask = row_mask; L.chunk_shift = chunk_shift;
+    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) throw std::invalid_argument("element size must be 1, 2 or 4 bytes");
+    return lds_layout_debug(L, elem_bytes);
+  }, py::arg("rows"), py::arg("row_bytes"), py::arg("elem_bytes"), py::arg("row_shift"), py::arg("row_mask"), py::arg("chunk_shift"),
+     "Layout(shape=[...], index=affine_map<...>) of an LDS tile with the XOR swizzle (row_shift, row_mask, chunk_shift); pure host");
+  m.def("accumulator_layout_string", &accumulator_layout_debug, py::arg("tile_m"), py::arg("tile_n"), py::arg("waves_m"), py::arg("waves_n"),
+        "Fragment(shape, index, thread, replicate) of the MFMA accumulators of a work-group tile; pure host");
 
   m.def("match_ops", [](py::object kernel) {
     py::list out;
