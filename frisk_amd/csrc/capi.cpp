@@ -138,6 +138,40 @@ static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, in
   (void)nw;
 }
 
+// Relative time of a problem on a kernel variant, used only to rank the variants.  One wave of work-groups = one per CU
+// (256); a K tile of a 256x256 tile costs 1.5 units when every CU runs one, and less when the chip is partly idle
+// (less contention in the L2 and a higher clock): factor 0.6 + 0.4 * fill.  The constants are measured on fp16 problems
+// between 1024^3 and 8192^3 and carry over to the 8-bit types, whose K tiles hold the same number of bytes.
+static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
+  const int64_t tiles = ((d->M + k->bm - 1) / k->bm) * ((d->N + k->bn - 1) / k->bn);
+  const double kt = (double)((d->K + k->bk - 1) / k->bk);
+  double c;  // cost of one K tile with the chip full
+  const int64_t area = (int64_t)k->bm * k->bn;
+  if (k->dtype == FRISK_F32) {
+    c = area >= 128 * 128 ? 1.93 : (k->bk >= 64 ? 1.0 : 0.55);
+  } else if (k->bm == 32) {
+    c = k->wk > 1 ? 0.8 : 0.25;  // 32x32 with a 4x deeper K tile; 32x128
+  } else if (area >= 256 * 256) {
+    c = k->wm * k->wn > 4 ? 1.56 : (k->stages_b > k->stages ? 1.5 : 1.55);  // 2 + 3 ring < 2 + 2 < 8 waves
+  } else if (area >= 256 * 128) {
+    c = 0.93;
+  } else {
+    // 3 + 3 tiles when the grid is one wave, 2 + 2 (two work-groups per CU) beyond
+    c = k->stages >= 3 ? (tiles <= 256 ? 0.46 : 0.55) : (tiles <= 256 ? 0.55 : 0.52);
+  }
+  if (k->guard) c *= 3.0;
+  const int64_t full = tiles / 256, rest = tiles % 256;
+  const double rest_fill = (double)rest / 256.0;
+  double cost = (double)full * kt * c;
+  if (rest) {
+    if (k->bm == 32)  // the skinny kernels are bound by streaming B and need the parallelism: idle CUs are lost bandwidth
+      cost += full ? kt * c : kt * c / std::max(rest_fill, 0.25);
+    else
+      cost += kt * c * (0.6 + 0.4 * rest_fill);
+  }
+  return cost;
+}
+
 static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_model, bool force_guard = false, bool no_split = false) {
   int st = validate(d);
   if (st != FRISK_OK) return st;
@@ -154,7 +188,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   const bool rows_aligned = (d->lda * es) % 16 == 0 && (d->ldb * es) % 16 == 0 && (d->ldc * os) % 16 == 0;
   const auto& ks = kernels();
   int best = -1;
-  int64_t best_tiles = 0;
+  double best_cost = 0.0;
   bool any_layout = false, tile_requested = d->tile_m || d->tile_n || d->tile_k || d->waves_m || d->waves_n || d->stages;
   for (size_t i = 0; i < ks.size(); ++i) {
     const KernelEntry* k = ks[i];
@@ -168,21 +202,10 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
     if (d->stages && d->stages != k->stages_b) continue;  // the deeper ring names the variant
     // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
     if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
-    if (k->guard && best >= 0 && !ks[best]->guard) continue;  // never prefer a guarded kernel over a fast one that fits
-    int64_t tiles = ((d->M + k->bm - 1) / k->bm) * ((d->N + k->bn - 1) / k->bn);
-    // largest tile that still gives every CU a work-group; otherwise the most work-groups
-    bool better;
-    if (best < 0) better = true;
-    else {
-      const KernelEntry* b = ks[best];
-      if (b->guard && !k->guard) { best = (int)i; best_tiles = tiles; continue; }
-      bool fills = tiles >= 256, bfills = best_tiles >= 256;
-      if (fills != bfills) better = fills;
-      else if (fills && (int64_t)k->bm * k->bn != (int64_t)b->bm * b->bn) better = (int64_t)k->bm * k->bn > (int64_t)b->bm * b->bn;
-      else if (!fills && tiles != best_tiles) better = tiles > best_tiles;
-      else better = false;  // same tile: the first listed variant is the tuned default
-    }
-    if (better) { best = (int)i; best_tiles = tiles; }
+    if (k->guard && best >= 0 && !ks[best]->guard) continue;  // never a guarded kernel when a fast one fits
+    const double cost = estimated_cost(k, d);
+    // ties: the first listed variant is the tuned default
+    if (best < 0 || (ks[best]->guard && !k->guard) || cost < best_cost) { best = (int)i; best_cost = cost; }
   }
   if (d->M == 0 || d->N == 0) {  // nothing to compute
     plan->grid_x = plan->grid_y = 0;

@@ -198,3 +198,22 @@ def test_lds_swizzle_representation_contains_the_reference_bank_swizzles():
         want = (np.broadcast_to(ts, idx.shape) * 8 * cols + idx) * 2  # atoms of 8 rows follow each other
         got = np.array([[R.lds_offset(lay, r, c * 2) for c in range(cols)] for r in range(rows)])
         assert np.array_equal(got, want), (cols, sh, mk, cs)
+
+
+def test_planner_ranks_variants_by_estimated_time():
+    """measured on the device: 2048^3 is fastest on 128x128 tiles with the deep ring (one wave of 256), 3072^3 on 256x256 tiles
+    although they fill only 144 of the 256 CUs, a problem with one 1024 side on 256x128 tiles, the fp8 decode shape on the 32x32
+    kernel whose waves split K, and a guarded kernel is never picked when a fast one fits"""
+    names = R.kernel_names()
+
+    def pick(dt, M, N, K, **kw):
+        return names[R.plan(R.make_desc(dt, M, N, K, dtype_out=R.BF16 if dt == R.E4M3 else None, **kw)).kernel_id]
+    assert pick(R.F16, 2048, 2048, 2048) == "f16_nn_128x128x64_w2x2_s3"
+    assert pick(R.F16, 3072, 3072, 3072) == "f16_nn_256x256x64_w2x2_s2x3"
+    assert pick(R.F16, 4096, 4096, 4096) == "f16_nn_256x256x64_w2x2_s2x3"
+    assert pick(R.BF16, 1024, 8192, 8192, transB=True) == "bf16_nt_256x128x64_w2x2_s3"
+    assert pick(R.F16, 8192, 8192, 8192) == "f16_nn_256x256x64_w2x2_s2x3"
+    assert pick(R.E4M3, 32, 8192, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s4_splitk"
+    assert pick(R.F16, 1024, 1024, 1024) == "f16_nn_32x128x64_w1x4_s3_splitk"
+    assert pick(R.I8, 6144, 6144, 6144) == "i8_nn_256x256x128_w2x2_s2x3"
+    assert not pick(R.F16, 64, 384, 2048).endswith("_guard") and pick(R.F16, 65, 384, 2048).endswith("_guard")
