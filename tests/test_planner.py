@@ -207,7 +207,7 @@ def test_planner_ranks_variants_by_estimated_time():
     names = R.kernel_names()
 
     def pick(dt, M, N, K, **kw):
-        return names[R.plan(R.make_desc(dt, M, N, K, dtype_out=R.BF16 if dt == R.E4M3 else None, **kw)).kernel_id]
+        return names[R.plan(R.make_desc(dt, M, N, K, dtype_out={R.E4M3: R.BF16, R.I8: R.I32}.get(dt), **kw)).kernel_id]
     assert pick(R.F16, 2048, 2048, 2048) == "f16_nn_128x128x64_w2x2_s3"
     assert pick(R.F16, 3072, 3072, 3072) == "f16_nn_256x256x64_w2x2_s2x3"
     assert pick(R.F16, 4096, 4096, 4096) == "f16_nn_256x256x64_w2x2_s2x3"
