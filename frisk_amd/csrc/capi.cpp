@@ -14,6 +14,7 @@
 #include "gemm_internal.h"
 #include "lds_model.h"
 #include "tile_ops.h"
+#include "attention.h"
 
 namespace frisk {
 
@@ -302,6 +303,7 @@ int frisk_hip_init(void) {
   if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
   for (const KernelEntry* k : kernels())
     if (hipError_t e = k->prepare(); e != hipSuccess) return fail(FRISK_ERR_DEVICE, "preparing %s failed: %s", k->name, hipGetErrorString(e));
+  if (hipError_t e = prepare_attention(); e != hipSuccess) return fail(FRISK_ERR_DEVICE, "preparing the attention kernels failed: %s", hipGetErrorString(e));
   return FRISK_OK;
 }
 
@@ -449,6 +451,33 @@ int frisk_hip_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int
   hipError_t e = launch_reduce(dtype, src, rows, cols, ld, dim, kind, clear ? 1 : 0, dst, (float*)workspace, slices, rows_on_16_bytes(dtype, src, ld),
                                (hipStream_t)stream);
   if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "reduce launch failed: %s", hipGetErrorString(e));
+  return FRISK_OK;
+}
+
+int frisk_hip_attention(const frisk_attention_desc* d, const void* Q, const void* K, const void* V, void* O, float* lse, void* stream) {
+  if (!d) return fail(FRISK_ERR_NULL, "attention descriptor is null");
+  if (d->abi_version != FRISK_HIP_ABI_VERSION) return fail(FRISK_ERR_ABI, "descriptor abi_version %d, library %d", d->abi_version, FRISK_HIP_ABI_VERSION);
+  if (d->dtype != FRISK_F16 && d->dtype != FRISK_BF16) return fail(FRISK_ERR_DTYPE, "attention element type %d is not f16 or bf16", d->dtype);
+  if (d->batch < 0 || d->heads < 0 || d->seq_q < 0 || d->seq_k < 0) return fail(FRISK_ERR_SHAPE, "negative extent");
+  if (d->head_dim != kAttnHeadDim) return fail(FRISK_ERR_SHAPE, "head_dim %lld: the attention kernel is built for %d", (long long)d->head_dim, kAttnHeadDim);
+  if (d->seq_q % kAttnQueriesPerGroup) return fail(FRISK_ERR_SHAPE, "seq_q %lld is not a multiple of %d", (long long)d->seq_q, kAttnQueriesPerGroup);
+  if (d->seq_k % kAttnKeysPerTile || d->seq_k == 0) return fail(FRISK_ERR_SHAPE, "seq_k %lld is not a positive multiple of %d", (long long)d->seq_k, kAttnKeysPerTile);
+  if (!(d->scale > 0.f) || !std::isfinite(d->scale)) return fail(FRISK_ERR_ARGUMENT, "softmax scale %g is not a positive finite number", (double)d->scale);
+  const int64_t bh = d->batch * d->heads, groups = bh * (d->seq_q / kAttnQueriesPerGroup);
+  if (d->seq_q > INT32_MAX || d->seq_k > INT32_MAX || bh > INT32_MAX || groups > INT32_MAX) return fail(FRISK_ERR_SHAPE, "extent exceeds 2^31-1");
+  if (groups == 0) return FRISK_OK;
+  if (!Q || !K || !V || !O) return fail(FRISK_ERR_NULL, "attention operand pointer is null");
+  if (((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O) & 15) return fail(FRISK_ERR_ALIGNMENT, "attention operands must be 16-byte aligned");
+  if ((uintptr_t)lse & 3) return fail(FRISK_ERR_ALIGNMENT, "lse must be 4-byte aligned");
+  if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
+  AttentionParams p;
+  p.Q = Q; p.K = K; p.V = V; p.O = O; p.lse = lse;
+  p.batch_heads = (int32_t)bh; p.seq_q = (int32_t)d->seq_q; p.seq_k = (int32_t)d->seq_k;
+  p.q_blocks = (int32_t)(d->seq_q / kAttnQueriesPerGroup);
+  p.xcd_remap = groups % 8 == 0 ? 1 : 0;
+  p.scale_log2 = d->scale * 1.4426950408889634f;
+  hipError_t e = launch_attention(d->dtype, d->k_transposed ? 1 : 0, p, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "attention launch failed: %s", hipGetErrorString(e));
   return FRISK_OK;
 }
 

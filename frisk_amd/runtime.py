@@ -50,6 +50,12 @@ class GemmPlan(ctypes.Structure):
                 ("workspace_bytes", ctypes.c_size_t), ("flops", ctypes.c_double), ("bytes", ctypes.c_double)]
 
 
+class AttentionDesc(ctypes.Structure):
+    _fields_ = [("abi_version", ctypes.c_int32), ("dtype", ctypes.c_int32), ("batch", ctypes.c_int64), ("heads", ctypes.c_int64),
+                ("seq_q", ctypes.c_int64), ("seq_k", ctypes.c_int64), ("head_dim", ctypes.c_int64), ("scale", ctypes.c_float),
+                ("k_transposed", ctypes.c_uint8), ("reserved", ctypes.c_uint8 * 3)]
+
+
 globals().update({name: code for code, name in STATUS_NAMES.items()})  # OK, ERR_NULL, ... as module constants
 
 
@@ -64,7 +70,7 @@ _lib = None
 EXPORTS = ["frisk_hip_init", "frisk_hip_abi_version", "frisk_hip_last_error", "frisk_hip_plan", "frisk_hip_workspace_bytes",
            "frisk_hip_gemm", "frisk_hip_lds_access_cycles", "frisk_hip_lds_search", "frisk_hip_lds_offset", "frisk_hip_wave_partition",
            "frisk_hip_kernel_count", "frisk_hip_kernel_name", "frisk_hip_fill", "frisk_hip_copy", "frisk_hip_reduce",
-           "frisk_hip_reduce_workspace_bytes"]
+           "frisk_hip_reduce_workspace_bytes", "frisk_hip_attention"]
 
 
 def lib():
@@ -98,6 +104,7 @@ def lib():
     L.frisk_hip_copy.argtypes = [ctypes.c_int, vp, i64, ctypes.c_int, vp, i64, i64, i64, vp]
     L.frisk_hip_reduce_workspace_bytes.restype = ctypes.c_size_t
     L.frisk_hip_reduce_workspace_bytes.argtypes = [ctypes.c_int, i64, i64, ctypes.c_int]
+    L.frisk_hip_attention.argtypes = [ctypes.POINTER(AttentionDesc), vp, vp, vp, vp, vp, vp]
     L.frisk_hip_reduce.argtypes = [ctypes.c_int, vp, i64, i64, i64, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, ctypes.c_size_t, vp]
     if L.frisk_hip_abi_version() != ABI_VERSION:
         raise ImportError("libfrisk_hip.so has ABI %d, binding expects %d" % (L.frisk_hip_abi_version(), ABI_VERSION))
@@ -173,6 +180,21 @@ def reduce(dtype, src_ptr, rows, cols, ld, dim, kind, clear, dst_ptr, workspace_
     """frisk.reduce along `dim` with kind "add" | "mul" | "min" | "max" (or its enum value)"""
     k = REDUCE_KINDS[kind] if isinstance(kind, str) else kind
     _check(lib().frisk_hip_reduce(dtype, src_ptr, rows, cols, ld, dim, k, int(bool(clear)), dst_ptr, workspace_ptr, workspace_bytes, stream))
+
+
+def make_attention_desc(dtype, batch, heads, seq_q, seq_k, head_dim=128, scale=None, k_transposed=False):
+    d = AttentionDesc()
+    d.abi_version = ABI_VERSION
+    d.dtype = dtype
+    d.batch, d.heads, d.seq_q, d.seq_k, d.head_dim = batch, heads, seq_q, seq_k, head_dim
+    d.scale = head_dim ** -0.5 if scale is None else scale
+    d.k_transposed = int(bool(k_transposed))
+    return d
+
+
+def attention(desc, Q_ptr, K_ptr, V_ptr, O_ptr, lse_ptr=None, stream=None):
+    """fused softmax(scale * Q K^T) V (asynchronous on `stream`); lse_ptr optionally receives the row log-sum-exp"""
+    _check(lib().frisk_hip_attention(ctypes.byref(desc), Q_ptr, K_ptr, V_ptr, O_ptr, lse_ptr, stream))
 
 
 def wave_partition(policy, tile_m, tile_n, num_waves):

@@ -206,6 +206,32 @@ size_t frisk_hip_reduce_workspace_bytes(int dtype, int64_t rows, int64_t cols, i
 int frisk_hip_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int64_t ld, int dim, int kind, int clear, void* dst,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------------------------------------
+ * Fused attention forward: O = softmax(scale * Q K^T) V per (batch, head), the kernel sketched in the
+ * reference's tmp/ir.mlir:87-157 (frisk.copy Q; frisk.for over key tiles { copy K; gemm; reduce max;
+ * block exp2; reduce sum; block rescale; copy V; gemm }; copy O) executed as one launch with a running
+ * maximum and denominator.  The sketch multiplies scores by a constant and uses exp2
+ * (tmp/ir.mlir:91,114-127): that constant is scale * log2(e) here.
+ * Tensors are dense: Q [batch, heads, seq_q, head_dim], V [batch, heads, seq_k, head_dim],
+ * O like Q, K like V or, with k_transposed = 1, [batch, heads, head_dim, seq_k] (the layout of the sketch's
+ * second argument, tmp/ir.mlir:88).  Products accumulate in fp32; the probabilities are rounded to dtype
+ * before the second product.  Supported: head_dim 128, seq_q a multiple of 256, seq_k a multiple of 64,
+ * 16-byte aligned pointers; anything else is FRISK_ERR_SHAPE / FRISK_ERR_ALIGNMENT.
+ * ------------------------------------------------------------------------------------------------ */
+typedef struct frisk_attention_desc {
+  int32_t abi_version;   /* FRISK_HIP_ABI_VERSION */
+  int32_t dtype;         /* FRISK_F16 or FRISK_BF16: element type of Q, K, V and O */
+  int64_t batch, heads, seq_q, seq_k, head_dim;
+  float scale;           /* > 0; 1/sqrt(head_dim) is the usual choice */
+  uint8_t k_transposed;
+  uint8_t reserved[3];
+} frisk_attention_desc;
+
+/* lse (may be NULL): [batch, heads, seq_q] floats, log(sum_k exp(scale * s_k)) of every query row.
+ * Asynchronous on `stream`; nothing is allocated. */
+int frisk_hip_attention(const frisk_attention_desc* desc, const void* Q, const void* K, const void* V, void* O, float* lse,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif
