@@ -206,6 +206,15 @@ def main():
         ops[name] = {"GB/s": round(moved / (ms * 1e-3) / 1e9, 1), "frac_of_8TB/s": round(moved / (ms * 1e-3) / 8e12, 4), "kernel_ms": round(ms, 5)}
     del src16, dst16
 
+    # fused attention forward at the shape of the reference's sketch: 1 x 32 heads x 4096 x 128, fp16
+    ab, ah, aseq, ad = 1, 32, 4096, 128
+    aq, ak, av = (torch.randn(ab * ah, aseq, ad, device=dev, generator=g).half() for _ in range(3))
+    ao = torch.empty_like(aq)
+    adesc = R.make_attention_desc(R.F16, ab, ah, aseq, aseq, ad)
+    attn_ms = time_op(lambda: R.attention(adesc, aq.data_ptr(), ak.data_ptr(), av.data_ptr(), ao.data_ptr(), None, cs))
+    attn_tflops = 4.0 * ab * ah * aseq * aseq * ad / (attn_ms * 1e-3) / 1e12
+    del aq, ak, av, ao
+
     line = {
         "metric": "GEMM TFLOP/s at 4096^3 fp16 (fp32 accumulate), 1 GPU",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -226,6 +235,10 @@ def main():
                                     "workload": "fp8 e4m3 M=32 N=K=8192 NT, per-tensor scales, bf16 out; algorithmic bytes "
                                                 "|A|+|B|+|C|+scales per launch, B rotating over 6 buffers"},
         "tile_ops_32768x8192_f16": ops,
+        "attention_1x32x4096x128_f16": {"bound": "mfma", "achieved": round(attn_tflops, 2), "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
+                                        "frac": round(attn_tflops / PEAK_TFLOPS["f16"], 4), "kernel_ms": round(attn_ms, 5),
+                                        "workload": "softmax(Q K^T / sqrt(128)) V, 32 heads, 4096 queries x 4096 keys, head_dim 128, "
+                                                    "fp16 in / out, fp32 accumulate; 4 * heads * seq^2 * head_dim flops per launch"},
     }
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(M, N, K)

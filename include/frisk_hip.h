@@ -227,7 +227,8 @@ typedef struct frisk_attention_desc {
   uint8_t reserved[3];
 } frisk_attention_desc;
 
-/* lse (may be NULL): [batch, heads, seq_q] floats, log(sum_k exp(scale * s_k)) of every query row.
+/* lse (may be NULL): [batch, heads, seq_q] floats, log(sum_k exp(scale * s_k)) of every query row, from the
+ * probabilities as rounded for the second product (the denominator the output is normalised by).
  * Asynchronous on `stream`; nothing is allocated. */
 int frisk_hip_attention(const frisk_attention_desc* desc, const void* Q, const void* K, const void* V, void* O, float* lse,
                         void* stream);
