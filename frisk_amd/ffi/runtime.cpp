@@ -12,6 +12,7 @@
 #include "ffi.h"
 #include "frisk_hip.h"
 #include "mini_ir.h"
+#include "layout_infer.h"
 
 namespace frisk_ffi {
 
@@ -132,21 +133,29 @@ std::string lds_layout_debug(const frisk_lds_layout& L, int elem_bytes) {
 }
 
 // Accumulator fragment of a work-group tile in the same debug form: Fragment(shape, index, thread, replicate).
-// A wave owns a (BM / WM) x (BN / WN) block as 32x32 MFMA atoms kept transposed: inside an atom, element (m, n)
-// lives in lane (m mod 32) + 32 * ((n mod 8) floordiv 4), accumulator register (n mod 4) + 4 * ((n mod 32) floordiv 8).
-std::string accumulator_layout_debug(int64_t bm, int64_t bn, int64_t wm, int64_t wn) {
-  if (wm <= 0 || wn <= 0 || bm % (wm * 32) || bn % (wn * 32)) throw std::invalid_argument("the wave grid must split the tile into whole 32x32 atoms");
-  const int64_t wtm = bm / wm, wtn = bn / wn, an = wtn / 32;
-  auto c = [](int64_t v) { return AffineExpr::constant(v); };
-  AffineExpr i = AffineExpr::dim(0), j = AffineExpr::dim(1);
-  AffineExpr lane = i.mod(c(32)) + j.mod(c(8)).floor_div(c(4)) * 32;
-  AffineExpr wave = i.floor_div(c(wtm)) * wn + j.floor_div(c(wtn));
-  AffineExpr thread = lane + wave * 64;
-  AffineExpr reg = j.mod(c(4)) + j.mod(c(32)).floor_div(c(8)) * 4;
-  AffineExpr atom = i.mod(c(wtm)).floor_div(c(32)) * an + j.mod(c(wtn)).floor_div(c(32));
-  AffineExpr index = reg + atom * 16;
-  return "Fragment(shape=[" + std::to_string(bm) + ", " + std::to_string(bn) + "], index=affine_map<" + AffineMap(2, 0, {index}).str() +
-         ">, thread=affine_map<" + AffineMap(2, 0, {thread}).str() + ">, replicate=1)";
+std::string accumulator_layout_debug(int64_t bm, int64_t bn, int64_t wm, int64_t wn) { return accumulator_layout(bm, bn, wm, wn).debug(); }
+
+// LayoutAttr <-> Python: {"shape": [..], "index": AffineMap, "thread": AffineMap or None, "replicate": int or None}; to
+// Python also "debug", the text printLayoutDebug gives.
+py::object layout_to_py(const LayoutAttr& l) {
+  if (!l) return py::none();
+  py::dict d;
+  d["shape"] = l.shape;
+  d["index"] = l.index ? py::cast(l.index) : py::object(py::none());
+  d["thread"] = l.thread ? py::cast(l.thread) : py::object(py::none());
+  d["replicate"] = l.replicate ? py::object(py::int_(*l.replicate)) : py::object(py::none());
+  d["debug"] = l.debug();
+  return std::move(d);
+}
+LayoutAttr layout_from_py(const py::object& o) {
+  if (o.is_none()) return LayoutAttr::none();
+  py::dict d = o.cast<py::dict>();
+  LayoutAttr l;
+  l.shape = d["shape"].cast<std::vector<int64_t>>();
+  if (d.contains("index") && !d["index"].is_none()) l.index = d["index"].cast<AffineMap>();
+  if (d.contains("thread") && !d["thread"].is_none()) l.thread = d["thread"].cast<AffineMap>();
+  if (d.contains("replicate") && !d["replicate"].is_none()) l.replicate = d["replicate"].cast<int64_t>();
+  return l;
 }
 
 py::dict program_dict(const GemmProgram& g) {
@@ -229,6 +238,66 @@ void init_ffi_runtime(py::module_&& m) {
   m.def("accumulator_layout_string", &accumulator_layout_debug, py::arg("tile_m"), py::arg("tile_n"), py::arg("waves_m"), py::arg("waves_n"),
         "Fragment(shape, index, thread, replicate) of the MFMA accumulators of a work-group tile; pure host");
 
+  m.def("accumulator_layout", [](int64_t bm, int64_t bn, int64_t wm, int64_t wn) { return layout_to_py(accumulator_layout(bm, bn, wm, wn)); },
+        py::arg("tile_m"), py::arg("tile_n"), py::arg("waves_m"), py::arg("waves_n"),
+        "layout attribute (shape, index map, thread map, replicate) of the MFMA accumulators of a work-group tile; pure host");
+  m.def("used_extent_for_dim", [](const AffineMap& map, int pos, int64_t extent) -> py::object {
+    auto v = compute_used_extent_for_dim(map, pos, extent);
+    return v ? py::object(py::int_(*v)) : py::object(py::none());
+  }, py::arg("map"), py::arg("dim"), py::arg("extent"),
+        "number of distinct values the map's results take along one dim of the given extent (None: not analysable); pure host");
+  m.def("infer_reduce_layout", [](py::object src, std::vector<int64_t> src_shape, std::vector<int64_t> dst_shape, int64_t dim, int64_t threads,
+                                  py::object existing) {
+    const LayoutAttr have = layout_from_py(existing);
+    return layout_to_py(infer_reduce_layout(layout_from_py(src), src_shape, dst_shape, dim, threads, existing.is_none() ? nullptr : &have));
+  }, py::arg("src"), py::arg("src_shape"), py::arg("dst_shape"), py::arg("dim"), py::arg("threads") = 0, py::arg("existing") = py::none(),
+        "layout of the destination of frisk.reduce from the layout of its source (both in registers); None when the source has no "
+        "index or thread map; ValueError with the op's diagnostic otherwise; pure host");
+  m.def("default_buffer_layout", [](std::vector<int64_t> shape, int element_bits, py::object space, int wave_size, int64_t threads) {
+    return layout_to_py(default_buffer_layout((MemorySpace)py::int_(space).cast<int>(), shape, element_bits, wave_size, threads));
+  }, py::arg("shape"), py::arg("element_bits"), py::arg("space"), py::arg("wave_size") = 64, py::arg("threads") = 1,
+        "default layout of a buffer that no GEMM uses: padded row-major (shared), a lane grid over the last two dims (local), row-major "
+        "(global); one-element buffers are replicated over all threads; pure host");
+  m.def("infer_layouts", [](py::object kernel) {
+    // ParallelOp::inferLayout (lib/Dialect/Frisk/IR/FriskOps.cpp:1040-1092), the part that is not GEMM specific: every
+    // frisk.alloc_buffer under the kernel's frisk.parallel that no frisk.gemm uses gets its default layout; buffers a
+    // GEMM uses are left to the GEMM planner (runtime.plan) and reported with layout None.
+    Operation* k = op_of_handle(kernel);
+    if (!k || k->name != "frisk.kernel" || k->regions.empty() || k->regions[0]->blocks.empty()) throw std::invalid_argument("expected a frisk.kernel with a body");
+    Operation* par = nullptr;
+    for (Operation* op : k->regions[0]->blocks[0]->ops)
+      if (op->name == "frisk.parallel") { par = op; break; }
+    if (!par) throw std::invalid_argument("the kernel has no frisk.parallel");
+    const int64_t threads = par->int_attr("threads");
+    std::vector<Operation*> all;
+    std::function<void(Operation*)> walk = [&](Operation* op) {
+      for (Region* r : op->regions)
+        for (Block* b : r->blocks)
+          for (Operation* inner : b->ops) { all.push_back(inner); walk(inner); }
+    };
+    walk(par);
+    py::list out;
+    int n = 0;
+    for (Operation* op : all) {
+      if (op->name != "frisk.alloc_buffer" || op->results.empty()) continue;
+      ValueImpl* buf = op->results[0];
+      bool gemm_operand = false;
+      for (Operation* user : all)
+        if (user->name == "frisk.gemm")
+          for (const Value& v : user->operands) gemm_operand = gemm_operand || v.impl == buf;
+      const Type t = buf->type;
+      py::dict d;
+      d["buffer"] = n++;
+      d["shape"] = t.impl->shape;
+      d["memory_space"] = (int)op->int_attr("memory_space");
+      d["used_by_gemm"] = gemm_operand;
+      d["layout"] = gemm_operand ? py::object(py::none())
+                                 : layout_to_py(default_buffer_layout((MemorySpace)op->int_attr("memory_space"), t.impl->shape, t.element().bit_width(), 64, threads));
+      out.append(d);
+    }
+    return out;
+  }, py::arg("kernel"),
+        "default layouts of the kernel's alloc_buffers that no GEMM uses, in program order (wave of 64 lanes); pure host");
   m.def("match_ops", [](py::object kernel) {
     py::list out;
     for (const TileOpDesc& d : match_data_movement(op_of_handle(kernel))) out.append(tile_op_dict(d));

@@ -17,11 +17,12 @@ import numpy as np
 
 
 # ------------------------------------------------------------------ affine_map text evaluator
-_TOKEN = re.compile(r"\s*(floordiv|ceildiv|mod|d\d+|\d+|[()+\-*,])")
+_TOKEN = re.compile(r"\s*(floordiv|ceildiv|mod|d\d+|s\d+|\d+|[()+\-*,])")
 
 
 class _Parser:
-    def __init__(self, text, dims):
+    def __init__(self, text, dims, symbols=()):
+        self.symbols = symbols
         self.toks = _TOKEN.findall(text)
         if "".join(self.toks) != re.sub(r"\s+", "", text):
             raise ValueError("cannot tokenize affine expression: %r" % text)
@@ -70,26 +71,33 @@ class _Parser:
             return -self.factor()
         if t[0] == "d":
             return self.dims[int(t[1:])]
+        if t[0] == "s":
+            return self.symbols[int(t[1:])]
         return np.int64(int(t))
 
 
-def eval_affine_map(text, *dims):
-    """`affine_map<(d0, d1) -> (e0, e1, ...)>` evaluated at integer (arrays of) d0, d1, ...; returns the list of results"""
-    m = re.fullmatch(r"\s*affine_map<\(([^)]*)\)\s*->\s*\((.*)\)>\s*", text, re.S)
+def eval_affine_map(text, *dims, symbols=()):
+    """`affine_map<(d0, d1)[s0] -> (e0, e1, ...)>` (the `affine_map<>` wrapper and the symbol list are optional) evaluated at
+    integer (arrays of) d0, d1, ... and symbol values; returns the list of results"""
+    m = re.fullmatch(r"\s*(?:affine_map<)?\(([^)]*)\)\s*(?:\[([^\]]*)\])?\s*->\s*\((.*)\)>?\s*", text, re.S)
     if not m:
         raise ValueError("not an affine_map: %r" % text)
     names = [x.strip() for x in m.group(1).split(",") if x.strip()]
     if len(names) != len(dims):
         raise ValueError("map has %d dims, %d values given" % (len(names), len(dims)))
+    nsym = len([x for x in (m.group(2) or "").split(",") if x.strip()])
+    if nsym != len(symbols):
+        raise ValueError("map has %d symbols, %d values given" % (nsym, len(symbols)))
     dims = [np.asarray(d, dtype=np.int64) for d in dims]
-    p = _Parser(m.group(2), dims)
+    p = _Parser(m.group(3), dims, [np.asarray(v, dtype=np.int64) for v in symbols])
     out = [p.expr()]
     while p.peek() == ",":
         p.take()
         out.append(p.expr())
     if p.peek() is not None:
         raise ValueError("trailing tokens in %r" % text)
-    return [np.broadcast_to(np.asarray(o, dtype=np.int64), np.broadcast(*dims).shape) for o in out]
+    shape = np.broadcast(*dims, *[np.asarray(v) for v in symbols]).shape if (dims or symbols) else ()
+    return [np.broadcast_to(np.asarray(o, dtype=np.int64), shape) for o in out]
 
 
 def grid(rows, cols):
@@ -355,3 +363,30 @@ def bank_stats(index_fn, rows, cols, element_bytes, lane_vector, bank_count=32, 
         worst = max(worst, local)
         acc += local
     return {"avg_max": acc / samples if samples else 0.0, "max": worst, "samples": samples}
+
+
+# ------------------------------------------------------------------ brute-force statements of what the generic inference computes
+def used_extent_brute(map_text, shape, pos):
+    """the largest number of distinct result tuples the map takes along dim `pos` (extent shape[pos]) with the other
+    dims held fixed, over every setting of the others: what computeUsedExtentForDim (LayoutUtils.cpp:181-218) computes
+    structurally for maps that use the pieces of a dim as independent digits"""
+    import itertools
+    best = 0
+    others = [range(n) if k != pos else [0] for k, n in enumerate(shape)]
+    for fixed in itertools.product(*others):
+        dims = [np.arange(shape[pos]) if k == pos else np.int64(v) for k, v in enumerate(fixed)]
+        res = eval_affine_map(map_text, *dims)
+        best = max(best, len({tuple(int(r[t]) for r in res) for t in range(shape[pos])}))
+    return best
+
+
+def reduce_thread_sets(thread_map_text, shape, dim):
+    """for every coordinate of the reduction's destination (the source's with `dim` removed): the set of threads that
+    hold a source element reduced into it -- the threads that own a partial result, hence must hold the result"""
+    import itertools
+    out = {}
+    rest = [n for k, n in enumerate(shape) if k != dim]
+    for x in itertools.product(*[range(n) for n in rest]):
+        dims = list(x[:dim]) + [np.arange(shape[dim])] + list(x[dim:])
+        out[x] = frozenset(int(v) for v in eval_affine_map(thread_map_text, *dims)[0])
+    return out
