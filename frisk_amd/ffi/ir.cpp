@@ -6,6 +6,7 @@
 
 #include "ffi.h"
 #include "mini_ir.h"
+#include "ir_parser.h"
 
 namespace frisk_ffi {
 
@@ -501,6 +502,17 @@ void init_ffi_ir(py::module_&& m) {
       .def("get_src_memref", [](ReduceOp& s) { return s.op->operands[0]; })
       .def("get_dst_memref", [](ReduceOp& s) { return s.op->operands[1]; })
       .def("get_reduce_dim", [](ReduceOp& s) { return s.op->int_attr("dim"); });
+
+  // Text -> module: what mlir::parseSourceString gives a user of the reference's dialect; the grammar is the printed
+  // form (ir_parser.h).  The returned module carries the context as its `context` attribute, which keeps the IR alive.
+  m.def("parse_module", [](PyContext& c, const std::string& text) {
+    ModuleOp mo;
+    mo.op = parse_module_text(*c.ctx, text);
+    mo.ctx = c.ctx.get();
+    py::object o = py::cast(mo);
+    o.attr("context") = py::cast(c);
+    return o;
+  }, py::arg("context"), py::arg("text"), "parses the textual form of a module of frisk kernels; ValueError with line and column on a syntax error");
 
   // ---------------------------------------------------------------- builder (ffi/ir.cpp:144-471)
   py::class_<Builder>(m, "builder")

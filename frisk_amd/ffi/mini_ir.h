@@ -643,11 +643,9 @@ struct Printer {
     const std::string& n = op->name;
     if (n == "builtin.module") {
       os << "module";
+      if (!op->attrs.empty()) os << " attributes";
       attr_dict(op, {}, true);
-      if (!op->attrs.empty()) os << " ";
-      else os << " ";
-      for (Operation* k : op->regions[0]->blocks[0]->ops) (void)k;
-      os << "{\n";
+      os << " {\n";
       for (Operation* k : op->regions[0]->blocks[0]->ops) {
         if (k->name == "frisk.kernel" || k->name == "func.func") number_isolated(k);
         operation(k, ind + 1);
