@@ -430,7 +430,7 @@ void init_ffi_ir(py::module_&& m) {
         for (Operation* op : s.op->regions[0]->blocks[0]->ops)
           if (op->name == "frisk.kernel" && op->attr("sym_name")->s == name) { KernelOp k; k.op = op; k.ctx = s.ctx; return py::cast(k); }
         return py::none();
-      })
+      }, py::keep_alive<0, 1>())  // the kernel handle keeps the module object (and through its `context` attribute the IR) alive
       .def("has_kernel", [](ModuleOp& s, const std::string& name) {
         for (Operation* op : s.op->regions[0]->blocks[0]->ops)
           if (op->name == "frisk.kernel" && op->attr("sym_name")->s == name) return true;

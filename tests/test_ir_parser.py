@@ -142,7 +142,8 @@ def test_a_parsed_kernel_runs_like_the_built_one():
     M, N, K = 512, 384, 256
     h = F.create_session()
     h.tiled_gemm("g", M, N, K, "fp16", tile=(128, 128, 64), threads=256)
-    kernel = reparse(str(h.module)).get_kernel("g")
+    module = reparse(str(h.module))
+    kernel = module.get_kernel("g")
     A = O.encode(O.F16, O.normal(M * K, 5, 0, 0.1)).reshape(M, K)
     B = O.encode(O.F16, O.normal(K * N, 5, 1, 0.1)).reshape(K, N)
     dA, dB = to_dev(A), to_dev(B)
