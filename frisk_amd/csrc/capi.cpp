@@ -151,7 +151,8 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
   if (k->dtype == FRISK_F32) {
     c = area >= 128 * 128 ? 1.93 : (k->bk >= 64 ? 1.0 : 0.55);
   } else if (k->bm == 32) {
-    c = k->wk > 1 ? 0.8 : 0.25;  // 32x32 with a 4x deeper K tile; 32x128
+    // 32x32 with a 4x deeper K tile; 32x128 (8-bit: 60.1 us for 256 tiles x 64 K tiles, the rate of the 32x32 kernel per K tile)
+    c = k->wk > 1 ? 0.8 : (elem_size(k->dtype) == 1 ? 0.85 : 0.25);
   } else if (area >= 256 * 256) {
     c = k->wm * k->wn > 4 ? 1.56 : (k->stages_b > k->stages ? 1.5 : 1.55);  // 2 + 3 ring < 2 + 2 < 8 waves
   } else if (area >= 256 * 128) {
@@ -161,6 +162,13 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
     c = k->stages >= 3 ? (tiles <= 256 ? 0.46 : 0.55) : (tiles <= 256 ? 0.55 : 0.52);
   }
   if (k->guard) c *= 3.0;
+  if (k->bm == 32 && k->wk > 1) {
+    // The 32x32 kernel streams B.  With a ring of 4 tiles one work-group fills a CU: whole rounds of 256, each paying its
+    // own start (measured 14.8 us for 256 tiles, 35.8 for 512).  With a ring of 2 two work-groups share a CU: slower alone
+    // (17.5 us for 256 tiles), but beyond 256 tiles the rounds overlap (29.3 us for 512, 46.6 for 896).
+    if (k->stages >= 3) return (double)((tiles + 255) / 256) * kt * c * (tiles > 256 ? 1.2 : 1.0) / (tiles < 256 ? std::max((double)tiles / 256.0, 0.25) : 1.0);
+    return tiles <= 256 ? kt * c * 1.19 / std::max((double)tiles / 256.0, 0.25) : (double)tiles / 256.0 * kt * c;
+  }
   const int64_t full = tiles / 256, rest = tiles % 256;
   const double rest_fill = (double)rest / 256.0;
   double cost = (double)full * kt * c;
