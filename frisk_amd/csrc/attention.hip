@@ -180,9 +180,16 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
     for (int r = 0; r < RK::NREG; ++r) ck[r] = rk[r] + kbase;
     // fragment of unit x (0 .. N2-1: V, N2 .. N2+N1-1: K) goes to f[x % NB], read PF units ahead of its MFMA
     constexpr int PF = FRISK_ATTN_PREFETCH, NB = PF + 1;
+#ifdef FRISK_ATTN_ABLATE_LDS
+    int f[NB][4] = {};
+#else
     int f[NB][4];
+#endif
     const int last = scores ? N2 + N1 : N2;
     auto fetch = [&](int x) {
+#ifdef FRISK_ATTN_ABLATE_LDS
+      if (nkt > 0) return;  // development aid: fragments are never read
+#endif
       if (x < N2) v_read(vbase, x, f[x % NB]);
       else if (x < last) k_read(ck, x - N2, f[x % NB]);
     };
@@ -191,6 +198,9 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
 #pragma unroll
     for (int u = 0; u < N2; ++u) {
       const v4i vfrag = {f[u % NB][0], f[u % NB][1], f[u % NB][2], f[u % NB][3]};
+#ifdef FRISK_ATTN_ABLATE_MFMA
+      if (nkt < 0)
+#endif
       M::run(vfrag, pf[u / DA], o[u % DA]);
       fetch(u + PF);
       __builtin_amdgcn_sched_barrier(0);
@@ -201,6 +211,9 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
         const int x = u + N2;
         const v4i kfrag = {f[x % NB][0], f[x % NB][1], f[x % NB][2], f[x % NB][3]};
         if (u < KA) s[u % KA] = v16f{};  // folds into the MFMA's C operand: no registers are cleared
+#ifdef FRISK_ATTN_ABLATE_MFMA
+        if (nkt < 0)
+#endif
         M::run(kfrag, qf[u / KA], s[u % KA]);
         fetch(x + PF);
         __builtin_amdgcn_sched_barrier(0);
@@ -210,6 +223,15 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
   // V phase: probabilities of the tile whose scores are in s.  Score e of the lane, e = 16 ka + r, belongs to
   // 16-key step e / 8.
   auto v_phase = [&]() {
+#ifdef FRISK_ATTN_ABLATE_VALU
+    if (nkt > 0) {  // development aid: no softmax work at all
+#pragma unroll
+      for (int t = 0; t < KSTEPS; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(pf[t][j]));
+      return;
+    }
+#endif
     float mx = s[0][0];
 #pragma unroll
     for (int ka = 0; ka < KA; ++ka)
