@@ -204,6 +204,9 @@ def main():
                                                          rws_bytes, cs))):
         ms = time_op(fn)
         ops[name] = {"GB/s": round(moved / (ms * 1e-3) / 1e9, 1), "frac_of_8TB/s": round(moved / (ms * 1e-3) / 8e12, 4), "kernel_ms": round(ms, 5)}
+    # the reference's @online_softmax sketch at the same size class: one read and one write of every element
+    ms = time_op(lambda: R.softmax(R.F16, src16.data_ptr(), ocols, dst16.data_ptr(), ocols, orows, ocols, 1.25, None, cs))
+    ops["softmax_rows"] = {"GB/s": round(2 * nbytes / (ms * 1e-3) / 1e9, 1), "frac_of_8TB/s": round(2 * nbytes / (ms * 1e-3) / 8e12, 4), "kernel_ms": round(ms, 5)}
     del src16, dst16
 
     # fused attention forward at the shape of the reference's sketch: 1 x 32 heads x 4096 x 128, fp16

@@ -462,6 +462,20 @@ int frisk_hip_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int
   return FRISK_OK;
 }
 
+int frisk_hip_softmax(int dtype, const void* src, int64_t src_ld, void* dst, int64_t dst_ld, int64_t rows, int64_t cols, float scale_log2, float* lse,
+                      void* stream) {
+  if (int st = check_view("softmax source", dtype, src, rows, cols, src_ld)) return st;
+  if (int st = check_view("softmax destination", dtype, dst, rows, cols, dst_ld)) return st;
+  if (!std::isfinite(scale_log2)) return fail(FRISK_ERR_ARGUMENT, "softmax scale %g is not finite", (double)scale_log2);
+  if ((uintptr_t)lse & 3) return fail(FRISK_ERR_ALIGNMENT, "lse must be 4-byte aligned");
+  if (rows == 0 || cols == 0) return FRISK_OK;
+  if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
+  const int vec = rows_on_16_bytes(dtype, src, src_ld) && rows_on_16_bytes(dtype, dst, dst_ld) && (cols * elem_size(dtype)) % 16 == 0;
+  hipError_t e = launch_softmax_rows(dtype, src, src_ld, dst, dst_ld, rows, cols, scale_log2, lse, vec, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "softmax launch failed: %s", hipGetErrorString(e));
+  return FRISK_OK;
+}
+
 int frisk_hip_attention(const frisk_attention_desc* d, const void* Q, const void* K, const void* V, void* O, float* lse, void* stream) {
   if (!d) return fail(FRISK_ERR_NULL, "attention descriptor is null");
   if (d->abi_version != FRISK_HIP_ABI_VERSION) return fail(FRISK_ERR_ABI, "descriptor abi_version %d, library %d", d->abi_version, FRISK_HIP_ABI_VERSION);

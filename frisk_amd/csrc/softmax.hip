@@ -1,0 +1,163 @@
+// Row softmax in base 2: y[r][j] = 2^(c x[r][j]) / sum_j 2^(c x[r][j]), the kernel the reference sketches as
+// @online_softmax (tmp/ir.mlir:21-66): per row, chunks of 1024 go through frisk.copy, frisk.reduce max, a frisk.block
+// of exp2(x * cst - max * cst), frisk.reduce sum and a running log-sum (:33-57), then a second sweep writes
+// exp2(x * cst - lse) (:58-68).  Here a work-group of 256 lanes owns a row.  Rows of up to 64 elements per lane are
+// read once and held in registers (maximum, exponentials, sum, scaling: one read and one write of HBM per element);
+// longer rows take the sketch's two sweeps with a running maximum and sum per lane, the second sweep re-reading x.
+// A lane moves 16 bytes at a time where rows start on 16-byte boundaries and the row length is a whole number of
+// such groups; any other view is walked element by element.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "tile_ops.h"
+
+namespace frisk {
+namespace {
+
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+template <int DT> struct SElem;
+template <> struct SElem<FRISK_F32> { typedef float T; static __device__ float load(const T& x) { return x; } static __device__ T store(float x) { return x; } };
+template <> struct SElem<FRISK_F16> { typedef _Float16 T; static __device__ float load(const T& x) { return (float)x; } static __device__ T store(float x) { return (_Float16)x; } };
+template <> struct SElem<FRISK_BF16> { typedef __bf16 T; static __device__ float load(const T& x) { return (float)x; } static __device__ T store(float x) { return (__bf16)x; } };
+
+// (maximum, sum of 2^(v - maximum)) pairs combine associatively
+struct MaxSum {
+  float m, l;
+  __device__ void add(float v) {
+    if (v > m) { l = l * __builtin_amdgcn_exp2f(m - v) + 1.f; m = v; }
+    else l += __builtin_amdgcn_exp2f(v - m);
+  }
+  __device__ void merge(const MaxSum& o) {
+    const float nm = fmaxf(m, o.m);
+    // an empty partner has m = -inf, l = 0: its term must not become 0 * 2^(-inf - -inf)
+    const float a = m == nm ? l : l * __builtin_amdgcn_exp2f(m - nm), b = o.m == nm ? o.l : o.l * __builtin_amdgcn_exp2f(o.m - nm);
+    m = nm;
+    l = a + b;
+  }
+};
+
+__device__ __forceinline__ MaxSum block_merge(MaxSum v, float* lds) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    MaxSum o;
+    o.m = __shfl_xor(v.m, off);
+    o.l = __shfl_xor(v.l, off);
+    v.merge(o);
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) { lds[2 * wave] = v.m; lds[2 * wave + 1] = v.l; }
+  __syncthreads();
+  MaxSum r = {lds[0], lds[1]};
+#pragma unroll
+  for (int w = 1; w < 4; ++w) r.merge(MaxSum{lds[2 * w], lds[2 * w + 1]});
+  __syncthreads();
+  return r;
+}
+
+// NPT > 0: the row fits in NPT 16-byte groups per lane and is kept in registers.  NPT == 0: two sweeps, 16-byte
+// groups when `vec`, single elements otherwise.
+template <int DT, int NPT>
+__global__ void __launch_bounds__(256) softmax_rows_kernel(const typename SElem<DT>::T* src, int64_t sld, typename SElem<DT>::T* dst, int64_t dld, int64_t rows,
+                                                           int64_t cols, float c, float* lse, int vec) {
+  typedef typename SElem<DT>::T T;
+  constexpr int G = 16 / (int)sizeof(T);
+  __shared__ float lds[8];
+  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    const T* x = src + r * sld;
+    T* y = dst + r * dld;
+    if constexpr (NPT > 0) {
+      const int64_t groups = cols / G;
+      float v[NPT][G];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int q = 0; q < NPT; ++q) {
+        const int64_t g = (int64_t)q * 256 + threadIdx.x;
+        T in[G];
+        if (g < groups) *(v4u*)in = __builtin_nontemporal_load((const v4u*)(x + g * G));
+#pragma unroll
+        for (int e = 0; e < G; ++e) {
+          v[q][e] = g < groups ? SElem<DT>::load(in[e]) * c : -INFINITY;
+          mx = fmaxf(mx, v[q][e]);
+        }
+      }
+      const MaxSum top = block_merge(MaxSum{mx, 1.f}, lds);  // only the maximum is used here
+      float sum = 0.f;
+#pragma unroll
+      for (int q = 0; q < NPT; ++q)
+#pragma unroll
+        for (int e = 0; e < G; ++e) {
+          v[q][e] = __builtin_amdgcn_exp2f(v[q][e] - top.m);
+          sum += v[q][e];
+        }
+      const MaxSum all = block_merge(MaxSum{0.f, sum}, lds);  // equal maxima: the sums add
+      const float inv = 1.f / all.l;
+#pragma unroll
+      for (int q = 0; q < NPT; ++q) {
+        const int64_t g = (int64_t)q * 256 + threadIdx.x;
+        if (g < groups) {
+          T out[G];
+#pragma unroll
+          for (int e = 0; e < G; ++e) out[e] = SElem<DT>::store(v[q][e] * inv);
+          __builtin_nontemporal_store(*(const v4u*)out, (v4u*)(y + g * G));
+        }
+      }
+      if (lse && threadIdx.x == 0) lse[r] = top.m + __builtin_amdgcn_logf(all.l);
+    } else {
+      MaxSum acc = {-INFINITY, 0.f};
+      if (vec) {
+        for (int64_t g = threadIdx.x; g < cols / G; g += 256) {
+          T in[G];
+          *(v4u*)in = *(const v4u*)(x + g * G);
+#pragma unroll
+          for (int e = 0; e < G; ++e) acc.add(SElem<DT>::load(in[e]) * c);
+        }
+      } else {
+        for (int64_t j = threadIdx.x; j < cols; j += 256) acc.add(SElem<DT>::load(x[j]) * c);
+      }
+      const MaxSum all = block_merge(acc, lds);
+      const float ref = all.m + __builtin_amdgcn_logf(all.l);  // log2 of the denominator
+      if (vec) {
+        for (int64_t g = threadIdx.x; g < cols / G; g += 256) {
+          T in[G], out[G];
+          *(v4u*)in = *(const v4u*)(x + g * G);
+#pragma unroll
+          for (int e = 0; e < G; ++e) out[e] = SElem<DT>::store(__builtin_amdgcn_exp2f(SElem<DT>::load(in[e]) * c - ref));
+          __builtin_nontemporal_store(*(const v4u*)out, (v4u*)(y + g * G));
+        }
+      } else {
+        for (int64_t j = threadIdx.x; j < cols; j += 256) y[j] = SElem<DT>::store(__builtin_amdgcn_exp2f(SElem<DT>::load(x[j]) * c - ref));
+      }
+      if (lse && threadIdx.x == 0) lse[r] = ref;
+    }
+  }
+}
+
+template <int DT> hipError_t launch_typed(const void* src, int64_t sld, void* dst, int64_t dld, int64_t rows, int64_t cols, float c, float* lse, int vec,
+                                          hipStream_t s) {
+  typedef typename SElem<DT>::T T;
+  constexpr int G = 16 / (int)sizeof(T);
+  const unsigned grid = (unsigned)(rows < 256 * 64 ? rows : 256 * 64);
+  const int64_t per_pass = 256 * (int64_t)G;
+  const T* x = (const T*)src;
+  T* y = (T*)dst;
+  if (vec && cols <= per_pass) hipLaunchKernelGGL((softmax_rows_kernel<DT, 1>), dim3(grid), dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, vec);
+  else if (vec && cols <= 2 * per_pass) hipLaunchKernelGGL((softmax_rows_kernel<DT, 2>), dim3(grid), dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, vec);
+  else if (vec && cols <= 4 * per_pass) hipLaunchKernelGGL((softmax_rows_kernel<DT, 4>), dim3(grid), dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, vec);
+  else if (vec && cols <= 8 * per_pass) hipLaunchKernelGGL((softmax_rows_kernel<DT, 8>), dim3(grid), dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, vec);
+  else hipLaunchKernelGGL((softmax_rows_kernel<DT, 0>), dim3(grid), dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, vec);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+// vec_ok: pointers and leading dimensions put every row on a 16-byte boundary and cols is a whole number of 16-byte groups
+hipError_t launch_softmax_rows(int dtype, const void* src, int64_t sld, void* dst, int64_t dld, int64_t rows, int64_t cols, float scale_log2, float* lse,
+                               int vec_ok, hipStream_t s) {
+  switch (dtype) {
+    case FRISK_F32: return launch_typed<FRISK_F32>(src, sld, dst, dld, rows, cols, scale_log2, lse, vec_ok, s);
+    case FRISK_F16: return launch_typed<FRISK_F16>(src, sld, dst, dld, rows, cols, scale_log2, lse, vec_ok, s);
+    default: return launch_typed<FRISK_BF16>(src, sld, dst, dld, rows, cols, scale_log2, lse, vec_ok, s);
+  }
+}
+
+}  // namespace frisk

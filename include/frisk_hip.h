@@ -206,6 +206,16 @@ size_t frisk_hip_reduce_workspace_bytes(int dtype, int64_t rows, int64_t cols, i
 int frisk_hip_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int64_t ld, int dim, int kind, int clear, void* dst,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* Row softmax in base 2, the kernel sketched as @online_softmax in the reference's tmp/ir.mlir:21-66 (per row: copy,
+ * reduce max, block exp2(x * cst - max * cst), reduce sum, running log-sum; then exp2(x * cst - lse)):
+ *   dst[r][j] = 2^(scale_log2 * src[r][j]) / sum_j 2^(scale_log2 * src[r][j])
+ * on rank-2 views as above (F32, F16, BF16; arithmetic in fp32, result rounded to dtype).  scale_log2 is the sketch's
+ * `cst`; a natural softmax with scale s is scale_log2 = s * log2(e).  lse (may be NULL) receives, per row, the
+ * base-2 logarithm of the denominator, the sketch's `lse`.  dst may be src.  Rows of -inf only give NaN, as the
+ * arithmetic does. */
+int frisk_hip_softmax(int dtype, const void* src, int64_t src_ld, void* dst, int64_t dst_ld, int64_t rows, int64_t cols,
+                      float scale_log2, float* lse, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Fused attention forward: O = softmax(scale * Q K^T) V per (batch, head), the kernel sketched in the
  * reference's tmp/ir.mlir:87-157 (frisk.copy Q; frisk.for over key tiles { copy K; gemm; reduce max;

@@ -48,3 +48,29 @@ def reduce_f64(dtype, src, dim, kind, old=None):
 
 def reduce(dtype, src, dim, kind, old=None):
     return O.encode(dtype, reduce_f64(dtype, src, dim, kind, old).astype(np.float32))
+
+
+def softmax_f64(dtype, src, scale_log2):
+    """(y, lse2) in float64: y = 2^(c x) / sum_j 2^(c x) along dim 1, lse2 = log2 of the denominator"""
+    x = O.decode(dtype, np.ascontiguousarray(src).reshape(-1)).astype(np.float64).reshape(src.shape) * scale_log2
+    m = x.max(axis=1, keepdims=True)
+    e = np.exp2(x - m)
+    den = e.sum(axis=1, keepdims=True)
+    return e / den, (m + np.log2(den))[:, 0]
+
+
+def online_softmax_sketch(dtype, src, cst, chunk=1024):
+    """the reference's @online_softmax, op by op (tmp/ir.mlir:33-68), in float64: a running log-sum over chunks of the row
+    (copy; reduce max :37-38; block exp2(x * cst - max * cst) :39-47; reduce sum :48; lse update :49-60), then a second
+    sweep y = exp2(x * cst - lse) (:62-72)"""
+    x = O.decode(dtype, np.ascontiguousarray(src).reshape(-1)).astype(np.float64).reshape(src.shape)
+    rows, cols = x.shape
+    lse = np.full(rows, -np.inf)                                   # fill(lse, -inf)        :32
+    for c0 in range(0, cols, chunk):
+        xs = x[:, c0:c0 + chunk]
+        max_x = xs.max(axis=1)                                     # reduce max, clear = 1
+        exp_x = np.exp2(xs * cst - max_x[:, None] * cst)
+        sum_exp_x = exp_x.sum(axis=1)                              # reduce sum, clear = 1
+        with np.errstate(invalid="ignore"):
+            lse = max_x * cst + np.log2(np.where(np.isneginf(lse), 0.0, np.exp2(lse - max_x * cst)) + sum_exp_x)
+    return np.exp2(x * cst - lse[:, None]), lse

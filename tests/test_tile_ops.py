@@ -179,3 +179,81 @@ def test_reduce_gpu(hip, dt, dim):
                     assert np.array_equal(got, T.reduce(dt, vals, dim, kind, None if clear else old)), (rows, cols, pad, kind, clear, use_ws)
                 else:
                     _close(dt, got, T.reduce_f64(dt, vals, dim, kind, None if clear else old))
+
+
+# ------------------------------------------------------------------ row softmax (the @online_softmax sketch)
+def test_oracle_softmax_sketch_equals_plain_softmax_and_scipy():
+    from scipy.special import logsumexp, softmax
+    x = O.encode(O.F16, O.normal(5 * 3000, 41, 0, 3.0)).reshape(5, 3000)
+    cst = 1.25
+    y, lse = T.softmax_f64(O.F16, x, cst)
+    for chunk in (1024, 7, 3000, 5000):      # the running log-sum is an identity, whatever the chunking
+        ys, ls = T.online_softmax_sketch(O.F16, x, cst, chunk)
+        assert np.allclose(ys, y, rtol=1e-12, atol=1e-300) and np.allclose(ls, lse, rtol=1e-13)
+    xf = O.decode(O.F16, x.reshape(-1)).astype(np.float64).reshape(x.shape)
+    assert np.allclose(y, softmax(xf * cst * np.log(2.0), axis=1), rtol=1e-12)          # base 2 with cst = base e with cst * ln 2
+    assert np.allclose(lse * np.log(2.0), logsumexp(xf * cst * np.log(2.0), axis=1), rtol=1e-13)
+    assert np.allclose(y.sum(axis=1), 1.0, rtol=1e-13)
+    flat = O.encode(O.F32, np.full(64, 7.0, dtype=np.float32)).reshape(1, 64)
+    yc, lc = T.softmax_f64(O.F32, flat, 2.0)
+    assert np.allclose(yc, 1.0 / 64) and np.allclose(lc, 14.0 + 6.0)                       # constant row: uniform, lse = c x + log2 n
+
+
+def test_softmax_status_codes_before_any_launch():
+    from frisk_amd import runtime as R
+
+    def status(*a):
+        with pytest.raises(R.FriskHipError) as e:
+            R.softmax(*a)
+        return e.value.status
+    p = 1 << 20
+    assert status(R.I8, p, 8, p, 8, 4, 8) == R.ERR_DTYPE
+    assert status(R.F16, p, 4, p, 8, 4, 8) == R.ERR_SHAPE           # leading dimension below the row length
+    assert status(R.F16, None, 8, p, 8, 4, 8) == R.ERR_NULL
+    assert status(R.F16, p + 1, 8, p, 8, 4, 8) == R.ERR_ALIGNMENT
+    assert status(R.F16, p, 8, p, 8, 4, 8, float("inf")) == R.ERR_ARGUMENT
+    R.softmax(R.F16, None, 8, None, 8, 0, 8)                          # nothing to do
+
+
+SOFTMAX_VIEWS = [(1, 1, 0, 0), (3, 8, 0, 0), (7, 1000, 0, 0), (5, 1003, 3, 1), (64, 2048, 8, 0), (16, 4096, 0, 0), (9, 8192, 0, 0), (4, 16384, 0, 0),
+                 (3, 16392, 0, 0), (2, 70000, 0, 0), (300, 40, 0, 0)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", FLOATS, ids=[NAMES[d] for d in FLOATS])
+def test_softmax_gpu(hip, dt):
+    """every path: rows in registers (1, 2, 4, 8 groups per lane), two sweeps (long rows), element by element (odd views);
+    bar: each element within 2e-3 (f16), 8e-3 (bf16), 2e-5 (f32) of the float64 value relative to max(|r|, rms), rows sum
+    to one within that, log-sum within 1e-4"""
+    import torch
+    st = O.NP_STORAGE[dt]
+    es = np.dtype(st).itemsize
+    tol = {O.F32: 2e-5, O.F16: 2e-3, O.BF16: 8e-3}[dt]
+    stream = torch.cuda.current_stream().cuda_stream
+    for rows, cols, pad, shift in SOFTMAX_VIEWS:
+        for cst in (1.25, -0.4):
+            ld = cols + pad
+            vals = O.encode(dt, O.normal(rows * cols, 43, 0, 4.0)).reshape(rows, cols)
+            src = np.zeros(shift + rows * ld, dtype=st)
+            src[shift:].reshape(rows, ld)[:, :cols] = vals
+            dst0 = np.full(shift + rows * ld, 0x7B7B7B7B if es == 4 else 0x7B7B, dtype=st)
+            dS, dD = _dev(src), _dev(dst0)
+            dL = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
+            hip.softmax(dt, dS.data_ptr() + shift * es, ld, dD.data_ptr() + shift * es, ld, rows, cols, cst, dL.data_ptr(), stream)
+            torch.cuda.synchronize()
+            got = _host(dD, st)
+            view = got[shift:].reshape(rows, ld)
+            ref, lse = T.softmax_f64(dt, vals, cst)
+            g = O.decode(dt, np.ascontiguousarray(view[:, :cols]).reshape(-1)).astype(np.float64).reshape(rows, cols)
+            scale = np.maximum(np.abs(ref), np.sqrt(np.mean(ref * ref)))
+            assert np.all(np.isfinite(g)) and np.all(np.abs(g - ref) <= tol * scale), (rows, cols, pad, shift, cst, float(np.max(np.abs(g - ref) / scale)))
+            assert np.abs(dL.cpu().numpy() - lse).max() <= 1e-4 * max(1.0, np.abs(lse).max()), (rows, cols)
+            assert np.array_equal(view[:, cols:], dst0[shift:].reshape(rows, ld)[:, cols:]) and np.array_equal(got[:shift], dst0[:shift])   # nothing outside the view
+    # in place, and a masked column (-inf) gets probability exactly zero
+    vals = O.encode(dt, O.normal(4 * 512, 44, 0, 1.0)).reshape(4, 512)
+    vals[:, 17] = O.encode(dt, np.array([-np.inf], dtype=np.float32))[0]
+    d = _dev(vals)
+    hip.softmax(dt, d.data_ptr(), 512, d.data_ptr(), 512, 4, 512, 1.4426950408889634, None, stream)
+    torch.cuda.synchronize()
+    g = O.decode(dt, _host(d, st)).astype(np.float64).reshape(4, 512)
+    assert np.all(g[:, 17] == 0.0) and np.allclose(g.sum(axis=1), 1.0, atol=64 * tol)
