@@ -12,7 +12,7 @@ namespace {
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 // streaming reads: every byte is read once, so the caches are told not to keep it; on stores the hint pays in copy
-// (5.4 against 4.7 TB/s) and costs in fill (4.3 against 4.7 TB/s), so only copy uses it
+// between equally wide types (6.3 against 5.9 TB/s) and changes nothing in fill, so only copy uses it
 __device__ __forceinline__ v4u load16(const void* p) { return __builtin_nontemporal_load((const v4u*)p); }
 __device__ __forceinline__ void store16(void* p, v4u v) { *(v4u*)p = v; }
 __device__ __forceinline__ void store16_stream(void* p, v4u v) { __builtin_nontemporal_store(v, (v4u*)p); }
@@ -22,62 +22,104 @@ template <> struct Elem<FRISK_F32> { typedef float T; static __device__ float lo
 template <> struct Elem<FRISK_F16> { typedef _Float16 T; static __device__ float load(const T& x) { return (float)x; } static __device__ T store(float x) { return (_Float16)x; } };
 template <> struct Elem<FRISK_BF16> { typedef __bf16 T; static __device__ float load(const T& x) { return (float)x; } static __device__ T store(float x) { return (__bf16)x; } };
 
-// a rows x cols view is walked as (row, group of G columns); G columns of the narrower type fill 16 bytes
-__device__ __forceinline__ bool group_of(int64_t id, int64_t groups_per_row, int64_t rows, int64_t& r, int64_t& c0, int G) {
-  if (id >= groups_per_row * rows) return false;
-  r = id / groups_per_row;
-  c0 = (id % groups_per_row) * G;
-  return true;
-}
+// A rows x cols view is cut into groups of G columns (16 bytes of the narrower type) and walked without any division:
+// 2^lanes_log2 lanes of a work-group lie along a row, the remaining 256 >> lanes_log2 across rows, work-groups step
+// along the row in x and down the rows in y.  Every lane handles several groups per step, all loads issued before the
+// first store: two neighbours along the row (4 KiB apart) where the row is long enough to give both of them work
+// (ALONG; more than two measured slower), else the same columns of eight rows.
+constexpr int kPerLaneAlong = 2, kPerLaneAcross = 8;
 
-template <int DT> __global__ void __launch_bounds__(256) fill_kernel(typename Elem<DT>::T* dst, int64_t rows, int64_t cols, int64_t ld, float value, int vec_ok) {
+template <bool ALONG> struct Walk {
+  static constexpr int PER = ALONG ? kPerLaneAlong : kPerLaneAcross;
+  int64_t slabs, row_blocks, rows, groups_per_row;
+  int lanes, lane_group, lane_row, row_step;
+  __device__ Walk(int64_t rows_, int64_t groups_per_row_, int lanes_log2) : rows(rows_), groups_per_row(groups_per_row_) {
+    lanes = 1 << lanes_log2;
+    row_step = 256 >> lanes_log2;
+    lane_group = threadIdx.x & (lanes - 1);
+    lane_row = threadIdx.x >> lanes_log2;
+    const int64_t per_x = (int64_t)lanes * (ALONG ? PER : 1), per_y = (int64_t)row_step * (ALONG ? 1 : PER);
+    slabs = (groups_per_row + per_x - 1) / per_x;
+    row_blocks = (rows + per_y - 1) / per_y;
+  }
+  // the u-th group of this lane in step (slab, rb); false when it lies outside the view
+  __device__ bool at(int64_t slab, int64_t rb, int u, int64_t& row, int64_t& group) const {
+    group = (ALONG ? slab * PER + u : slab) * lanes + lane_group;
+    row = (ALONG ? rb : rb * PER + u) * row_step + lane_row;
+    return group < groups_per_row && row < rows;
+  }
+};
+
+template <int DT, bool ALONG> __global__ void __launch_bounds__(256)
+fill_kernel(typename Elem<DT>::T* dst, int64_t rows, int64_t cols, int64_t ld, float value, int vec_ok, int lanes_log2) {
   typedef typename Elem<DT>::T T;
   constexpr int G = 16 / sizeof(T);
-  const int64_t gpr = (cols + G - 1) / G;
+  const Walk<ALONG> w(rows, (cols + G - 1) / G, lanes_log2);
+  constexpr int PER = Walk<ALONG>::PER;
   const T v = Elem<DT>::store(value);
-  for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;; id += (int64_t)gridDim.x * 256) {
-    int64_t r, c0;
-    if (!group_of(id, gpr, rows, r, c0, G)) break;
-    T* p = dst + r * ld + c0;
-    if (vec_ok && c0 + G <= cols) {
-      T tmp[G];
+  T tmp[G];
 #pragma unroll
-      for (int e = 0; e < G; ++e) tmp[e] = v;
-      store16(p, *(const v4u*)tmp);
-    } else {
-      for (int e = 0; e < G && c0 + e < cols; ++e) p[e] = v;
+  for (int e = 0; e < G; ++e) tmp[e] = v;
+  for (int64_t rb = blockIdx.y; rb < w.row_blocks; rb += gridDim.y)
+    for (int64_t slab = blockIdx.x; slab < w.slabs; slab += gridDim.x) {
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        int64_t r, g;
+        if (!w.at(slab, rb, u, r, g)) continue;
+        const int64_t c0 = g * G;
+        T* p = dst + r * ld + c0;
+        if (vec_ok && c0 + G <= cols) store16(p, *(const v4u*)tmp);
+        else for (int e = 0; e < G && c0 + e < cols; ++e) p[e] = v;
+      }
     }
-  }
 }
 
-template <int SDT, int DDT> __global__ void __launch_bounds__(256)
-copy_kernel(const typename Elem<SDT>::T* src, int64_t sld, typename Elem<DDT>::T* dst, int64_t dld, int64_t rows, int64_t cols, int vec_ok) {
+template <int SDT, int DDT, bool ALONG> __global__ void __launch_bounds__(256)
+copy_kernel(const typename Elem<SDT>::T* src, int64_t sld, typename Elem<DDT>::T* dst, int64_t dld, int64_t rows, int64_t cols, int vec_ok, int lanes_log2) {
   typedef typename Elem<SDT>::T S;
   typedef typename Elem<DDT>::T D;
   constexpr int G = 16 / (sizeof(S) < sizeof(D) ? sizeof(S) : sizeof(D));  // 16 bytes of the narrower side, 32 of the wider
-  const int64_t gpr = (cols + G - 1) / G;
-  for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;; id += (int64_t)gridDim.x * 256) {
-    int64_t r, c0;
-    if (!group_of(id, gpr, rows, r, c0, G)) break;
-    const S* sp = src + r * sld + c0;
-    D* dp = dst + r * dld + c0;
-    if (vec_ok && c0 + G <= cols) {
-      S in[G];
-      D out[G];
+  const Walk<ALONG> w(rows, (cols + G - 1) / G, lanes_log2);
+  constexpr int PER = Walk<ALONG>::PER;
+  for (int64_t rb = blockIdx.y; rb < w.row_blocks; rb += gridDim.y)
+    for (int64_t slab = blockIdx.x; slab < w.slabs; slab += gridDim.x) {
+      S in[PER][G];
+      bool whole[PER];
+      // every load of the step is issued before the first store
 #pragma unroll
-      for (int q = 0; q < (int)(G * sizeof(S) / 16); ++q) ((v4u*)in)[q] = load16((const v4u*)sp + q);
+      for (int u = 0; u < PER; ++u) {
+        int64_t r, g;
+        whole[u] = w.at(slab, rb, u, r, g) && vec_ok && g * G + G <= cols;
+        if (whole[u]) {
 #pragma unroll
-      for (int e = 0; e < G; ++e) {
-        if constexpr (SDT == DDT) out[e] = in[e]; else out[e] = Elem<DDT>::store(Elem<SDT>::load(in[e]));
+          for (int q = 0; q < (int)(G * sizeof(S) / 16); ++q) ((v4u*)in[u])[q] = load16((const v4u*)(src + r * sld + g * G) + q);
+        }
       }
 #pragma unroll
-      for (int q = 0; q < (int)(G * sizeof(D) / 16); ++q) store16_stream((v4u*)dp + q, ((const v4u*)out)[q]);
-    } else {
-      for (int e = 0; e < G && c0 + e < cols; ++e) {
-        if constexpr (SDT == DDT) dp[e] = sp[e]; else dp[e] = Elem<DDT>::store(Elem<SDT>::load(sp[e]));
+      for (int u = 0; u < PER; ++u) {
+        int64_t r, g;
+        if (!w.at(slab, rb, u, r, g)) continue;
+        const int64_t c0 = g * G;
+        const S* sp = src + r * sld + c0;
+        D* dp = dst + r * dld + c0;
+        if (whole[u]) {
+          D out[G];
+#pragma unroll
+          for (int e = 0; e < G; ++e) {
+            if constexpr (SDT == DDT) out[e] = in[u][e]; else out[e] = Elem<DDT>::store(Elem<SDT>::load(in[u][e]));
+          }
+#pragma unroll
+          for (int q = 0; q < (int)(G * sizeof(D) / 16); ++q) {
+            // a lane's two stores of a widening copy each cover half of its 32 bytes: the cache has to merge them
+            if constexpr (sizeof(D) > sizeof(S)) store16((v4u*)dp + q, ((const v4u*)out)[q]); else store16_stream((v4u*)dp + q, ((const v4u*)out)[q]);
+          }
+        } else {
+          for (int e = 0; e < G && c0 + e < cols; ++e) {
+            if constexpr (SDT == DDT) dp[e] = sp[e]; else dp[e] = Elem<DDT>::store(Elem<SDT>::load(sp[e]));
+          }
+        }
       }
     }
-  }
 }
 
 // ------------------------------------------------------------------ reduce
@@ -192,16 +234,28 @@ reduce_finish_kernel(const float* partial, int slices, int64_t n, int clear, typ
   dst[i] = Elem<DT>::store(clear ? v : Op<KIND>::f(Elem<DT>::load(dst[i]), v));
 }
 
-unsigned blocks_for(int64_t work_items) {
-  int64_t b = (work_items + 255) / 256;
-  const int64_t cap = 256 * 16;  // 16 work-groups per CU keep every CU streaming; beyond that lanes loop
-  return (unsigned)(b < 1 ? 1 : (b > cap ? cap : b));
-}
+// grid and lane split of the division-free walk: lanes along a row = the power of two that covers the row's groups,
+// at most 256; x steps along the row, y down the rows (65535 at most, work-groups loop beyond that)
+struct WalkLaunch {
+  dim3 grid;
+  int lanes_log2, along;
+  WalkLaunch(int64_t rows, int64_t groups_per_row) {
+    lanes_log2 = 0;
+    while (lanes_log2 < 8 && (int64_t(1) << lanes_log2) < groups_per_row) ++lanes_log2;
+    along = groups_per_row >= 256 * kPerLaneAlong;
+    const int kPerLane = along ? kPerLaneAlong : kPerLaneAcross;
+    const int64_t per_x = (int64_t(1) << lanes_log2) * (along ? kPerLane : 1), per_y = (int64_t)(256 >> lanes_log2) * (along ? 1 : kPerLane);
+    const int64_t slabs = (groups_per_row + per_x - 1) / per_x, row_blocks = (rows + per_y - 1) / per_y;
+    grid = dim3((unsigned)(slabs < 1 ? 1 : (slabs > 0x7fffffff ? 0x7fffffff : slabs)), (unsigned)(row_blocks < 1 ? 1 : (row_blocks > 65535 ? 65535 : row_blocks)));
+  }
+};
 
 template <int DT> hipError_t fill_t(void* dst, int64_t rows, int64_t cols, int64_t ld, double value, int vec_ok, hipStream_t s) {
   typedef typename Elem<DT>::T T;
   constexpr int G = 16 / sizeof(T);
-  hipLaunchKernelGGL(fill_kernel<DT>, dim3(blocks_for(rows * ((cols + G - 1) / G))), dim3(256), 0, s, (T*)dst, rows, cols, ld, (float)value, vec_ok);
+  const WalkLaunch w(rows, (cols + G - 1) / G);
+  if (w.along) hipLaunchKernelGGL((fill_kernel<DT, true>), w.grid, dim3(256), 0, s, (T*)dst, rows, cols, ld, (float)value, vec_ok, w.lanes_log2);
+  else hipLaunchKernelGGL((fill_kernel<DT, false>), w.grid, dim3(256), 0, s, (T*)dst, rows, cols, ld, (float)value, vec_ok, w.lanes_log2);
   return hipGetLastError();
 }
 
@@ -209,7 +263,9 @@ template <int SDT, int DDT> hipError_t copy_t(const void* src, int64_t sld, void
   typedef typename Elem<SDT>::T S;
   typedef typename Elem<DDT>::T D;
   constexpr int G = 16 / (sizeof(S) < sizeof(D) ? sizeof(S) : sizeof(D));
-  hipLaunchKernelGGL((copy_kernel<SDT, DDT>), dim3(blocks_for(rows * ((cols + G - 1) / G))), dim3(256), 0, s, (const S*)src, sld, (D*)dst, dld, rows, cols, vec_ok);
+  const WalkLaunch w(rows, (cols + G - 1) / G);
+  if (w.along) hipLaunchKernelGGL((copy_kernel<SDT, DDT, true>), w.grid, dim3(256), 0, s, (const S*)src, sld, (D*)dst, dld, rows, cols, vec_ok, w.lanes_log2);
+  else hipLaunchKernelGGL((copy_kernel<SDT, DDT, false>), w.grid, dim3(256), 0, s, (const S*)src, sld, (D*)dst, dld, rows, cols, vec_ok, w.lanes_log2);
   return hipGetLastError();
 }
 
