@@ -169,13 +169,17 @@ reduce_rows_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, 
   }
 }
 
-// along dim 0: a work-group owns a strip of 32 x G columns (512 bytes of every row) and a slice of the rows; 32 column lanes x 8 row lanes
+// along dim 0: a work-group owns a strip of kStripLanes x G columns (kStripLanes x 16 bytes of every row) and a slice of the rows;
+// kStripLanes column lanes x kStripRows row lanes, four rows in flight per lane
+constexpr int kStripFlight = 4;  // rows in flight per lane; 2 to 16 measure within 4 % of each other
+constexpr int kStripLanes = 32, kStripRows = 256 / kStripLanes;  // 16 and 64 lanes measured 9 % and 15 % slower
+
 template <int DT, int KIND> __global__ void __launch_bounds__(256)
 reduce_cols_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, int64_t ld, int clear, typename Elem<DT>::T* dst, float* partial, int vec_ok) {
   typedef typename Elem<DT>::T T;
   constexpr int G = 16 / sizeof(T);
-  const int cl = threadIdx.x & 31, rl = threadIdx.x >> 5;
-  const int64_t c0 = ((int64_t)blockIdx.x * 32 + cl) * G;
+  const int cl = threadIdx.x % kStripLanes, rl = threadIdx.x / kStripLanes;
+  const int64_t c0 = ((int64_t)blockIdx.x * kStripLanes + cl) * G;
   const int64_t per = (rows + gridDim.y - 1) / gridDim.y;
   const int64_t r0 = (int64_t)blockIdx.y * per, r1 = r0 + per < rows ? r0 + per : rows;
   float acc[G];
@@ -184,17 +188,17 @@ reduce_cols_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, 
   if (c0 < cols) {
     int64_t r = r0 + rl;
     if (vec_ok && c0 + G <= cols) {
-      for (; r + 24 < r1; r += 32) {  // four rows in flight per lane
-        T in[4][G];
+      for (; r + (kStripFlight - 1) * kStripRows < r1; r += kStripFlight * kStripRows) {
+        T in[kStripFlight][G];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) *(v4u*)in[u] = load16(src + (r + 8 * u) * ld + c0);
+        for (int u = 0; u < kStripFlight; ++u) *(v4u*)in[u] = load16(src + (r + kStripRows * u) * ld + c0);
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < kStripFlight; ++u)
 #pragma unroll
           for (int e = 0; e < G; ++e) acc[e] = Op<KIND>::f(acc[e], Elem<DT>::load(in[u][e]));
       }
     }
-    for (; r < r1; r += 8) {
+    for (; r < r1; r += kStripRows) {
       const T* p = src + r * ld + c0;
       if (vec_ok && c0 + G <= cols) {
         T in[G];
@@ -206,7 +210,7 @@ reduce_cols_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, 
       }
     }
   }
-  __shared__ float red[8][32][G + 1];
+  __shared__ float red[kStripRows][kStripLanes][G + 1];
 #pragma unroll
   for (int e = 0; e < G; ++e) red[rl][cl][e] = acc[e];
   __syncthreads();
@@ -215,7 +219,7 @@ reduce_cols_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, 
     for (int e = 0; e < G; ++e) {
       float v = red[0][cl][e];
 #pragma unroll
-      for (int k = 1; k < 8; ++k) v = Op<KIND>::f(v, red[k][cl][e]);
+      for (int k = 1; k < kStripRows; ++k) v = Op<KIND>::f(v, red[k][cl][e]);
       if (c0 + e < cols) {
         if (gridDim.y > 1) partial[(int64_t)blockIdx.y * cols + c0 + e] = v;
         else dst[c0 + e] = Elem<DT>::store(clear ? v : Op<KIND>::f(Elem<DT>::load(dst[c0 + e]), v));
@@ -224,14 +228,32 @@ reduce_cols_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, 
   }
 }
 
-// second pass of a split reduction: out[i] = kind over s of partial[s][i] (combined with dst unless clear)
+// second pass of a split reduction: out[i] = kind over s of partial[s][i] (combined with dst unless clear).  64 outputs x 4
+// slice lanes per work-group: a lane combines every fourth slice with four loads in flight, so that 256 slices cost 16
+// memory round trips instead of 256.
 template <int DT, int KIND> __global__ void __launch_bounds__(256)
 reduce_finish_kernel(const float* partial, int slices, int64_t n, int clear, typename Elem<DT>::T* dst) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n) return;
-  float v = partial[i];
-  for (int s = 1; s < slices; ++s) v = Op<KIND>::f(v, partial[(int64_t)s * n + i]);
-  dst[i] = Elem<DT>::store(clear ? v : Op<KIND>::f(Elem<DT>::load(dst[i]), v));
+  const int ol = threadIdx.x & 63, sl = threadIdx.x >> 6;
+  const int64_t i = (int64_t)blockIdx.x * 64 + ol;
+  float v = Op<KIND>::id();
+  if (i < n) {
+    int s = sl;
+    for (; s + 12 < slices; s += 16) {
+      float t[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) t[u] = partial[(int64_t)(s + 4 * u) * n + i];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v = Op<KIND>::f(v, t[u]);
+    }
+    for (; s < slices; s += 4) v = Op<KIND>::f(v, partial[(int64_t)s * n + i]);
+  }
+  __shared__ float red[4][64];
+  red[sl][ol] = v;
+  __syncthreads();
+  if (sl == 0 && i < n) {
+    v = Op<KIND>::f(Op<KIND>::f(red[0][ol], red[1][ol]), Op<KIND>::f(red[2][ol], red[3][ol]));
+    dst[i] = Elem<DT>::store(clear ? v : Op<KIND>::f(Elem<DT>::load(dst[i]), v));
+  }
 }
 
 // grid and lane split of the division-free walk: lanes along a row = the power of two that covers the row's groups,
@@ -276,13 +298,13 @@ template <int DT, int KIND> hipError_t reduce_t(const void* src, int64_t rows, i
   if (dim == 1) {
     hipLaunchKernelGGL((reduce_rows_kernel<DT, KIND>), dim3((unsigned)rows, (unsigned)slices), dim3(256), 0, s, (const T*)src, rows, cols, ld, clear, (T*)dst, partial, vec_ok);
   } else {
-    const unsigned strips = (unsigned)((cols + 32 * G - 1) / (32 * G));
+    const unsigned strips = (unsigned)((cols + kStripLanes * G - 1) / (kStripLanes * G));
     hipLaunchKernelGGL((reduce_cols_kernel<DT, KIND>), dim3(strips, (unsigned)slices), dim3(256), 0, s, (const T*)src, rows, cols, ld, clear, (T*)dst, partial, vec_ok);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || slices == 1) return e;
   const int64_t n = dim == 1 ? rows : cols;
-  hipLaunchKernelGGL((reduce_finish_kernel<DT, KIND>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, partial, slices, n, clear, (T*)dst);
+  hipLaunchKernelGGL((reduce_finish_kernel<DT, KIND>), dim3((unsigned)((n + 63) / 64)), dim3(256), 0, s, partial, slices, n, clear, (T*)dst);
   return hipGetLastError();
 }
 
@@ -302,8 +324,8 @@ int reduce_slices(int dtype, int64_t rows, int64_t cols, int dim) {
   // Split the reduced extent so that about 1024 work-groups exist, each still reducing at least 16 KiB.
   const int es = dtype == FRISK_F32 ? 4 : 2;
   const int G = 16 / es;
-  const int64_t groups = dim == 1 ? rows : (cols + 32 * G - 1) / (32 * G);
-  const int64_t extent_bytes = dim == 1 ? cols * es : rows * 32 * 16;  // bytes one work-group would walk unsplit
+  const int64_t groups = dim == 1 ? rows : (cols + kStripLanes * G - 1) / (kStripLanes * G);
+  const int64_t extent_bytes = dim == 1 ? cols * es : rows * kStripLanes * 16;  // bytes one work-group would walk unsplit
   int slices = 1;
   while (groups * slices < 1024 && extent_bytes / (slices * 2) >= 16384 && slices < 256) slices *= 2;
   return slices;
