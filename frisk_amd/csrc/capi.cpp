@@ -470,8 +470,8 @@ int frisk_hip_softmax(int dtype, const void* src, int64_t src_ld, void* dst, int
   if ((uintptr_t)lse & 3) return fail(FRISK_ERR_ALIGNMENT, "lse must be 4-byte aligned");
   if (rows == 0 || cols == 0) return FRISK_OK;
   if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
-  const int vec = rows_on_16_bytes(dtype, src, src_ld) && rows_on_16_bytes(dtype, dst, dst_ld) && (cols * elem_size(dtype)) % 16 == 0;
-  hipError_t e = launch_softmax_rows(dtype, src, src_ld, dst, dst_ld, rows, cols, scale_log2, lse, vec, (hipStream_t)stream);
+  const int rows_aligned = rows_on_16_bytes(dtype, src, src_ld) && rows_on_16_bytes(dtype, dst, dst_ld);
+  hipError_t e = launch_softmax_rows(dtype, src, src_ld, dst, dst_ld, rows, cols, scale_log2, lse, rows_aligned, (hipStream_t)stream);
   if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "softmax launch failed: %s", hipGetErrorString(e));
   return FRISK_OK;
 }

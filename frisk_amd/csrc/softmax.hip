@@ -1,11 +1,12 @@
 // Row softmax in base 2: y[r][j] = 2^(c x[r][j]) / sum_j 2^(c x[r][j]), the kernel the reference sketches as
 // @online_softmax (tmp/ir.mlir:21-66): per row, chunks of 1024 go through frisk.copy, frisk.reduce max, a frisk.block
 // of exp2(x * cst - max * cst), frisk.reduce sum and a running log-sum (:33-57), then a second sweep writes
-// exp2(x * cst - lse) (:58-68).  Here a work-group of 256 lanes owns a row.  Rows of up to 64 elements per lane are
+// exp2(x * cst - lse) (:58-68).  Here rows of up to 256 groups of 16 bytes (2048 f16) are shared by 1 to 64 lanes of one
+// wave and combined by shuffles; longer rows get a work-group of 256 lanes each.  Rows of up to 64 elements per lane are
 // read once and held in registers (maximum, exponentials, sum, scaling: one read and one write of HBM per element);
 // longer rows take the sketch's two sweeps with a running maximum and sum per lane, the second sweep re-reading x.
-// A lane moves 16 bytes at a time where rows start on 16-byte boundaries and the row length is a whole number of
-// such groups; any other view is walked element by element.
+// A lane moves 16 bytes at a time where rows start on 16-byte boundaries; groups that are not whole and, in the
+// work-group kernels, any view whose row length is not a whole number of groups are walked element by element.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include "tile_ops.h"
@@ -54,7 +55,7 @@ __device__ __forceinline__ MaxSum block_merge(MaxSum v, float* lds) {
   return r;
 }
 
-// NPT > 0: the row fits in NPT 16-byte groups per lane and is kept in registers.  NPT == 0: two sweeps, 16-byte
+// Longer rows, a work-group each.  NPT > 0: the row fits in NPT 16-byte groups per lane and is kept in registers.  NPT == 0: two sweeps, 16-byte
 // groups when `vec`, single elements otherwise.
 template <int DT, int NPT>
 __global__ void __launch_bounds__(256) softmax_rows_kernel(const typename SElem<DT>::T* src, int64_t sld, typename SElem<DT>::T* dst, int64_t dld, int64_t rows,
@@ -132,16 +133,91 @@ __global__ void __launch_bounds__(256) softmax_rows_kernel(const typename SElem<
   }
 }
 
-template <int DT> hipError_t launch_typed(const void* src, int64_t sld, void* dst, int64_t dld, int64_t rows, int64_t cols, float c, float* lse, int vec,
+// Rows of at most 256 groups of 16 bytes: 2^lanes_log2 <= 64 lanes of one wave share a row, each holding up to NPT groups in
+// registers, and combine maximum and sum by shuffles (no LDS, no barrier); a work-group holds 256 >> lanes_log2 rows.  Any
+// alignment: a group that is not a whole, aligned 16 bytes is walked element by element.
+template <int DT, int NPT>
+__global__ void __launch_bounds__(256) softmax_short_rows_kernel(const typename SElem<DT>::T* src, int64_t sld, typename SElem<DT>::T* dst, int64_t dld, int64_t rows,
+                                                                 int64_t cols, float c, float* lse, int vec, int lanes_log2) {
+  typedef typename SElem<DT>::T T;
+  constexpr int G = 16 / (int)sizeof(T);
+  const int lanes = 1 << lanes_log2, lane = threadIdx.x & (lanes - 1), rows_per_group = 256 >> lanes_log2;
+  const int64_t blocks = (rows + rows_per_group - 1) / rows_per_group;
+  for (int64_t rb = blockIdx.x; rb < blocks; rb += gridDim.x) {
+    const int64_t r = rb * rows_per_group + (threadIdx.x >> lanes_log2);
+    const bool live = r < rows;  // lanes of rows past the end still take part in the shuffles
+    const T* x = src + r * sld;
+    T* y = dst + r * dld;
+    float v[NPT][G];
+    bool whole[NPT];
+    T in[NPT][G];
+#pragma unroll
+    for (int q = 0; q < NPT; ++q) {
+      const int64_t c0 = (int64_t)(q * lanes + lane) * G;
+      whole[q] = live && vec && c0 + G <= cols;
+      if (whole[q]) *(v4u*)in[q] = __builtin_nontemporal_load((const v4u*)(x + c0));
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int q = 0; q < NPT; ++q) {
+      const int64_t c0 = (int64_t)(q * lanes + lane) * G;
+#pragma unroll
+      for (int e = 0; e < G; ++e) {
+        if (whole[q]) v[q][e] = SElem<DT>::load(in[q][e]) * c;
+        else v[q][e] = live && c0 + e < cols ? SElem<DT>::load(x[c0 + e]) * c : -INFINITY;
+        mx = fmaxf(mx, v[q][e]);
+      }
+    }
+    for (int off = lanes >> 1; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float sum = 0.f;
+#pragma unroll
+    for (int q = 0; q < NPT; ++q)
+#pragma unroll
+      for (int e = 0; e < G; ++e) {
+        v[q][e] = __builtin_amdgcn_exp2f(v[q][e] - mx);
+        sum += v[q][e];
+      }
+    for (int off = lanes >> 1; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const float inv = 1.f / sum;
+#pragma unroll
+    for (int q = 0; q < NPT; ++q) {
+      const int64_t c0 = (int64_t)(q * lanes + lane) * G;
+      if (whole[q]) {
+        T out[G];
+#pragma unroll
+        for (int e = 0; e < G; ++e) out[e] = SElem<DT>::store(v[q][e] * inv);
+        __builtin_nontemporal_store(*(const v4u*)out, (v4u*)(y + c0));
+      } else if (live) {
+#pragma unroll
+        for (int e = 0; e < G; ++e)
+          if (c0 + e < cols) y[c0 + e] = SElem<DT>::store(v[q][e] * inv);
+      }
+    }
+    if (lse && live && lane == 0) lse[r] = mx + __builtin_amdgcn_logf(sum);
+  }
+}
+
+template <int DT> hipError_t launch_typed(const void* src, int64_t sld, void* dst, int64_t dld, int64_t rows, int64_t cols, float c, float* lse, int rows_aligned,
                                           hipStream_t s) {
   typedef typename SElem<DT>::T T;
   constexpr int G = 16 / (int)sizeof(T);
+  const int vec = rows_aligned && cols % G == 0;
   const unsigned grid = (unsigned)(rows < 256 * 64 ? rows : 256 * 64);
   const int64_t per_pass = 256 * (int64_t)G;
   const T* x = (const T*)src;
   T* y = (T*)dst;
-  if (vec && cols <= per_pass) hipLaunchKernelGGL((softmax_rows_kernel<DT, 1>), dim3(grid), dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, vec);
-  else if (vec && cols <= 2 * per_pass) hipLaunchKernelGGL((softmax_rows_kernel<DT, 2>), dim3(grid), dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, vec);
+  const int64_t groups = (cols + G - 1) / G;
+  if (groups <= 256) {  // here a row that ends in a partial group still moves its whole groups 16 bytes at a time
+    int lanes_log2 = 0;
+    while (lanes_log2 < 6 && (int64_t(1) << lanes_log2) < groups) ++lanes_log2;
+    const int64_t rows_per_group = 256 >> lanes_log2, blocks = (rows + rows_per_group - 1) / rows_per_group;
+    const dim3 sgrid((unsigned)(blocks < (1 << 22) ? blocks : (1 << 22)));
+    if (groups <= 64) hipLaunchKernelGGL((softmax_short_rows_kernel<DT, 1>), sgrid, dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, rows_aligned, lanes_log2);
+    else if (groups <= 128) hipLaunchKernelGGL((softmax_short_rows_kernel<DT, 2>), sgrid, dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, rows_aligned, lanes_log2);
+    else hipLaunchKernelGGL((softmax_short_rows_kernel<DT, 4>), sgrid, dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, rows_aligned, lanes_log2);
+    return hipGetLastError();
+  }
+  if (vec && cols <= 2 * per_pass) hipLaunchKernelGGL((softmax_rows_kernel<DT, 2>), dim3(grid), dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, vec);
   else if (vec && cols <= 4 * per_pass) hipLaunchKernelGGL((softmax_rows_kernel<DT, 4>), dim3(grid), dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, vec);
   else if (vec && cols <= 8 * per_pass) hipLaunchKernelGGL((softmax_rows_kernel<DT, 8>), dim3(grid), dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, vec);
   else hipLaunchKernelGGL((softmax_rows_kernel<DT, 0>), dim3(grid), dim3(256), 0, s, x, sld, y, dld, rows, cols, c, lse, vec);
@@ -150,13 +226,13 @@ template <int DT> hipError_t launch_typed(const void* src, int64_t sld, void* ds
 
 }  // namespace
 
-// vec_ok: pointers and leading dimensions put every row on a 16-byte boundary and cols is a whole number of 16-byte groups
+// rows_aligned: pointers and leading dimensions put every row of both views on a 16-byte boundary
 hipError_t launch_softmax_rows(int dtype, const void* src, int64_t sld, void* dst, int64_t dld, int64_t rows, int64_t cols, float scale_log2, float* lse,
-                               int vec_ok, hipStream_t s) {
+                               int rows_aligned, hipStream_t s) {
   switch (dtype) {
-    case FRISK_F32: return launch_typed<FRISK_F32>(src, sld, dst, dld, rows, cols, scale_log2, lse, vec_ok, s);
-    case FRISK_F16: return launch_typed<FRISK_F16>(src, sld, dst, dld, rows, cols, scale_log2, lse, vec_ok, s);
-    default: return launch_typed<FRISK_BF16>(src, sld, dst, dld, rows, cols, scale_log2, lse, vec_ok, s);
+    case FRISK_F32: return launch_typed<FRISK_F32>(src, sld, dst, dld, rows, cols, scale_log2, lse, rows_aligned, s);
+    case FRISK_F16: return launch_typed<FRISK_F16>(src, sld, dst, dld, rows, cols, scale_log2, lse, rows_aligned, s);
+    default: return launch_typed<FRISK_BF16>(src, sld, dst, dld, rows, cols, scale_log2, lse, rows_aligned, s);
   }
 }
 

@@ -14,7 +14,7 @@ hipError_t launch_copy(int src_dtype, const void* src, int64_t src_ld, int dst_d
 int reduce_slices(int dtype, int64_t rows, int64_t cols, int dim);
 hipError_t launch_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int64_t ld, int dim, int kind, int clear, void* dst, float* partial, int slices,
                          int vec_ok, hipStream_t s);
-// row softmax in base 2 (softmax.hip); vec_ok as above, with cols a whole number of 16-byte groups
+// row softmax in base 2 (softmax.hip); rows_aligned: every row of both views starts on a 16-byte boundary
 hipError_t launch_softmax_rows(int dtype, const void* src, int64_t sld, void* dst, int64_t dld, int64_t rows, int64_t cols, float scale_log2, float* lse,
-                               int vec_ok, hipStream_t s);
+                               int rows_aligned, hipStream_t s);
 }  // namespace frisk

@@ -135,95 +135,145 @@ template <int KIND> __device__ __forceinline__ float wave_reduce(float v) {
   return v;
 }
 
-// along dim 1: work-group (x = row, y = column slice) reduces its slice of one row; lanes stride over 16-byte groups.
+// along dim 1: work-group (x = row, y = column slice) reduces every gridDim.y-th run of 256 16-byte groups of one row, so that
+// the slices of a row read neighbouring memory at any time.
 // With gridDim.y == 1 the result goes to dst (combined with the old value unless clear), else to partial[y][row].
 template <int DT, int KIND> __global__ void __launch_bounds__(256)
 reduce_rows_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, int64_t ld, int clear, typename Elem<DT>::T* dst, float* partial, int vec_ok) {
   typedef typename Elem<DT>::T T;
   constexpr int G = 16 / sizeof(T);
-  const int64_t r = blockIdx.x;
   const int64_t gpr = (cols + G - 1) / G;
-  const int64_t per = (gpr + gridDim.y - 1) / gridDim.y;
-  const int64_t g0 = (int64_t)blockIdx.y * per, g1 = g0 + per < gpr ? g0 + per : gpr;
-  float acc = Op<KIND>::id();
-  const T* row = src + r * ld;
-  for (int64_t g = g0 + threadIdx.x; g < g1; g += 256) {
-    const int64_t c0 = g * G;
-    if (vec_ok && c0 + G <= cols) {
-      T in[G];
-      *(v4u*)in = load16(row + c0);
-#pragma unroll
-      for (int e = 0; e < G; ++e) acc = Op<KIND>::f(acc, Elem<DT>::load(in[e]));
-    } else {
-      for (int e = 0; e < G && c0 + e < cols; ++e) acc = Op<KIND>::f(acc, Elem<DT>::load(row[c0 + e]));
-    }
-  }
   __shared__ float wsum[4];
-  acc = wave_reduce<KIND>(acc);
-  if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = acc;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    float v = Op<KIND>::f(Op<KIND>::f(wsum[0], wsum[1]), Op<KIND>::f(wsum[2], wsum[3]));
-    if (gridDim.y > 1) partial[(int64_t)blockIdx.y * rows + r] = v;
-    else dst[r] = Elem<DT>::store(clear ? v : Op<KIND>::f(Elem<DT>::load(dst[r]), v));
+  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    float acc = Op<KIND>::id();
+    const T* row = src + r * ld;
+    for (int64_t g = (int64_t)blockIdx.y * 256 + threadIdx.x; g < gpr; g += (int64_t)gridDim.y * 256) {
+      const int64_t c0 = g * G;
+      if (vec_ok && c0 + G <= cols) {
+        T in[G];
+        *(v4u*)in = load16(row + c0);
+#pragma unroll
+        for (int e = 0; e < G; ++e) acc = Op<KIND>::f(acc, Elem<DT>::load(in[e]));
+      } else {
+        for (int e = 0; e < G && c0 + e < cols; ++e) acc = Op<KIND>::f(acc, Elem<DT>::load(row[c0 + e]));
+      }
+    }
+    acc = wave_reduce<KIND>(acc);
+    if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float v = Op<KIND>::f(Op<KIND>::f(wsum[0], wsum[1]), Op<KIND>::f(wsum[2], wsum[3]));
+      if (gridDim.y > 1) partial[(int64_t)blockIdx.y * rows + r] = v;
+      else dst[r] = Elem<DT>::store(clear ? v : Op<KIND>::f(Elem<DT>::load(dst[r]), v));
+    }
+    __syncthreads();
   }
 }
 
-// along dim 0: a work-group owns a strip of kStripLanes x G columns (kStripLanes x 16 bytes of every row) and a slice of the rows;
-// kStripLanes column lanes x kStripRows row lanes, four rows in flight per lane
-constexpr int kStripFlight = 4;  // rows in flight per lane; 2 to 16 measure within 4 % of each other
-constexpr int kStripLanes = 32, kStripRows = 256 / kStripLanes;  // 16 and 64 lanes measured 9 % and 15 % slower
+// along dim 1, rows of at most 256 groups of 16 bytes: 2^lanes_log2 <= 64 lanes of one wave share a row, each taking up to
+// NPT groups, and combine by shuffles; a work-group holds 256 >> lanes_log2 rows and takes 4 / NPT such sets of rows per
+// step, so that every lane has four loads in flight before the first is used.
+template <int DT, int KIND, int NPT> __global__ void __launch_bounds__(256)
+reduce_short_rows_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, int64_t ld, int clear, typename Elem<DT>::T* dst, int vec_ok, int lanes_log2) {
+  typedef typename Elem<DT>::T T;
+  constexpr int G = 16 / sizeof(T), SETS = 4 / NPT;
+  const int lanes = 1 << lanes_log2, lane = threadIdx.x & (lanes - 1), rows_per_set = 256 >> lanes_log2;
+  const int64_t blocks = (rows + rows_per_set * SETS - 1) / (rows_per_set * SETS);
+  for (int64_t rb = blockIdx.x; rb < blocks; rb += gridDim.x) {
+    T in[SETS][NPT][G];
+    bool whole[SETS][NPT];
+#pragma unroll
+    for (int t = 0; t < SETS; ++t) {
+      const int64_t r = (rb * SETS + t) * rows_per_set + (threadIdx.x >> lanes_log2);
+#pragma unroll
+      for (int q = 0; q < NPT; ++q) {
+        const int64_t c0 = (int64_t)(q * lanes + lane) * G;
+        whole[t][q] = r < rows && vec_ok && c0 + G <= cols;
+        if (whole[t][q]) *(v4u*)in[t][q] = load16(src + r * ld + c0);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < SETS; ++t) {
+      const int64_t r = (rb * SETS + t) * rows_per_set + (threadIdx.x >> lanes_log2);
+      const bool live = r < rows;  // lanes of rows past the end still take part in the shuffles
+      float acc = Op<KIND>::id();
+#pragma unroll
+      for (int q = 0; q < NPT; ++q) {
+        const int64_t c0 = (int64_t)(q * lanes + lane) * G;
+        if (whole[t][q]) {
+#pragma unroll
+          for (int e = 0; e < G; ++e) acc = Op<KIND>::f(acc, Elem<DT>::load(in[t][q][e]));
+        } else if (live) {
+          for (int e = 0; e < G && c0 + e < cols; ++e) acc = Op<KIND>::f(acc, Elem<DT>::load(src[r * ld + c0 + e]));
+        }
+      }
+      for (int off = lanes >> 1; off >= 1; off >>= 1) acc = Op<KIND>::f(acc, __shfl_xor(acc, off, 64));
+      if (live && lane == 0) dst[r] = Elem<DT>::store(clear ? acc : Op<KIND>::f(Elem<DT>::load(dst[r]), acc));
+    }
+  }
+}
 
-template <int DT, int KIND> __global__ void __launch_bounds__(256)
-reduce_cols_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, int64_t ld, int clear, typename Elem<DT>::T* dst, float* partial, int vec_ok) {
+// along dim 0: a work-group owns a strip of 2^lanes_log2 x G columns and every gridDim.y-th chunk of rows; 2^lanes_log2 column
+// lanes x (256 >> lanes_log2) row lanes, kStripFlight rows in flight per lane.  The strip is kStripLanes x 16 bytes of every
+// row, or the power of two that covers a narrower view (of a dense one a wave then reads consecutive memory), or wider
+// when the view has too few rows to give every row lane a full set of loads.  Four rows in flight (2 to 16 measure within
+// 4 % of each other) when the view has many strips; a single strip gives one work-group per slice, 256 at most, and takes
+// 16 (5.5 against 4.2 TB/s on a 1M x 128 f16 view).  The row lanes combine by halving in LDS.
+constexpr int kStripLanes = 32;  // 16 and 64 lanes measured 9 % and 15 % slower on wide views
+
+template <int DT, int KIND, int kStripFlight> __global__ void __launch_bounds__(256)
+reduce_cols_kernel(const typename Elem<DT>::T* src, int64_t rows, int64_t cols, int64_t ld, int clear, typename Elem<DT>::T* dst, float* partial, int vec_ok,
+                   int lanes_log2) {
   typedef typename Elem<DT>::T T;
   constexpr int G = 16 / sizeof(T);
-  const int cl = threadIdx.x % kStripLanes, rl = threadIdx.x / kStripLanes;
-  const int64_t c0 = ((int64_t)blockIdx.x * kStripLanes + cl) * G;
-  const int64_t per = (rows + gridDim.y - 1) / gridDim.y;
-  const int64_t r0 = (int64_t)blockIdx.y * per, r1 = r0 + per < rows ? r0 + per : rows;
+  const int cl = threadIdx.x & ((1 << lanes_log2) - 1), rl = threadIdx.x >> lanes_log2, row_lanes = 256 >> lanes_log2;
+  const int64_t c0 = (((int64_t)blockIdx.x << lanes_log2) + cl) * G;
+  const int64_t chunk = (int64_t)kStripFlight * row_lanes;
   float acc[G];
 #pragma unroll
   for (int e = 0; e < G; ++e) acc[e] = Op<KIND>::id();
   if (c0 < cols) {
-    int64_t r = r0 + rl;
-    if (vec_ok && c0 + G <= cols) {
-      for (; r + (kStripFlight - 1) * kStripRows < r1; r += kStripFlight * kStripRows) {
+    const bool whole = vec_ok && c0 + G <= cols;
+    for (int64_t base = (int64_t)blockIdx.y * chunk; base < rows; base += (int64_t)gridDim.y * chunk) {
+      if (whole && base + chunk <= rows) {
         T in[kStripFlight][G];
 #pragma unroll
-        for (int u = 0; u < kStripFlight; ++u) *(v4u*)in[u] = load16(src + (r + kStripRows * u) * ld + c0);
+        for (int u = 0; u < kStripFlight; ++u) *(v4u*)in[u] = load16(src + (base + rl + (int64_t)row_lanes * u) * ld + c0);
 #pragma unroll
         for (int u = 0; u < kStripFlight; ++u)
 #pragma unroll
           for (int e = 0; e < G; ++e) acc[e] = Op<KIND>::f(acc[e], Elem<DT>::load(in[u][e]));
-      }
-    }
-    for (; r < r1; r += kStripRows) {
-      const T* p = src + r * ld + c0;
-      if (vec_ok && c0 + G <= cols) {
-        T in[G];
-        *(v4u*)in = load16(p);
-#pragma unroll
-        for (int e = 0; e < G; ++e) acc[e] = Op<KIND>::f(acc[e], Elem<DT>::load(in[e]));
       } else {
-        for (int e = 0; e < G && c0 + e < cols; ++e) acc[e] = Op<KIND>::f(acc[e], Elem<DT>::load(p[e]));
+        for (int64_t r = base + rl; r < rows && r < base + chunk; r += row_lanes) {
+          const T* p = src + r * ld + c0;
+          if (whole) {
+            T in[G];
+            *(v4u*)in = load16(p);
+#pragma unroll
+            for (int e = 0; e < G; ++e) acc[e] = Op<KIND>::f(acc[e], Elem<DT>::load(in[e]));
+          } else {
+            for (int e = 0; e < G && c0 + e < cols; ++e) acc[e] = Op<KIND>::f(acc[e], Elem<DT>::load(p[e]));
+          }
+        }
       }
     }
   }
-  __shared__ float red[kStripRows][kStripLanes][G + 1];
+  __shared__ float red[256][G + 1];  // [row lane * column lanes + column lane]
 #pragma unroll
-  for (int e = 0; e < G; ++e) red[rl][cl][e] = acc[e];
+  for (int e = 0; e < G; ++e) red[threadIdx.x][e] = acc[e];
   __syncthreads();
+  for (int half = row_lanes >> 1; half >= 1; half >>= 1) {
+    if (rl < half) {
+#pragma unroll
+      for (int e = 0; e < G; ++e) red[threadIdx.x][e] = Op<KIND>::f(red[threadIdx.x][e], red[threadIdx.x + (half << lanes_log2)][e]);
+    }
+    __syncthreads();
+  }
   if (rl == 0 && c0 < cols) {
-#pragma unroll
-    for (int e = 0; e < G; ++e) {
-      float v = red[0][cl][e];
-#pragma unroll
-      for (int k = 1; k < kStripRows; ++k) v = Op<KIND>::f(v, red[k][cl][e]);
-      if (c0 + e < cols) {
-        if (gridDim.y > 1) partial[(int64_t)blockIdx.y * cols + c0 + e] = v;
-        else dst[c0 + e] = Elem<DT>::store(clear ? v : Op<KIND>::f(Elem<DT>::load(dst[c0 + e]), v));
-      }
+    for (int e = 0; e < G && c0 + e < cols; ++e) {
+      const float v = red[cl][e];
+      if (gridDim.y > 1) partial[(int64_t)blockIdx.y * cols + c0 + e] = v;
+      else dst[c0 + e] = Elem<DT>::store(clear ? v : Op<KIND>::f(Elem<DT>::load(dst[c0 + e]), v));
     }
   }
 }
@@ -291,15 +341,37 @@ template <int SDT, int DDT> hipError_t copy_t(const void* src, int64_t sld, void
   return hipGetLastError();
 }
 
+// a launch may hold fewer than 2^32 lanes: grids are capped and work-groups loop
+constexpr int64_t kMaxGrid = 1 << 22;
+
 template <int DT, int KIND> hipError_t reduce_t(const void* src, int64_t rows, int64_t cols, int64_t ld, int dim, int clear, void* dst, float* partial,
                                                 int slices, int vec_ok, hipStream_t s) {
   typedef typename Elem<DT>::T T;
   constexpr int G = 16 / sizeof(T);
+  const int64_t gpr = (cols + G - 1) / G;
   if (dim == 1) {
-    hipLaunchKernelGGL((reduce_rows_kernel<DT, KIND>), dim3((unsigned)rows, (unsigned)slices), dim3(256), 0, s, (const T*)src, rows, cols, ld, clear, (T*)dst, partial, vec_ok);
+    if (gpr <= 256 && slices == 1) {
+      int lanes_log2 = 0;
+      while (lanes_log2 < 6 && (int64_t(1) << lanes_log2) < gpr) ++lanes_log2;
+      const int64_t rows_per_step = (256 >> lanes_log2) * (gpr <= 64 ? 4 : (gpr <= 128 ? 2 : 1)), blocks = (rows + rows_per_step - 1) / rows_per_step;
+      const dim3 grid((unsigned)(blocks < kMaxGrid ? blocks : kMaxGrid));
+      if (gpr <= 64) hipLaunchKernelGGL((reduce_short_rows_kernel<DT, KIND, 1>), grid, dim3(256), 0, s, (const T*)src, rows, cols, ld, clear, (T*)dst, vec_ok, lanes_log2);
+      else if (gpr <= 128) hipLaunchKernelGGL((reduce_short_rows_kernel<DT, KIND, 2>), grid, dim3(256), 0, s, (const T*)src, rows, cols, ld, clear, (T*)dst, vec_ok, lanes_log2);
+      else hipLaunchKernelGGL((reduce_short_rows_kernel<DT, KIND, 4>), grid, dim3(256), 0, s, (const T*)src, rows, cols, ld, clear, (T*)dst, vec_ok, lanes_log2);
+    } else {
+      hipLaunchKernelGGL((reduce_rows_kernel<DT, KIND>), dim3((unsigned)(rows < kMaxGrid ? rows : kMaxGrid), (unsigned)slices), dim3(256), 0, s, (const T*)src, rows, cols,
+                         ld, clear, (T*)dst, partial, vec_ok);
+    }
   } else {
-    const unsigned strips = (unsigned)((cols + kStripLanes * G - 1) / (kStripLanes * G));
-    hipLaunchKernelGGL((reduce_cols_kernel<DT, KIND>), dim3(strips, (unsigned)slices), dim3(256), 0, s, (const T*)src, rows, cols, ld, clear, (T*)dst, partial, vec_ok);
+    int lanes_log2 = 0;
+    while ((1 << lanes_log2) < kStripLanes && (int64_t(1) << lanes_log2) < gpr) ++lanes_log2;
+    while (lanes_log2 < 8 && (int64_t(1) << lanes_log2) < gpr && (256 >> lanes_log2) * 4 > rows) ++lanes_log2;  // few rows: wider strips
+    const unsigned strips = (unsigned)((gpr + (1 << lanes_log2) - 1) >> lanes_log2);
+    // a view of one strip gives at most one work-group per slice: its lanes keep more rows in flight instead
+    if (strips == 1) hipLaunchKernelGGL((reduce_cols_kernel<DT, KIND, 16>), dim3(strips, (unsigned)slices), dim3(256), 0, s, (const T*)src, rows, cols, ld, clear, (T*)dst,
+                                        partial, vec_ok, lanes_log2);
+    else hipLaunchKernelGGL((reduce_cols_kernel<DT, KIND, 4>), dim3(strips, (unsigned)slices), dim3(256), 0, s, (const T*)src, rows, cols, ld, clear, (T*)dst, partial,
+                            vec_ok, lanes_log2);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || slices == 1) return e;
@@ -325,7 +397,8 @@ int reduce_slices(int dtype, int64_t rows, int64_t cols, int dim) {
   const int es = dtype == FRISK_F32 ? 4 : 2;
   const int G = 16 / es;
   const int64_t groups = dim == 1 ? rows : (cols + kStripLanes * G - 1) / (kStripLanes * G);
-  const int64_t extent_bytes = dim == 1 ? cols * es : rows * kStripLanes * 16;  // bytes one work-group would walk unsplit
+  const int64_t strip_bytes = cols * es < kStripLanes * 16 ? cols * es : kStripLanes * 16;
+  const int64_t extent_bytes = dim == 1 ? cols * es : rows * strip_bytes;  // bytes one work-group would walk unsplit
   int slices = 1;
   while (groups * slices < 1024 && extent_bytes / (slices * 2) >= 16384 && slices < 256) slices *= 2;
   return slices;

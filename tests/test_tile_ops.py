@@ -141,7 +141,9 @@ def _close(dt, got, ref64):
     assert np.all(np.isfinite(g)) and np.all(np.abs(g - r) <= tol * np.maximum(scale, 1e-30)), float(np.max(np.abs(g - r) / np.maximum(scale, 1e-30)))
 
 
-REDUCE_VIEWS = [(1, 1, 0), (7, 5, 0), (64, 256, 0), (33, 1000, 3), (300, 9, 1), (4, 70000, 0), (70000, 4, 0), (2048, 2048, 0), (16, 1 << 18, 0), (1 << 16, 40, 8)]
+REDUCE_VIEWS = [(1, 1, 0), (7, 5, 0), (64, 256, 0), (33, 1000, 3), (300, 9, 1), (4, 70000, 0), (70000, 4, 0), (2048, 2048, 0), (16, 1 << 18, 0), (1 << 16, 40, 8),
+                # short rows shared by 1 ... 64 lanes with 1, 2 and 4 groups per lane; views narrower than a column strip
+                (1000, 24, 0), (999, 100, 4), (130, 600, 0), (77, 1500, 4), (50, 1003, 5), (1 << 17, 16, 0), (5000, 8, 0)]
 
 
 @pytest.mark.gpu
@@ -216,13 +218,16 @@ def test_softmax_status_codes_before_any_launch():
 
 
 SOFTMAX_VIEWS = [(1, 1, 0, 0), (3, 8, 0, 0), (7, 1000, 0, 0), (5, 1003, 3, 1), (64, 2048, 8, 0), (16, 4096, 0, 0), (9, 8192, 0, 0), (4, 16384, 0, 0),
-                 (3, 16392, 0, 0), (2, 70000, 0, 0), (300, 40, 0, 0)]
+                 (3, 16392, 0, 0), (2, 70000, 0, 0), (300, 40, 0, 0),
+                 # rows shared by 1 ... 64 lanes of a wave with 1, 2 and 4 groups per lane, whole and partial last groups
+                 (513, 8, 0, 0), (1000, 24, 0, 0), (999, 100, 4, 0), (130, 600, 0, 0), (77, 1500, 4, 0), (50, 1003, 5, 0), (31, 2040, 8, 0)]
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dt", FLOATS, ids=[NAMES[d] for d in FLOATS])
 def test_softmax_gpu(hip, dt):
-    """every path: rows in registers (1, 2, 4, 8 groups per lane), two sweeps (long rows), element by element (odd views);
+    """every path: rows shared by the lanes of a wave, a work-group per row with the row in registers (2, 4, 8 groups per
+    lane), two sweeps (long rows), element by element (odd views);
     bar: each element within 2e-3 (f16), 8e-3 (bf16), 2e-5 (f32) of the float64 value relative to max(|r|, rms), rows sum
     to one within that, log-sum within 1e-4"""
     import torch
