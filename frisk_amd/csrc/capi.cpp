@@ -462,8 +462,14 @@ int frisk_hip_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int
   return FRISK_OK;
 }
 
+size_t frisk_hip_softmax_workspace_bytes(int dtype, int64_t rows, int64_t cols) {
+  if ((dtype != FRISK_F32 && dtype != FRISK_F16 && dtype != FRISK_BF16) || rows <= 0 || cols <= 0) return 0;
+  const int slices = softmax_slices(dtype, rows, cols);
+  return slices > 1 ? (size_t)rows * (size_t)slices * 8 : 0;
+}
+
 int frisk_hip_softmax(int dtype, const void* src, int64_t src_ld, void* dst, int64_t dst_ld, int64_t rows, int64_t cols, float scale_log2, float* lse,
-                      void* stream) {
+                      void* workspace, size_t workspace_bytes, void* stream) {
   if (int st = check_view("softmax source", dtype, src, rows, cols, src_ld)) return st;
   if (int st = check_view("softmax destination", dtype, dst, rows, cols, dst_ld)) return st;
   if (!std::isfinite(scale_log2)) return fail(FRISK_ERR_ARGUMENT, "softmax scale %g is not finite", (double)scale_log2);
@@ -471,7 +477,10 @@ int frisk_hip_softmax(int dtype, const void* src, int64_t src_ld, void* dst, int
   if (rows == 0 || cols == 0) return FRISK_OK;
   if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
   const int rows_aligned = rows_on_16_bytes(dtype, src, src_ld) && rows_on_16_bytes(dtype, dst, dst_ld);
-  hipError_t e = launch_softmax_rows(dtype, src, src_ld, dst, dst_ld, rows, cols, scale_log2, lse, rows_aligned, (hipStream_t)stream);
+  int slices = softmax_slices(dtype, rows, cols);
+  // without a (large enough, 4-byte aligned) workspace the rows are not split: same result, fewer work-groups
+  if (slices > 1 && (!workspace || workspace_bytes < (size_t)rows * (size_t)slices * 8 || ((uintptr_t)workspace & 3))) slices = 1;
+  hipError_t e = launch_softmax_rows(dtype, src, src_ld, dst, dst_ld, rows, cols, scale_log2, lse, rows_aligned, (float*)workspace, slices, (hipStream_t)stream);
   if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "softmax launch failed: %s", hipGetErrorString(e));
   return FRISK_OK;
 }

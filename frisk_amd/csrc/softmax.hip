@@ -197,8 +197,67 @@ __global__ void __launch_bounds__(256) softmax_short_rows_kernel(const typename 
   }
 }
 
+// A few very long rows: a row is dealt to gridDim.y work-groups in runs of 256 groups (neighbouring work-groups read
+// neighbouring memory).  First launch: every work-group leaves the (maximum, sum) of its share in partial[row][slice];
+// second launch: every work-group merges the row's pairs and writes its share of exp2(x * c - log-sum).  Two reads and
+// one write per element, as in the two sweeps above, but on rows x slices work-groups instead of rows.
+template <int DT>
+__global__ void __launch_bounds__(256) softmax_split_stats_kernel(const typename SElem<DT>::T* src, int64_t sld, int64_t cols, float c, float* partial, int vec) {
+  typedef typename SElem<DT>::T T;
+  constexpr int G = 16 / (int)sizeof(T);
+  __shared__ float lds[8];
+  const T* x = src + (int64_t)blockIdx.x * sld;
+  MaxSum acc = {-INFINITY, 0.f};
+  if (vec) {
+    for (int64_t g = (int64_t)blockIdx.y * 256 + threadIdx.x; g < cols / G; g += (int64_t)gridDim.y * 256) {
+      T in[G];
+      *(v4u*)in = *(const v4u*)(x + g * G);
+#pragma unroll
+      for (int e = 0; e < G; ++e) acc.add(SElem<DT>::load(in[e]) * c);
+    }
+  } else {
+    for (int64_t j = (int64_t)blockIdx.y * 256 + threadIdx.x; j < cols; j += (int64_t)gridDim.y * 256) acc.add(SElem<DT>::load(x[j]) * c);
+  }
+  const MaxSum all = block_merge(acc, lds);
+  if (threadIdx.x == 0) {
+    float* out = partial + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * 2;
+    out[0] = all.m;
+    out[1] = all.l;
+  }
+}
+
+template <int DT>
+__global__ void __launch_bounds__(256) softmax_split_write_kernel(const typename SElem<DT>::T* src, int64_t sld, typename SElem<DT>::T* dst, int64_t dld, int64_t cols,
+                                                                  float c, float* lse, const float* partial, int vec) {
+  typedef typename SElem<DT>::T T;
+  constexpr int G = 16 / (int)sizeof(T);
+  __shared__ float lds[8];
+  const T* x = src + (int64_t)blockIdx.x * sld;
+  T* y = dst + (int64_t)blockIdx.x * dld;
+  MaxSum acc = {-INFINITY, 0.f};
+  for (int k = threadIdx.x; k < (int)gridDim.y; k += 256) {
+    const float* in = partial + ((int64_t)blockIdx.x * gridDim.y + k) * 2;
+    acc.merge(MaxSum{in[0], in[1]});
+  }
+  const MaxSum all = block_merge(acc, lds);
+  const float ref = all.m + __builtin_amdgcn_logf(all.l);  // log2 of the denominator
+  if (vec) {
+    for (int64_t g = (int64_t)blockIdx.y * 256 + threadIdx.x; g < cols / G; g += (int64_t)gridDim.y * 256) {
+      T in[G], out[G];
+      *(v4u*)in = __builtin_nontemporal_load((const v4u*)(x + g * G));
+#pragma unroll
+      for (int e = 0; e < G; ++e) out[e] = SElem<DT>::store(__builtin_amdgcn_exp2f(SElem<DT>::load(in[e]) * c - ref));
+      __builtin_nontemporal_store(*(const v4u*)out, (v4u*)(y + g * G));
+    }
+  } else {
+    for (int64_t j = (int64_t)blockIdx.y * 256 + threadIdx.x; j < cols; j += (int64_t)gridDim.y * 256)
+      y[j] = SElem<DT>::store(__builtin_amdgcn_exp2f(SElem<DT>::load(x[j]) * c - ref));
+  }
+  if (lse && blockIdx.y == 0 && threadIdx.x == 0) lse[blockIdx.x] = ref;
+}
+
 template <int DT> hipError_t launch_typed(const void* src, int64_t sld, void* dst, int64_t dld, int64_t rows, int64_t cols, float c, float* lse, int rows_aligned,
-                                          hipStream_t s) {
+                                          float* partial, int slices, hipStream_t s) {
   typedef typename SElem<DT>::T T;
   constexpr int G = 16 / (int)sizeof(T);
   const int vec = rows_aligned && cols % G == 0;
@@ -207,6 +266,12 @@ template <int DT> hipError_t launch_typed(const void* src, int64_t sld, void* ds
   const T* x = (const T*)src;
   T* y = (T*)dst;
   const int64_t groups = (cols + G - 1) / G;
+  if (slices > 1) {
+    const dim3 sgrid((unsigned)rows, (unsigned)slices);
+    hipLaunchKernelGGL((softmax_split_stats_kernel<DT>), sgrid, dim3(256), 0, s, x, sld, cols, c, partial, vec);
+    hipLaunchKernelGGL((softmax_split_write_kernel<DT>), sgrid, dim3(256), 0, s, x, sld, y, dld, cols, c, lse, (const float*)partial, vec);
+    return hipGetLastError();
+  }
   if (groups <= 256) {  // here a row that ends in a partial group still moves its whole groups 16 bytes at a time
     int lanes_log2 = 0;
     while (lanes_log2 < 6 && (int64_t(1) << lanes_log2) < groups) ++lanes_log2;
@@ -226,13 +291,21 @@ template <int DT> hipError_t launch_typed(const void* src, int64_t sld, void* ds
 
 }  // namespace
 
+int softmax_slices(int dtype, int64_t rows, int64_t cols) {
+  // Fewer than 1024 rows of at least 32 KiB: split each so that about 1024 work-groups exist, each with at least 16 KiB.
+  const int64_t row_bytes = cols * (dtype == FRISK_F32 ? 4 : 2);
+  int slices = 1;
+  while (rows * slices < 1024 && row_bytes / (slices * 2) >= 16384 && slices < 256) slices *= 2;
+  return slices;
+}
+
 // rows_aligned: pointers and leading dimensions put every row of both views on a 16-byte boundary
 hipError_t launch_softmax_rows(int dtype, const void* src, int64_t sld, void* dst, int64_t dld, int64_t rows, int64_t cols, float scale_log2, float* lse,
-                               int rows_aligned, hipStream_t s) {
+                               int rows_aligned, float* partial, int slices, hipStream_t s) {
   switch (dtype) {
-    case FRISK_F32: return launch_typed<FRISK_F32>(src, sld, dst, dld, rows, cols, scale_log2, lse, rows_aligned, s);
-    case FRISK_F16: return launch_typed<FRISK_F16>(src, sld, dst, dld, rows, cols, scale_log2, lse, rows_aligned, s);
-    default: return launch_typed<FRISK_BF16>(src, sld, dst, dld, rows, cols, scale_log2, lse, rows_aligned, s);
+    case FRISK_F32: return launch_typed<FRISK_F32>(src, sld, dst, dld, rows, cols, scale_log2, lse, rows_aligned, partial, slices, s);
+    case FRISK_F16: return launch_typed<FRISK_F16>(src, sld, dst, dld, rows, cols, scale_log2, lse, rows_aligned, partial, slices, s);
+    default: return launch_typed<FRISK_BF16>(src, sld, dst, dld, rows, cols, scale_log2, lse, rows_aligned, partial, slices, s);
   }
 }
 

@@ -16,5 +16,7 @@ hipError_t launch_reduce(int dtype, const void* src, int64_t rows, int64_t cols,
                          int vec_ok, hipStream_t s);
 // row softmax in base 2 (softmax.hip); rows_aligned: every row of both views starts on a 16-byte boundary
 hipError_t launch_softmax_rows(int dtype, const void* src, int64_t sld, void* dst, int64_t dld, int64_t rows, int64_t cols, float scale_log2, float* lse,
-                               int rows_aligned, hipStream_t s);
+                               int rows_aligned, float* partial, int slices, hipStream_t s);
+// work-groups a row is split over (1 = not split); a split needs rows * slices * 2 floats of workspace
+int softmax_slices(int dtype, int64_t rows, int64_t cols);
 }  // namespace frisk

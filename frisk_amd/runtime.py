@@ -70,7 +70,7 @@ _lib = None
 EXPORTS = ["frisk_hip_init", "frisk_hip_abi_version", "frisk_hip_last_error", "frisk_hip_plan", "frisk_hip_workspace_bytes",
            "frisk_hip_gemm", "frisk_hip_lds_access_cycles", "frisk_hip_lds_search", "frisk_hip_lds_offset", "frisk_hip_wave_partition",
            "frisk_hip_kernel_count", "frisk_hip_kernel_name", "frisk_hip_fill", "frisk_hip_copy", "frisk_hip_reduce",
-           "frisk_hip_reduce_workspace_bytes", "frisk_hip_attention", "frisk_hip_softmax"]
+           "frisk_hip_reduce_workspace_bytes", "frisk_hip_attention", "frisk_hip_softmax", "frisk_hip_softmax_workspace_bytes"]
 
 
 def lib():
@@ -104,7 +104,9 @@ def lib():
     L.frisk_hip_copy.argtypes = [ctypes.c_int, vp, i64, ctypes.c_int, vp, i64, i64, i64, vp]
     L.frisk_hip_reduce_workspace_bytes.restype = ctypes.c_size_t
     L.frisk_hip_reduce_workspace_bytes.argtypes = [ctypes.c_int, i64, i64, ctypes.c_int]
-    L.frisk_hip_softmax.argtypes = [ctypes.c_int, vp, i64, vp, i64, i64, i64, ctypes.c_float, vp, vp]
+    L.frisk_hip_softmax.argtypes = [ctypes.c_int, vp, i64, vp, i64, i64, i64, ctypes.c_float, vp, vp, ctypes.c_size_t, vp]
+    L.frisk_hip_softmax_workspace_bytes.argtypes = [ctypes.c_int, i64, i64]
+    L.frisk_hip_softmax_workspace_bytes.restype = ctypes.c_size_t
     L.frisk_hip_attention.argtypes = [ctypes.POINTER(AttentionDesc), vp, vp, vp, vp, vp, vp]
     L.frisk_hip_reduce.argtypes = [ctypes.c_int, vp, i64, i64, i64, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, ctypes.c_size_t, vp]
     if L.frisk_hip_abi_version() != ABI_VERSION:
@@ -183,9 +185,15 @@ def reduce(dtype, src_ptr, rows, cols, ld, dim, kind, clear, dst_ptr, workspace_
     _check(lib().frisk_hip_reduce(dtype, src_ptr, rows, cols, ld, dim, k, int(bool(clear)), dst_ptr, workspace_ptr, workspace_bytes, stream))
 
 
-def softmax(dtype, src_ptr, src_ld, dst_ptr, dst_ld, rows, cols, scale_log2=1.4426950408889634, lse_ptr=None, stream=None):
-    """row softmax in base 2: dst = 2^(scale_log2 * src) / row sum; the default scale makes it the natural softmax"""
-    _check(lib().frisk_hip_softmax(dtype, src_ptr, src_ld, dst_ptr, dst_ld, rows, cols, scale_log2, lse_ptr, stream))
+def softmax_workspace_bytes(dtype, rows, cols):
+    return int(lib().frisk_hip_softmax_workspace_bytes(dtype, rows, cols))
+
+
+def softmax(dtype, src_ptr, src_ld, dst_ptr, dst_ld, rows, cols, scale_log2=1.4426950408889634, lse_ptr=None, stream=None, workspace_ptr=None,
+            workspace_bytes=0):
+    """row softmax in base 2: dst = 2^(scale_log2 * src) / row sum; the default scale makes it the natural softmax.
+    A workspace of softmax_workspace_bytes lets a few very long rows be split over several work-groups each."""
+    _check(lib().frisk_hip_softmax(dtype, src_ptr, src_ld, dst_ptr, dst_ld, rows, cols, scale_log2, lse_ptr, workspace_ptr, workspace_bytes, stream))
 
 
 def make_attention_desc(dtype, batch, heads, seq_q, seq_k, head_dim=128, scale=None, k_transposed=False):

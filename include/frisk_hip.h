@@ -212,9 +212,12 @@ int frisk_hip_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int
  * on rank-2 views as above (F32, F16, BF16; arithmetic in fp32, result rounded to dtype).  scale_log2 is the sketch's
  * `cst`; a natural softmax with scale s is scale_log2 = s * log2(e).  lse (may be NULL) receives, per row, the
  * base-2 logarithm of the denominator, the sketch's `lse`.  dst may be src.  Rows of -inf only give NaN, as the
- * arithmetic does. */
+ * arithmetic does.  A few very long rows (fewer than 1024 rows of at least 32 KiB) are split over several work-groups
+ * each when the caller passes `workspace` (frisk_hip_softmax_workspace_bytes, pure host; 0 for other shapes); without
+ * one they run unsplit, a work-group per row. */
+size_t frisk_hip_softmax_workspace_bytes(int dtype, int64_t rows, int64_t cols);
 int frisk_hip_softmax(int dtype, const void* src, int64_t src_ld, void* dst, int64_t dst_ld, int64_t rows, int64_t cols,
-                      float scale_log2, float* lse, void* stream);
+                      float scale_log2, float* lse, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Fused attention forward: O = softmax(scale * Q K^T) V per (batch, head), the kernel sketched in the

@@ -215,25 +215,31 @@ def test_softmax_status_codes_before_any_launch():
     assert status(R.F16, p + 1, 8, p, 8, 4, 8) == R.ERR_ALIGNMENT
     assert status(R.F16, p, 8, p, 8, 4, 8, float("inf")) == R.ERR_ARGUMENT
     R.softmax(R.F16, None, 8, None, 8, 0, 8)                          # nothing to do
+    # pure host: only fewer than 1024 rows of at least 32 KiB ask for a workspace, 8 bytes per row and slice
+    assert R.softmax_workspace_bytes(R.F16, 8, 1 << 24) == 8 * 128 * 8 and R.softmax_workspace_bytes(R.F16, 128, 1 << 20) == 128 * 8 * 8
+    assert R.softmax_workspace_bytes(R.F16, 2000, 1 << 20) == 0 and R.softmax_workspace_bytes(R.F32, 4, 4096) == 0 and R.softmax_workspace_bytes(R.I8, 4, 1 << 20) == 0
 
 
 SOFTMAX_VIEWS = [(1, 1, 0, 0), (3, 8, 0, 0), (7, 1000, 0, 0), (5, 1003, 3, 1), (64, 2048, 8, 0), (16, 4096, 0, 0), (9, 8192, 0, 0), (4, 16384, 0, 0),
                  (3, 16392, 0, 0), (2, 70000, 0, 0), (300, 40, 0, 0),
                  # rows shared by 1 ... 64 lanes of a wave with 1, 2 and 4 groups per lane, whole and partial last groups
-                 (513, 8, 0, 0), (1000, 24, 0, 0), (999, 100, 4, 0), (130, 600, 0, 0), (77, 1500, 4, 0), (50, 1003, 5, 0), (31, 2040, 8, 0)]
+                 (513, 8, 0, 0), (1000, 24, 0, 0), (999, 100, 4, 0), (130, 600, 0, 0), (77, 1500, 4, 0), (50, 1003, 5, 0), (31, 2040, 8, 0),
+                 # long rows split over work-groups through the workspace: aligned, odd, padded
+                 (3, 300000, 0, 0), (2, 100003, 5, 1), (40, 32768, 8, 0)]
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dt", FLOATS, ids=[NAMES[d] for d in FLOATS])
 def test_softmax_gpu(hip, dt):
     """every path: rows shared by the lanes of a wave, a work-group per row with the row in registers (2, 4, 8 groups per
-    lane), two sweeps (long rows), element by element (odd views);
+    lane), two sweeps (long rows), long rows split over work-groups (with a workspace), element by element (odd views);
     bar: each element within 2e-3 (f16), 8e-3 (bf16), 2e-5 (f32) of the float64 value relative to max(|r|, rms), rows sum
     to one within that, log-sum within 1e-4"""
     import torch
     st = O.NP_STORAGE[dt]
     es = np.dtype(st).itemsize
     tol = {O.F32: 2e-5, O.F16: 2e-3, O.BF16: 8e-3}[dt]
+    floor = 2.0 ** -25 if dt == O.F16 else 0.0      # probabilities of very long rows are f16 subnormals: half a step of 2^-24
     stream = torch.cuda.current_stream().cuda_stream
     for rows, cols, pad, shift in SOFTMAX_VIEWS:
         for cst in (1.25, -0.4):
@@ -242,18 +248,24 @@ def test_softmax_gpu(hip, dt):
             src = np.zeros(shift + rows * ld, dtype=st)
             src[shift:].reshape(rows, ld)[:, :cols] = vals
             dst0 = np.full(shift + rows * ld, 0x7B7B7B7B if es == 4 else 0x7B7B, dtype=st)
-            dS, dD = _dev(src), _dev(dst0)
-            dL = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
-            hip.softmax(dt, dS.data_ptr() + shift * es, ld, dD.data_ptr() + shift * es, ld, rows, cols, cst, dL.data_ptr(), stream)
-            torch.cuda.synchronize()
-            got = _host(dD, st)
-            view = got[shift:].reshape(rows, ld)
             ref, lse = T.softmax_f64(dt, vals, cst)
-            g = O.decode(dt, np.ascontiguousarray(view[:, :cols]).reshape(-1)).astype(np.float64).reshape(rows, cols)
             scale = np.maximum(np.abs(ref), np.sqrt(np.mean(ref * ref)))
-            assert np.all(np.isfinite(g)) and np.all(np.abs(g - ref) <= tol * scale), (rows, cols, pad, shift, cst, float(np.max(np.abs(g - ref) / scale)))
-            assert np.abs(dL.cpu().numpy() - lse).max() <= 1e-4 * max(1.0, np.abs(lse).max()), (rows, cols)
-            assert np.array_equal(view[:, cols:], dst0[shift:].reshape(rows, ld)[:, cols:]) and np.array_equal(got[:shift], dst0[:shift])   # nothing outside the view
+            ws_bytes = hip.softmax_workspace_bytes(dt, rows, cols)
+            assert (ws_bytes > 0) == (cols * es >= 32768), (rows, cols)     # only a few very long rows are split
+            ws = torch.full((max(ws_bytes, 4),), 0xFF, dtype=torch.uint8, device="cuda")
+            dS = _dev(src)
+            for use_ws in ((False, True) if ws_bytes else (False,)):
+                dD = _dev(dst0)
+                dL = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
+                hip.softmax(dt, dS.data_ptr() + shift * es, ld, dD.data_ptr() + shift * es, ld, rows, cols, cst, dL.data_ptr(), stream,
+                            ws.data_ptr() if use_ws else None, ws_bytes if use_ws else 0)
+                torch.cuda.synchronize()
+                got = _host(dD, st)
+                view = got[shift:].reshape(rows, ld)
+                g = O.decode(dt, np.ascontiguousarray(view[:, :cols]).reshape(-1)).astype(np.float64).reshape(rows, cols)
+                assert np.all(np.isfinite(g)) and np.all(np.abs(g - ref) <= tol * scale + floor), (rows, cols, pad, shift, cst, use_ws, float(np.max(np.abs(g - ref) / scale)))
+                assert np.abs(dL.cpu().numpy() - lse).max() <= 1e-4 * max(1.0, np.abs(lse).max()), (rows, cols, use_ws)
+                assert np.array_equal(view[:, cols:], dst0[shift:].reshape(rows, ld)[:, cols:]) and np.array_equal(got[:shift], dst0[:shift])   # nothing outside the view
     # in place, and a masked column (-inf) gets probability exactly zero
     vals = O.encode(dt, O.normal(4 * 512, 44, 0, 1.0)).reshape(4, 512)
     vals[:, 17] = O.encode(dt, np.array([-np.inf], dtype=np.float32))[0]
