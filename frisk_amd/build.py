@@ -81,24 +81,28 @@ def build_ffi(verbose=True):
 
 
 def build_tools(verbose=True):
-    """the hardware probe behind the LDS cost model (frisk_amd/csrc/tools/lds_probe.hip) -> lib/lds_probe"""
-    out = os.path.join(LIBDIR, "lds_probe")
+    """the hardware probes the kernel designs rest on: the LDS cost model's (csrc/tools/lds_probe.hip -> lib/lds_probe) and the
+    matrix / vector pipe's (csrc/tools/pipe_probe.hip -> lib/pipe_probe)"""
     os.makedirs(LIBDIR, exist_ok=True)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           "-Wno-unused-value", os.path.join(CSRC, "tools", "lds_probe.hip"), "-o", out]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("building lds_probe failed:\n" + r.stderr)
-    if verbose:
-        print("built", out)
-    return out
+    outs = []
+    for name in ("lds_probe", "pipe_probe"):
+        out = os.path.join(LIBDIR, name)
+        cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               "-Wno-unused-value", os.path.join(CSRC, "tools", name + ".hip"), "-o", out]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("building %s failed:\n%s" % (name, r.stderr))
+        if verbose:
+            print("built", out)
+        outs.append(out)
+    return outs
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--if-missing", action="store_true")
     ap.add_argument("-j", type=int, default=None)
-    ap.add_argument("--tools", action="store_true", help="build only the hardware probe")
+    ap.add_argument("--tools", action="store_true", help="build only the hardware probes")
     a = ap.parse_args()
     if a.tools:
         build_tools()
