@@ -139,6 +139,18 @@ static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, in
   (void)nw;
 }
 
+// Tail split: a grid of a little more than a whole number of rounds of 256 tiles leaves most CUs idle in its last round.
+// With a kernel that has the split-K store path, the last tiles % 256 tiles (at most half a round) are computed by 2, 4 or
+// 8 work-groups each, every one taking an equal share of the K tiles (at least 4).  Returns that count, 1 for no split.
+static int tail_split_of(const KernelEntry* k, int64_t tiles, int64_t kt, bool whole_k_tiles) {
+  if (!k->splitk || k->bm < 128 || k->wk > 1 || !whole_k_tiles || tiles <= 256) return 1;
+  const int64_t rest = tiles % 256;
+  if (rest == 0 || rest > 128) return 1;
+  for (int s = 8; s >= 2; s /= 2)
+    if (rest * s <= 256 && kt % s == 0 && kt / s >= 4) return s;
+  return 1;
+}
+
 // Relative time of a problem on a kernel variant, used only to rank the variants.  One wave of work-groups = one per CU
 // (256); a K tile of a 256x256 tile costs 1.5 units when every CU runs one, and less when the chip is partly idle
 // (less contention in the L2 and a higher clock): factor 0.6 + 0.4 * fill.  The constants are measured on fp16 problems
@@ -172,6 +184,11 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
   const int64_t full = tiles / 256, rest = tiles % 256;
   const double rest_fill = (double)rest / 256.0;
   double cost = (double)full * kt * c;
+  if (const int ts = tail_split_of(k, tiles, (int64_t)kt, d->K % k->bk == 0); ts > 1) {
+    // the last `rest` tiles as ts work-groups each, a ts-th of the K tiles apiece, plus the pass that sums them
+    // (a dependent launch, and rest * ts tiles of 32-bit partial sums to read)
+    return cost + kt / ts * c * (0.6 + 0.4 * rest_fill * ts) + 5.0 + 0.04 * (double)(rest * ts);
+  }
   if (rest) {
     if (k->bm == 32)  // the skinny kernels are bound by streaming B and need the parallelism: idle CUs are lost bandwidth
       cost += full ? kt * c : kt * c / std::max(rest_fill, 0.25);
@@ -254,12 +271,20 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
     } else if (d->split_k == 0 && tiles < 256) {  // up to one work-group per CU, at least 4 K tiles per slice
       for (int c = 2; c <= 64; c *= 2)
         if (kt % c == 0 && kt / c >= 4 && tiles * c <= 256) split = c;
+    } else if (d->split_k == 0) {
+      const int ts = tail_split_of(k, tiles, kt, true);
+      if (ts > 1) {
+        plan->tail_split = ts;
+        plan->tail_tiles = (int)(tiles % 256);
+        plan->workspace_bytes = (size_t)ts * (size_t)plan->tail_tiles * (size_t)k->bm * (size_t)k->bn * 4;
+      }
     }
   } else if (d->split_k > 1 && !no_split) {
     return fail(FRISK_ERR_TILE, "split_k=%d: the chosen kernel %s has no split-K path", d->split_k, k->name);
   }
   plan->split_k = split;
   if (split > 1) plan->workspace_bytes = (size_t)split * (size_t)d->M * (size_t)d->N * 4;
+  if (plan->tail_split <= 1) { plan->tail_split = 1; plan->tail_tiles = 0; }
   return FRISK_OK;
 }
 
@@ -346,7 +371,7 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
     st = make_plan(desc, &plan, false, plan.guarded != 0, true);
     if (st != FRISK_OK) return st;
   }
-  if (plan.split_k > 1 && ((uintptr_t)workspace & 15)) return fail(FRISK_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
+  if ((plan.split_k > 1 || plan.tail_split > 1) && ((uintptr_t)workspace & 15)) return fail(FRISK_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
   if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
 
   GemmParams p;
@@ -363,12 +388,21 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
   const KernelEntry* k = kernels()[plan.kernel_id];
   p.split_k = plan.split_k;
   p.kt_per_slice = (int)((desc->K + k->bk - 1) / k->bk) / plan.split_k;
-  p.partial = plan.split_k > 1 ? workspace : nullptr;
+  p.partial = plan.split_k > 1 || plan.tail_split > 1 ? workspace : nullptr;
+  p.tail_split = plan.tail_split;
+  p.tail_tiles = plan.tail_tiles;
+  p.tail_from = p.tiles_m * p.tiles_n - plan.tail_tiles;
+  p.tail_kt = plan.tail_split > 1 ? p.kt_per_slice / plan.tail_split : 0;
+  p.tile_m = k->bm; p.tile_n = k->bn;
   hipError_t e = k->launch(p, (hipStream_t)stream);
   if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "launch of %s failed: %s", k->name, hipGetErrorString(e));
   if (plan.split_k > 1) {
     e = launch_splitk_reduce(p, desc->dtype_acc == FRISK_I32, (hipStream_t)stream);
     if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "launch of the split-K reduction failed: %s", hipGetErrorString(e));
+  }
+  if (plan.tail_split > 1) {
+    e = launch_tail_reduce(p, desc->dtype_acc == FRISK_I32, (hipStream_t)stream);
+    if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "launch of the tail reduction failed: %s", hipGetErrorString(e));
   }
   return FRISK_OK;
 }

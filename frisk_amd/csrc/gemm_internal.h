@@ -21,7 +21,32 @@ struct GemmParams {
   // slice the kernel writes raw 32-bit accumulators to partial[slice][M][N] and a second kernel sums the slices.
   int split_k, kt_per_slice;
   void* partial;
+  // Tail split: the last `tail_tiles` tiles of a grid that is a little more than a whole number of rounds of 256 are
+  // each computed by `tail_split` work-groups, `tail_kt` K tiles apiece.  Work-group ids from `tail_from` on are tail
+  // units (tile = tail_from + unit / tail_split, slice = unit % tail_split); they leave raw accumulators in
+  // partial[slice][tile - tail_from][BM][BN] and a second kernel sums them.  tail_split <= 1: no tail.
+  int tail_from, tail_tiles, tail_split, tail_kt;
+  int tile_m, tile_n;  // BM, BN of the kernel (for the tail reduction)
 };
+
+// Hardware hands consecutive work-group ids to the 8 XCDs round-robin.  Give each XCD a contiguous range of "compact"
+// ids, then walk the tile grid in column-major order inside bands of GM tile rows, so the work-groups resident on one
+// XCD (one L2) cover a GM x (resident/GM) block of tiles.
+__host__ __device__ inline void tile_of_workgroup(int wg, int tiles_m, int tiles_n, int gm, int xcd_remap, int& tm, int& tn) {
+  int total = tiles_m * tiles_n;
+  int cid = wg;
+  if (xcd_remap) {
+    int per = total >> 3;
+    if (wg < per * 8) cid = (wg & 7) * per + (wg >> 3);
+  }
+  int band = gm * tiles_n;
+  int b = cid / band;
+  int first_m = b * gm;
+  int rows = tiles_m - first_m < gm ? tiles_m - first_m : gm;
+  int in = cid - b * band;
+  tm = first_m + in % rows;
+  tn = in / rows;
+}
 
 // One compiled kernel variant.
 struct KernelEntry {
@@ -40,6 +65,8 @@ struct KernelEntry {
 
 // sums the split-K slices and applies the epilogue (splitk_reduce.hip)
 hipError_t launch_splitk_reduce(const GemmParams& p, int acc_is_int, hipStream_t stream);
+// the same for the tiles of a tail split
+hipError_t launch_tail_reduce(const GemmParams& p, int acc_is_int, hipStream_t stream);
 
 // defined in kernels_*.hip
 extern const KernelEntry kKernelsF16[];

@@ -47,7 +47,8 @@ class GemmPlan(ctypes.Structure):
                 ("mfma_k", ctypes.c_int32), ("stages", ctypes.c_int32), ("stages_b", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
                 ("grid_x", ctypes.c_int32), ("grid_y", ctypes.c_int32), ("split_k", ctypes.c_int32),
                 ("xcd_remap", ctypes.c_int32), ("guarded", ctypes.c_int32), ("lds_a", LdsLayout), ("lds_b", LdsLayout),
-                ("workspace_bytes", ctypes.c_size_t), ("flops", ctypes.c_double), ("bytes", ctypes.c_double)]
+                ("workspace_bytes", ctypes.c_size_t), ("flops", ctypes.c_double), ("bytes", ctypes.c_double),
+                ("tail_tiles", ctypes.c_int32), ("tail_split", ctypes.c_int32)]
 
 
 class AttentionDesc(ctypes.Structure):

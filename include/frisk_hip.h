@@ -122,6 +122,9 @@ typedef struct frisk_gemm_plan {
   size_t workspace_bytes;
   double flops;                      /* 2.M.N.K */
   double bytes;                      /* |A| + |B| + |C| (+ scales) */
+  int32_t tail_tiles, tail_split;    /* tail_split > 1: the last tail_tiles tiles (grid % 256, a partly filled last round) are
+                                        computed by tail_split work-groups each, a share of the K tiles apiece, and summed
+                                        through the workspace */
 } frisk_gemm_plan;
 
 int frisk_hip_abi_version(void);
@@ -138,7 +141,8 @@ const char* frisk_hip_last_error(void);
 int frisk_hip_plan(const frisk_gemm_desc* desc, frisk_gemm_plan* plan);
 
 /* Pure host: bytes of device workspace `frisk_hip_gemm` wants for this descriptor: split_k * M * N * 4 when the
- * plan splits K, else 0.  With split_k = 0 in the descriptor a launch without workspace still runs, unsplit. */
+ * plan splits K, tail_split * tail_tiles * tile_m * tile_n * 4 for a tail split, else 0.  With split_k = 0 in the
+ * descriptor a launch without workspace still runs, unsplit. */
 size_t frisk_hip_workspace_bytes(const frisk_gemm_desc* desc);
 
 /* Launch on `stream` (a hipStream_t, may be NULL for the default stream).

@@ -340,6 +340,53 @@ def test_split_k_status_codes(hip):
     assert e.value.status == hip.ERR_TILE
 
 
+# ------------------------------------------------------------------ grids a little over a whole number of rounds: tail split
+@pytest.mark.parametrize("dtype,transA,transB", [(O.F16, 0, 0), (O.BF16, 0, 1), (O.F16, 1, 0), (O.BF16, 1, 1), (O.I8, 0, 0), (O.E4M3, 0, 1)])
+def test_tail_split(hip, dtype, transA, transB):
+    """17 x 17 = 289 tiles of 256 x 256: one round of 256 and 33 left over, which run as 4 work-groups each (a quarter of the
+    16 K tiles apiece) and are summed through the workspace; without a workspace the same launch runs unsplit.  Both give
+    the oracle's result (int8: the same bits)"""
+    M = N = 17 * 256
+    K = 16 * BK[dtype]
+    sa, sb = stored_shapes(M, N, K, transA, transB)
+    A = make_operand(dtype, *sa, seed=61, tensor=0, scale=0.5)
+    B = make_operand(dtype, *sb, seed=61, tensor=1, scale=0.5)
+    out_dt = DEFAULT_OUT[dtype]
+    ref = O.gemm_i32(A, B, transA, transB) if dtype == O.I8 else O.gemm_f64(dtype, A, B, transA, transB)
+    p = hip.plan(hip.make_desc(dtype, M, N, K, dtype_out=out_dt, transA=bool(transA), transB=bool(transB)))
+    assert (p.tile_m, p.tile_n, p.tail_tiles, p.tail_split) == (256, 256, 33, 4) and p.workspace_bytes == 4 * 33 * 256 * 256 * 4
+    for workspace in (True, False):
+        note(f"case tail split {NAMES[dtype]} tA={transA} tB={transB} {M}x{N}x{K} workspace={workspace}")
+        got = run_gemm(hip, dtype, A, B, transA, transB, out_dt, M, N, K, workspace=workspace)
+        if dtype == O.I8:
+            assert np.array_equal(got, ref)
+        else:
+            check(dtype, out_dt, got, ref)
+
+
+def test_tail_split_epilogues_and_accumulate(hip):
+    M = N = 17 * 256
+    K = 16 * 128
+    A = make_operand(O.I8, M, K, seed=62, tensor=0)
+    B = make_operand(O.I8, K, N, seed=62, tensor=1)
+    sA, sB = O.uniform(M, 62, 2, 0.001, 0.02), O.uniform(N, 62, 3, 0.001, 0.02)
+    acc = O.gemm_i32(A, B)
+    note("case tail split int8 dequant epilogue")
+    got = run_gemm(hip, O.I8, A, B, 0, 0, O.F16, M, N, K, epilogue=hip.EPI_ROW_COL_SCALE, sA=sA, sB=sB)
+    assert np.array_equal(got, O.epilogue_rowcol_f16(acc, sA, sB))
+    C0 = (np.arange(M * N, dtype=np.int64).reshape(M, N) % 91 - 45).astype(np.int32)
+    note("case tail split int8 accumulate into int32")
+    goti = run_gemm(hip, O.I8, A, B, 0, 0, O.I32, M, N, K, C_init=C0, clear_accum=False)
+    assert np.array_equal(goti, acc + C0)
+    K = 16 * 64
+    Ah = make_operand(O.F16, M, K, seed=63, tensor=0, scale=0.5)
+    Bh = make_operand(O.F16, N, K, seed=63, tensor=1, scale=0.5)
+    C0f = O.uniform(M * N, 63, 2, -1.0, 1.0).reshape(M, N).astype(np.float32)
+    note("case tail split fp16 -> fp32 accumulate, padded ldc")
+    gotf = run_gemm(hip, O.F16, Ah, Bh, 0, 1, O.F32, M, N, K, C_init=C0f, clear_accum=False, pad=8)
+    check(O.F16, O.F32, gotf, O.gemm_f64(O.F16, Ah, Bh, False, True) + C0f.astype(np.float64))
+
+
 def test_config_fp8_skinny_decode(hip):
     """M = 32, N = K = 8192, e4m3 with per-tensor scales, bf16 output: every row checked"""
     M, N, K = 32, 8192, 8192

@@ -218,5 +218,12 @@ def test_planner_ranks_variants_by_estimated_time():
     assert pick(R.E4M3, 32, 16384, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s2_splitk"
     assert pick(R.E4M3, 32, 32768, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s2_splitk"
     assert pick(R.F16, 1024, 1024, 1024) == "f16_nn_32x128x64_w1x4_s3_splitk"
-    assert pick(R.I8, 6144, 6144, 6144) == "i8_nn_256x256x128_w2x2_s2x3"
+    # 576 tiles = 2 rounds + 64: the variant with the split-K store path, its last 64 tiles as 4 work-groups each
+    assert pick(R.I8, 6144, 6144, 6144) == "i8_nn_256x256x128_w2x2_s2x3_splitk"
+    p = R.plan(R.make_desc(R.I8, 6144, 6144, 6144, dtype_out=R.I32))
+    assert (p.tail_tiles, p.tail_split, p.split_k) == (64, 4, 1) and p.workspace_bytes == 4 * 64 * 256 * 256 * 4
+    # whole rounds, more than half a round left over, or a descriptor that forbids splitting: no tail
+    for shape, kw in (((8192, 8192, 8192), {}), ((5120, 5120, 5120), {}), ((6144, 6144, 6144), {"split_k": 1})):
+        p = R.plan(R.make_desc(R.F16, *shape, **kw))
+        assert (p.tail_tiles, p.tail_split) == (0, 1) and p.workspace_bytes == 0, shape
     assert not pick(R.F16, 64, 384, 2048).endswith("_guard") and pick(R.F16, 65, 384, 2048).endswith("_guard")
