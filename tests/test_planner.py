@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_plans_of_the_benchmark_configurations():
     cases = [
-        (R.F32, 1024, 1024, 1024, 0, 0, R.F32, (64, 64, 64)),
+        (R.F32, 1024, 1024, 1024, 0, 0, R.F32, (64, 64, 128)),   # 8 waves: two sets of four share each K tile
         (R.F16, 4096, 4096, 4096, 0, 0, R.F16, (256, 256, 64)),
         (R.BF16, 8192, 8192, 8192, 0, 1, R.BF16, (256, 256, 64)),
         (R.I8, 4096, 4096, 4096, 0, 0, R.F16, (256, 256, 128)),
@@ -40,7 +40,7 @@ def test_plans_of_the_benchmark_configurations():
         assert (p.tile_m, p.tile_n, p.tile_k) == tile
         assert p.grid_x == N // tile[1] and p.grid_y == M // tile[0]
         assert p.grid_x * p.grid_y >= 256 and p.xcd_remap == 1
-        assert p.threads == 64 * p.waves_m * p.waves_n and p.lds_bytes <= 160 * 1024
+        assert p.threads == 64 * p.waves_m * p.waves_n * p.waves_k and p.lds_bytes <= 160 * 1024
         assert p.mfma_m == 32 and p.mfma_n == 32
         assert p.flops == 2.0 * M * N * K
         assert p.lds_a.k_contiguous == (0 if tA else 1) and p.lds_b.k_contiguous == (1 if tB else 0)
