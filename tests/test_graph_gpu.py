@@ -65,3 +65,63 @@ def test_gemm_split_k_and_reduce_replay_from_a_graph(hip):
     B = dB.cpu().numpy().view(np.uint16).reshape(K, N)
     r = O.compare(O.F16, want[0].view(np.uint16).reshape(M, N), O.gemm_f64(O.F16, A, B))
     assert r["max_rel"] <= 1e-2 and r["fro_rel"] <= 1e-2, r
+
+
+def test_tail_split_softmax_split_and_attention_replay_from_a_graph(hip):
+    """the two-launch paths added later (GEMM tail split + its reduction, softmax of a few long rows split over work-groups)
+    and the attention kernel, captured and replayed: same bits as eager"""
+    import torch
+    hip.init()
+    M = N = 17 * 256
+    K = 1024
+    dA = to_dev(make_operand(O.F16, M, K, seed=81, tensor=0, scale=0.25))
+    dB = to_dev(make_operand(O.F16, K, N, seed=81, tensor=1, scale=0.25))
+    dC = torch.zeros(M * N * 2, dtype=torch.uint8, device="cuda")
+    dg = hip.make_desc(O.F16, M, N, K)
+    pg = hip.plan(dg)
+    assert pg.tail_split == 4 and pg.workspace_bytes > 0
+    wsg = torch.empty(pg.workspace_bytes, dtype=torch.uint8, device="cuda")
+    rows, cols = 4, 1 << 17
+    dX = to_dev(make_operand(O.F16, rows, cols, seed=82, tensor=0, scale=2.0))
+    dY = torch.zeros(rows * cols * 2, dtype=torch.uint8, device="cuda")
+    wss_bytes = hip.softmax_workspace_bytes(O.F16, rows, cols)
+    assert wss_bytes > 0
+    wss = torch.empty(wss_bytes, dtype=torch.uint8, device="cuda")
+    heads, seq = 2, 512
+    dQ = to_dev(make_operand(O.F16, heads * seq, 128, seed=83, tensor=0, scale=1.0))
+    dK = to_dev(make_operand(O.F16, heads * seq, 128, seed=83, tensor=1, scale=1.0))
+    dV = to_dev(make_operand(O.F16, heads * seq, 128, seed=83, tensor=2, scale=1.0))
+    dO = torch.zeros(heads * seq * 128 * 2, dtype=torch.uint8, device="cuda")
+    da = hip.make_attention_desc(O.F16, 1, heads, seq, seq)
+
+    def launches(stream):
+        hip.gemm(dg, dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), None, None, wsg.data_ptr(), wsg.numel(), stream)
+        hip.softmax(O.F16, dX.data_ptr(), cols, dY.data_ptr(), cols, rows, cols, 1.25, None, stream, wss.data_ptr(), wss.numel())
+        hip.attention(da, dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(), dO.data_ptr(), None, stream)
+
+    def snapshot():
+        torch.cuda.synchronize()
+        return dC.cpu().numpy().copy(), dY.cpu().numpy().copy(), dO.cpu().numpy().copy()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launches(side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launches(torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        dA.copy_(to_dev(make_operand(O.F16, M, K, seed=90 + rep, tensor=0, scale=0.25)))
+        dX.copy_(to_dev(make_operand(O.F16, rows, cols, seed=90 + rep, tensor=1, scale=2.0)))
+        dQ.copy_(to_dev(make_operand(O.F16, heads * seq, 128, seed=90 + rep, tensor=2, scale=1.0)))
+        launches(torch.cuda.current_stream().cuda_stream)
+        want = snapshot()
+        for t in (dC, dY, dO, wsg, wss):
+            t.fill_(0xA5)
+        torch.cuda.synchronize()
+        graph.replay()
+        got = snapshot()
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w), "replay %d differs from the eager launches" % rep
