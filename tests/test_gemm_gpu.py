@@ -364,6 +364,19 @@ def test_tail_split(hip, dtype, transA, transB):
             check(dtype, out_dt, got, ref)
 
 
+def test_tail_split_with_the_xcd_tile_map(hip):
+    """11 x 24 = 264 tiles, a multiple of 8, so work-group ids are regrouped per XCD; the 8 tiles left over after one round run as
+    8 work-groups each (2 of the 16 K tiles apiece would be too few: 32 K tiles, 4 apiece)"""
+    M, N, K = 11 * 256, 24 * 256, 32 * 64
+    A = make_operand(O.F16, M, K, seed=64, tensor=0, scale=0.5)
+    B = make_operand(O.F16, N, K, seed=64, tensor=1, scale=0.5)
+    p = hip.plan(hip.make_desc(O.F16, M, N, K, transB=True))
+    assert (p.tail_tiles, p.tail_split, p.xcd_remap) == (8, 8, 1)
+    note(f"case tail split with xcd map {M}x{N}x{K}")
+    got = run_gemm(hip, O.F16, A, B, 0, 1, O.F16, M, N, K)
+    check(O.F16, O.F16, got, O.gemm_f64(O.F16, A, B, False, True))
+
+
 def test_tail_split_epilogues_and_accumulate(hip):
     M = N = 17 * 256
     K = 16 * 128
