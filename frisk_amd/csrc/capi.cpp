@@ -220,23 +220,31 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   int best = -1;
   double best_cost = 0.0;
   bool any_layout = false, tile_requested = d->tile_m || d->tile_n || d->tile_k || d->waves_m || d->waves_n || d->stages;
-  for (size_t i = 0; i < ks.size(); ++i) {
-    const KernelEntry* k = ks[i];
-    if (k->dtype != d->dtype_ab || k->transA != (d->transA != 0) || k->transB != (d->transB != 0)) continue;
-    any_layout = true;
-    if (d->tile_m && d->tile_m != k->bm) continue;
-    if (d->tile_n && d->tile_n != k->bn) continue;
-    if (d->tile_k && d->tile_k != k->bk) continue;
-    if (d->waves_m && d->waves_m != k->wm) continue;
-    if (d->waves_n && d->waves_n != k->wn) continue;
-    if (d->stages && d->stages != k->stages_b) continue;  // the deeper ring names the variant
-    // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
-    if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
-    if (k->guard && best >= 0 && !ks[best]->guard) continue;  // never a guarded kernel when a fast one fits
-    const double cost = estimated_cost(k, d);
-    // ties: the first listed variant is the tuned default
-    if (best < 0 || (ks[best]->guard && !k->guard) || cost < best_cost) { best = (int)i; best_cost = cost; }
-  }
+  auto search = [&](bool want_split) {
+    for (size_t i = 0; i < ks.size(); ++i) {
+      const KernelEntry* k = ks[i];
+      if (k->dtype != d->dtype_ab || k->transA != (d->transA != 0) || k->transB != (d->transB != 0)) continue;
+      any_layout = true;
+      if (d->tile_m && d->tile_m != k->bm) continue;
+      if (d->tile_n && d->tile_n != k->bn) continue;
+      if (d->tile_k && d->tile_k != k->bk) continue;
+      if (d->waves_m && d->waves_m != k->wm) continue;
+      if (d->waves_n && d->waves_n != k->wn) continue;
+      if (d->stages && d->stages != k->stages_b) continue;  // the deeper ring names the variant
+      if (want_split && !k->splitk) continue;
+      // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
+      if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
+      if (k->guard && best >= 0 && !ks[best]->guard) continue;  // never a guarded kernel when a fast one fits
+      const double cost = estimated_cost(k, d);
+      // ties: the first listed variant is the tuned default
+      if (best < 0 || (ks[best]->guard && !k->guard) || cost < best_cost) { best = (int)i; best_cost = cost; }
+    }
+  };
+  // an explicit split_k looks among the variants with the split-K store path first; if none of them fits, the choice among
+  // all variants reports below that it cannot split
+  const bool explicit_split = d->split_k > 1 && !no_split;
+  search(explicit_split);
+  if (best < 0 && explicit_split) search(false);
   if (d->M == 0 || d->N == 0) {  // nothing to compute
     plan->grid_x = plan->grid_y = 0;
     return FRISK_OK;

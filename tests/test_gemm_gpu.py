@@ -333,11 +333,14 @@ def test_split_k_status_codes(hip):
     with pytest.raises(hip.FriskHipError) as e:
         hip.gemm(d, buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), None, None, None, 0, None)
     assert e.value.status == hip.ERR_WORKSPACE
-    # a kernel without the split path refuses an explicit split
-    d = hip.make_desc(O.F16, 256, 256, 2048, transA=True, split_k=4)
+    # no fp32 kernel has the split path: an explicit split is refused
+    d = hip.make_desc(O.F32, 256, 256, 2048, split_k=4)
     with pytest.raises(hip.FriskHipError) as e:
         hip.plan(d)
     assert e.value.status == hip.ERR_TILE
+    # an explicit split looks for a variant that can split: the 256 x 256 tile has one in every layout
+    p = hip.plan(hip.make_desc(O.F16, 256, 256, 2048, transA=True, split_k=4))
+    assert p.split_k == 4 and hip.kernel_names()[p.kernel_id].endswith("_splitk")
 
 
 # ------------------------------------------------------------------ grids a little over a whole number of rounds: tail split
@@ -362,6 +365,21 @@ def test_tail_split(hip, dtype, transA, transB):
             assert np.array_equal(got, ref)
         else:
             check(dtype, out_dt, got, ref)
+
+
+def test_explicit_split_k_on_the_large_tile(hip):
+    """512 x 512 x 4096 on 256 x 256 tiles with split_k = 8: 4 tiles x 8 slices, summed by the reduction kernel"""
+    M, N, K = 512, 512, 4096
+    A = make_operand(O.F16, K, M, seed=65, tensor=0, scale=0.5)   # stored transposed
+    B = make_operand(O.F16, K, N, seed=65, tensor=1, scale=0.5)
+    note("case explicit split_k=8 on 256x256 tiles, TN")
+    got = run_gemm(hip, O.F16, A, B, 1, 0, O.F16, M, N, K, tile=(256, 256, 64), split_k=8)
+    check(O.F16, O.F16, got, O.gemm_f64(O.F16, A, B, True, False))
+    Ai = make_operand(O.I8, M, K, seed=66, tensor=0)
+    Bi = make_operand(O.I8, K, N, seed=66, tensor=1)
+    note("case explicit split_k=4 on 256x256 tiles, int8")
+    goti = run_gemm(hip, O.I8, Ai, Bi, 0, 0, O.I32, M, N, K, tile=(256, 256, 128), split_k=4)
+    assert np.array_equal(goti, O.gemm_i32(Ai, Bi))
 
 
 def test_tail_split_with_the_xcd_tile_map(hip):
