@@ -147,7 +147,7 @@ static int tail_split_of(const KernelEntry* k, int64_t tiles, int64_t kt, bool w
   const int64_t rest = tiles % 256;
   if (rest == 0 || rest > 128) return 1;
   for (int s = 8; s >= 2; s /= 2)
-    if (rest * s <= 256 && kt % s == 0 && kt / s >= 4) return s;
+    if (rest * s <= 256 && kt % s == 0 && kt / s >= 8) return s;  // shallower slices do not repay the second launch (measured)
   return 1;
 }
 

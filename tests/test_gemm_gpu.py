@@ -347,10 +347,10 @@ def test_split_k_status_codes(hip):
 @pytest.mark.parametrize("dtype,transA,transB", [(O.F16, 0, 0), (O.BF16, 0, 1), (O.F16, 1, 0), (O.BF16, 1, 1), (O.I8, 0, 0), (O.E4M3, 0, 1)])
 def test_tail_split(hip, dtype, transA, transB):
     """17 x 17 = 289 tiles of 256 x 256: one round of 256 and 33 left over, which run as 4 work-groups each (a quarter of the
-    16 K tiles apiece) and are summed through the workspace; without a workspace the same launch runs unsplit.  Both give
+    32 K tiles apiece) and are summed through the workspace; without a workspace the same launch runs unsplit.  Both give
     the oracle's result (int8: the same bits)"""
     M = N = 17 * 256
-    K = 16 * BK[dtype]
+    K = 32 * BK[dtype]
     sa, sb = stored_shapes(M, N, K, transA, transB)
     A = make_operand(dtype, *sa, seed=61, tensor=0, scale=0.5)
     B = make_operand(dtype, *sb, seed=61, tensor=1, scale=0.5)
@@ -384,8 +384,8 @@ def test_explicit_split_k_on_the_large_tile(hip):
 
 def test_tail_split_with_the_xcd_tile_map(hip):
     """11 x 24 = 264 tiles, a multiple of 8, so work-group ids are regrouped per XCD; the 8 tiles left over after one round run as
-    8 work-groups each (2 of the 16 K tiles apiece would be too few: 32 K tiles, 4 apiece)"""
-    M, N, K = 11 * 256, 24 * 256, 32 * 64
+    8 work-groups each, 8 of the 64 K tiles apiece"""
+    M, N, K = 11 * 256, 24 * 256, 64 * 64
     A = make_operand(O.F16, M, K, seed=64, tensor=0, scale=0.5)
     B = make_operand(O.F16, N, K, seed=64, tensor=1, scale=0.5)
     p = hip.plan(hip.make_desc(O.F16, M, N, K, transB=True))
@@ -397,7 +397,7 @@ def test_tail_split_with_the_xcd_tile_map(hip):
 
 def test_tail_split_epilogues_and_accumulate(hip):
     M = N = 17 * 256
-    K = 16 * 128
+    K = 32 * 128
     A = make_operand(O.I8, M, K, seed=62, tensor=0)
     B = make_operand(O.I8, K, N, seed=62, tensor=1)
     sA, sB = O.uniform(M, 62, 2, 0.001, 0.02), O.uniform(N, 62, 3, 0.001, 0.02)
@@ -409,7 +409,7 @@ def test_tail_split_epilogues_and_accumulate(hip):
     note("case tail split int8 accumulate into int32")
     goti = run_gemm(hip, O.I8, A, B, 0, 0, O.I32, M, N, K, C_init=C0, clear_accum=False)
     assert np.array_equal(goti, acc + C0)
-    K = 16 * 64
+    K = 32 * 64
     Ah = make_operand(O.F16, M, K, seed=63, tensor=0, scale=0.5)
     Bh = make_operand(O.F16, N, K, seed=63, tensor=1, scale=0.5)
     C0f = O.uniform(M * N, 63, 2, -1.0, 1.0).reshape(M, N).astype(np.float32)

@@ -73,7 +73,7 @@ def test_tail_split_softmax_split_and_attention_replay_from_a_graph(hip):
     import torch
     hip.init()
     M = N = 17 * 256
-    K = 1024
+    K = 2048
     dA = to_dev(make_operand(O.F16, M, K, seed=81, tensor=0, scale=0.25))
     dB = to_dev(make_operand(O.F16, K, N, seed=81, tensor=1, scale=0.25))
     dC = torch.zeros(M * N * 2, dtype=torch.uint8, device="cuda")
