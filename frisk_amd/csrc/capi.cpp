@@ -120,8 +120,8 @@ static int validate(const frisk_gemm_desc* d) {
   return FRISK_OK;
 }
 
-static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, int mn, int bk, int nw, bool with_model) {
-  TileShape t{kcontig ? mn : bk, (kcontig ? bk : mn) * es, kcontig, es, fragb, mn, bk};
+static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, int mn, int bk, int nw, bool with_model, int atom) {
+  TileShape t{kcontig ? mn : bk, (kcontig ? bk : mn) * es, kcontig, es, fragb, mn, bk, atom};
   Swizzle s = default_swizzle(kcontig, es, t.rowb);
   L->rows = t.rows;
   L->row_bytes = t.rowb;
@@ -130,8 +130,8 @@ static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, in
   L->row_mask = s.mk;
   L->chunk_shift = s.cs;
   L->read_instr = es == 4 ? 3 : (kcontig ? 0 : (es == 2 ? 1 : 2));
-  int atoms = mn / 32 < 4 ? mn / 32 : 4;
-  int n_access = atoms * ((bk * es) / (2 * fragb)) * frag_instr_count(kcontig, es, fragb);
+  int atoms = mn / atom < 4 ? mn / atom : 4;
+  int n_access = atoms * ((bk * es) / frag_kstep_bytes(fragb, atom)) * frag_instr_count(kcontig, es, fragb);
   // evaluating the bank model costs ~0.1 ms of host time: only when the caller asks for the plan
   L->read_cycles = (with_model && n_access) ? (float)swizzle_read_cycles(t, s) / (float)n_access : 0.f;
   // the direct-to-LDS transfer writes 64 consecutive 16-byte slots: no conflicts by construction
@@ -171,6 +171,10 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
     c = k->wk > 1 ? 0.8 : (elem_size(k->dtype) == 1 ? 0.85 : 0.25);
   } else if (area >= 256 * 256) {
     c = k->wm * k->wn > 4 ? 1.56 : (k->stages_b > k->stages ? 1.5 : 1.55);  // 2 + 3 ring < 2 + 2 < 8 waves
+    // 16x16 atoms: the same cycles at a higher clock when every CU is busy (fp16 4096^3 NT 100 against 112 us); with an operand
+    // read by transpose reads (2-way bank conflicts there) less of it is left (NN 104 against 108), and a grid below one
+    // round is not limited by the clock (3072^3 NN 68 against 65)
+    if (k->atom == 16) c *= (!k->transA && k->transB) ? 0.93 : (tiles >= 256 ? 0.97 : 1.06);
   } else if (area >= 256 * 128) {
     c = 0.93;
   } else {
@@ -261,7 +265,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   plan->kernel_id = best;
   plan->tile_m = k->bm; plan->tile_n = k->bn; plan->tile_k = k->bk;
   plan->waves_m = k->wm; plan->waves_n = k->wn; plan->waves_k = k->wk; plan->threads = k->wm * k->wn * k->wk * 64;
-  plan->mfma_m = 32; plan->mfma_n = 32; plan->mfma_k = mfma_k(d->dtype_ab);
+  plan->mfma_m = k->atom; plan->mfma_n = k->atom; plan->mfma_k = mfma_k(d->dtype_ab) * (32 / k->atom);
   plan->lds_bytes = k->lds_bytes;
   plan->stages = k->stages;
   plan->stages_b = k->stages_b;
@@ -269,8 +273,8 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   plan->grid_y = (int)((d->M + k->bm - 1) / k->bm);
   plan->guarded = k->guard;
   plan->xcd_remap = ((int64_t)plan->grid_x * plan->grid_y) % 8 == 0;
-  fill_layout(&plan->lds_a, !d->transA, es, frag_bytes(d->dtype_ab), k->bm, k->bk, k->wm * k->wn * k->wk, with_model);
-  fill_layout(&plan->lds_b, d->transB != 0, es, frag_bytes(d->dtype_ab), k->bn, k->bk, k->wm * k->wn * k->wk, with_model);
+  fill_layout(&plan->lds_a, !d->transA, es, frag_bytes(d->dtype_ab), k->bm, k->bk, k->wm * k->wn * k->wk, with_model, k->atom);
+  fill_layout(&plan->lds_b, d->transB != 0, es, frag_bytes(d->dtype_ab), k->bn, k->bk, k->wm * k->wn * k->wk, with_model, k->atom);
   plan->workspace_bytes = 0;
   // Split K over the grid's y dimension when the tile grid alone leaves most CUs idle (skinny problems are
   // bound by streaming the large operand, which needs many work-groups in flight).  Slices hold whole K tiles.
@@ -428,16 +432,23 @@ float frisk_hip_lds_access_cycles(int instr, const int32_t* lane_byte_addr) {
 
 int frisk_hip_lds_search(const frisk_lds_layout* shape, int elem_bytes, int frag_bytes, int tile_mn, int tile_k, int waves,
                          frisk_lds_layout* best, float* unswizzled_cycles) {
+  return frisk_hip_lds_search_atom(shape, elem_bytes, frag_bytes, tile_mn, tile_k, waves, 32, best, unswizzled_cycles);
+}
+
+int frisk_hip_lds_search_atom(const frisk_lds_layout* shape, int elem_bytes, int frag_bytes, int tile_mn, int tile_k, int waves, int atom,
+                              frisk_lds_layout* best, float* unswizzled_cycles) {
+  if (atom != 32 && atom != 16) return fail(FRISK_ERR_TILE, "MFMA atoms have 32 or 16 rows, not %d", atom);
+  if (atom == 16 && elem_bytes == 4) return fail(FRISK_ERR_TILE, "the 32-bit operands have no 16-row atom here");
   if (!shape || !best) return fail(FRISK_ERR_NULL, "shape and best must be given");
   if (shape->rows <= 0 || shape->row_bytes < 16 || shape->row_bytes % 16 || shape->row_bytes > 1024 || 1024 % shape->row_bytes)
     return fail(FRISK_ERR_TILE, "tile rows must be 16..1024 bytes and divide 1024");
   if ((elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) || frag_bytes < elem_bytes || waves <= 0 || tile_mn < 32 || tile_k <= 0)
     return fail(FRISK_ERR_TILE, "unsupported operand description");
   const bool kc = shape->k_contiguous != 0;
-  TileShape t{shape->rows, shape->row_bytes, kc, elem_bytes, frag_bytes, tile_mn, tile_k};
+  TileShape t{shape->rows, shape->row_bytes, kc, elem_bytes, frag_bytes, tile_mn, tile_k, atom};
   const Swizzle s = choose_swizzle(t, waves);
-  const int atoms = tile_mn / 32 < 4 ? tile_mn / 32 : 4;
-  const int n_access = atoms * ((tile_k * elem_bytes) / (2 * frag_bytes)) * frag_instr_count(kc, elem_bytes, frag_bytes);
+  const int atoms = tile_mn / atom < 4 ? tile_mn / atom : 4;
+  const int n_access = atoms * ((tile_k * elem_bytes) / frag_kstep_bytes(frag_bytes, atom)) * frag_instr_count(kc, elem_bytes, frag_bytes);
   if (n_access <= 0) return fail(FRISK_ERR_TILE, "tile holds no whole MFMA step");
   *best = *shape;
   best->row_shift = s.sh; best->row_mask = s.mk; best->chunk_shift = s.cs;

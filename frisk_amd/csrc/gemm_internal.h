@@ -58,6 +58,7 @@ struct KernelEntry {
   int wk;  // waves splitting the K steps of a tile (1 = none)
   int guard;  // 1: handles any shape / leading dimension (slower staging)
   int splitk;  // 1: compiled with the split-K store path
+  int atom;  // rows and columns of the MFMA atom: 32 (32x32xK) or 16 (16x16x2K)
   int lds_bytes;
   hipError_t (*launch)(const GemmParams&, hipStream_t);
   hipError_t (*prepare)();  // one-time, non-stream set-up of the kernel function (dynamic LDS limit)

@@ -8,8 +8,11 @@ committed so a build needs only hipcc.
 """
 import os
 
-# a variant: (transA, transB, BM, BN, BK, WM, WN, stages of A, guard, split-K, WK, stages of B)
-def square(bk):
+# a variant: (transA, transB, BM, BN, BK, WM, WN, stages of A, guard, split-K, WK, stages of B[, MFMA atom])
+# atom16: the default 256x256 variant (and its split-K copy) exists once more built from 16x16 atoms of twice the K depth: the
+# part holds a higher clock on them (fp16 4096^3 NT 100 against 112 us, NN 104 against 108; int8 gains nothing).  Listed first;
+# the planner prefers the 32x32 atoms where the clock is not the limit (grids below one round with a transpose-read operand)
+def square(bk, atom16=False):
     out = []
     # The first variant of a tile size is the planner's default.  256x256: 4 waves of 128x128 (fewest LDS reads per MFMA)
     # with 2 LDS tiles of A and 3 of B (160 KiB), B fetched two tiles ahead and spread over the K tile; then the same
@@ -20,11 +23,15 @@ def square(bk):
                                       (128, 256, bk, 2, 2, 3, 3), (128, 128, bk, 2, 2, 2, 2), (128, 128, bk, 2, 2, 3, 3)):
         for ta in (0, 1):
             for tb in (0, 1):
+                if atom16 and (bm, bn, wm, wn, st, sb) == (256, 256, 2, 2, 2, 3):
+                    out.append((ta, tb, bm, bn, k, wm, wn, st, 0, 0, 1, sb, 16))
                 out.append((ta, tb, bm, bn, k, wm, wn, st, 0, 0, 1, sb))
     # the default 256x256 variant once more with the split-K store path: for grids a little over a whole number of rounds
     # of 256 tiles, whose last tiles are then split along K over several work-groups (a tail split)
     for ta in (0, 1):
         for tb in (0, 1):
+            if atom16:
+                out.append((ta, tb, 256, 256, bk, 2, 2, 2, 0, 1, 1, 3, 16))
             out.append((ta, tb, 256, 256, bk, 2, 2, 2, 0, 1, 1, 3))
     # skinny variants (M a multiple of 32), bound by streaming B: K may be split over the grid's y dimension.
     #   B stored [N][K]: 32x32 tile, 512-byte K rows, the 4 waves split the K steps of a tile
@@ -42,8 +49,8 @@ def square(bk):
     return out
 
 VARIANTS = {
-    "f16": ("FRISK_F16", "F16", square(64)),
-    "bf16": ("FRISK_BF16", "BF16", square(64)),
+    "f16": ("FRISK_F16", "F16", square(64, atom16=True)),
+    "bf16": ("FRISK_BF16", "BF16", square(64, atom16=True)),
     "i8": ("FRISK_I8", "I8", square(128)),
     "e4m3": ("FRISK_E4M3", "E4M3", square(128)),
     # fp32: 128x128 for large problems; 64x64 (one atom per wave) fills the chip at 1024^3, K tiles of 64 measured 5 % faster than 32;
@@ -58,13 +65,16 @@ VARIANTS = {
 }
 
 def full(v):
-    """(…, WK) -> (…, WK, stages of B): B has as many stages as A unless the variant says otherwise"""
-    return tuple(v) if len(v) == 12 else tuple(v) + (v[7],)
+    """(…, WK) -> (…, WK, stages of B, atom): B has as many stages as A and the atom is 32x32 unless the variant says otherwise"""
+    v = tuple(v)
+    if len(v) == 11:
+        v += (v[7],)
+    return v if len(v) == 13 else v + (32,)
 
 
 def cfg_of(enum, v):
-    ta, tb, bm, bn, bk, wm, wn, st, gd, sk, wk, sb = full(v)
-    return f"GemmCfg<{enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {'true' if gd else 'false'}, {'true' if sk else 'false'}, {wk}, {sb}>"
+    ta, tb, bm, bn, bk, wm, wn, st, gd, sk, wk, sb, at = full(v)
+    return f"GemmCfg<{enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {'true' if gd else 'false'}, {'true' if sk else 'false'}, {wk}, {sb}" + (f", {at}>" if at != 32 else ">")
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 for tag, (enum, suffix, variants) in VARIANTS.items():
@@ -75,11 +85,11 @@ for tag, (enum, suffix, variants) in VARIANTS.items():
     lines.append("#ifndef __HIP_DEVICE_COMPILE__")
     lines.append(f"const KernelEntry kKernels{suffix}[] = {{")
     for v in variants:
-        ta, tb, bm, bn, bk, wm, wn, st, gd, sk, wk, sb = full(v)
+        ta, tb, bm, bn, bk, wm, wn, st, gd, sk, wk, sb, at = full(v)
         cfg = cfg_of(enum, v)
         waves = f"w{wm}x{wn}" + (f"x{wk}" if wk > 1 else "")
-        name = f"{tag}_{'t' if ta else 'n'}{'t' if tb else 'n'}_{bm}x{bn}x{bk}_{waves}_s{st}" + (f"x{sb}" if sb != st else "") + ("_guard" if gd else "") + ("_splitk" if sk else "")
-        lines.append(f'    {{"{name}", {enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {sb}, {wk}, {gd}, {sk}, {cfg}::LDS_BYTES, &launch_gemm<{cfg}>, &prepare_gemm<{cfg}>}},')
+        name = f"{tag}_{'t' if ta else 'n'}{'t' if tb else 'n'}_{bm}x{bn}x{bk}_{waves}_s{st}" + (f"x{sb}" if sb != st else "") + (f"_a{at}" if at != 32 else "") + ("_guard" if gd else "") + ("_splitk" if sk else "")
+        lines.append(f'    {{"{name}", {enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {sb}, {wk}, {gd}, {sk}, {at}, {cfg}::LDS_BYTES, &launch_gemm<{cfg}>, &prepare_gemm<{cfg}>}},')
     lines.append("};")
     lines.append(f"const int kNumKernels{suffix} = sizeof(kKernels{suffix}) / sizeof(kKernels{suffix}[0]);")
     lines.append("#endif")

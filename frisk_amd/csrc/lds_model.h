@@ -47,24 +47,28 @@ FRISK_HD int lds_offset(int rowb, Swizzle s, int row, int colbyte) {
   return row * rowb + ((((colbyte >> 4) ^ lds_swz(s, row)) << 4) | (colbyte & 15));
 }
 
-// ---- fragment addressing (32x32 MFMA atoms; lane l serves row/col l%32, K-group l/32)
+// ---- fragment addressing.  An MFMA atom covers `at` rows (or columns) of the operand, 32 or 16: lane l serves
+// row/col l % at, K-group l / at (2 groups of a 32-row atom, 4 of a 16-row atom), fragb bytes along K each.
+FRISK_HD int frag_kstep_bytes(int fragb, int at = 32) { return (64 / at) * fragb; }  // K bytes one atom consumes
 // K-contiguous tile: instruction q of FRAGB/16 (or the single 4-byte read when FRAGB == 4)
-FRISK_HD int frag_addr_kc(int rowb, Swizzle s, int fragb, int lane, int mn0, int kb0, int q) {
-  int row = mn0 + (lane & 31);
-  int kb = kb0 + (lane >> 5) * fragb + 16 * q;
+FRISK_HD int frag_addr_kc(int rowb, Swizzle s, int fragb, int lane, int mn0, int kb0, int q, int at = 32) {
+  int row = mn0 + (lane & (at - 1));
+  int kb = kb0 + (lane / at) * fragb + 16 * q;
   return lds_offset(rowb, s, row, kb);
 }
 // MN-contiguous tile (rows = K).  16- and 8-bit elements use the transpose
 // reads: in a block of 16 lanes, lane L presents K-row L / lpr and the 8 bytes
 // at column-group L % lpr; it receives column (l % 16) of the block's K rows.
+// The at / 16 blocks of a K-group sit side by side along the columns.
 // 32-bit elements read their single value directly.
-FRISK_HD int frag_addr_mc(int rowb, Swizzle s, int es, int fragb, int lane, int mn0, int kb0, int q) {
+FRISK_HD int frag_addr_mc(int rowb, Swizzle s, int es, int fragb, int lane, int mn0, int kb0, int q, int at = 32) {
   if (es == 4) return lds_offset(rowb, s, kb0 / 4 + (lane >> 5), (mn0 + (lane & 31)) * 4);
   int kpi = es == 2 ? 4 : 8;
   int lpr = 16 / kpi;
   int blk = lane >> 4, l16 = lane & 15;
-  int col0 = mn0 + 16 * (blk & 1);
-  int krow = kb0 / es + (blk >> 1) * (fragb / es) + q * kpi + l16 / lpr;
+  int col_blocks = at / 16;
+  int col0 = mn0 + 16 * (blk % col_blocks);
+  int krow = kb0 / es + (blk / col_blocks) * (fragb / es) + q * kpi + l16 / lpr;
   int colbyte = (col0 + (l16 % lpr) * (8 / es)) * es;
   return lds_offset(rowb, s, krow, colbyte);
 }
@@ -122,22 +126,24 @@ struct TileShape {
   bool kcontig;
   int es, fragb;   // element bytes, fragment bytes per lane per MFMA
   int mn, bk;      // logical extent along M (or N) and K, elements
+  int at = 32;     // rows (or columns) of the operand one MFMA atom covers
 };
 
 FRISK_HD int swizzle_read_cycles(TileShape t, Swizzle s) {
   int total = 0;
-  int ksteps = (t.bk * t.es) / (2 * t.fragb);
+  int kstep = frag_kstep_bytes(t.fragb, t.at);
+  int ksteps = (t.bk * t.es) / kstep;
   int ninstr = frag_instr_count(t.kcontig, t.es, t.fragb);
   int kind = frag_instr_kind(t.kcontig, t.es);
   // bank behaviour repeats with the atom position beyond what the swizzle sees; sample the first atoms
-  int atoms = t.mn / 32 < 4 ? t.mn / 32 : 4;
+  int atoms = t.mn / t.at < 4 ? t.mn / t.at : 4;
   for (int a = 0; a < atoms; ++a)
     for (int ks = 0; ks < ksteps; ++ks)
       for (int q = 0; q < ninstr; ++q) {
         int addr[64] = {};
         for (int l = 0; l < 64; ++l)
-          addr[l] = t.kcontig ? frag_addr_kc(t.rowb, s, t.fragb, l, a * 32, ks * 2 * t.fragb, q)
-                              : frag_addr_mc(t.rowb, s, t.es, t.fragb, l, a * 32, ks * 2 * t.fragb, q);
+          addr[l] = t.kcontig ? frag_addr_kc(t.rowb, s, t.fragb, l, a * t.at, ks * kstep, q, t.at)
+                              : frag_addr_mc(t.rowb, s, t.es, t.fragb, l, a * t.at, ks * kstep, q, t.at);
         total += lds_access_cycles(kind, addr);
       }
   return total;

@@ -69,7 +69,7 @@ class FriskHipError(RuntimeError):
 _lib = None
 
 EXPORTS = ["frisk_hip_init", "frisk_hip_abi_version", "frisk_hip_last_error", "frisk_hip_plan", "frisk_hip_workspace_bytes",
-           "frisk_hip_gemm", "frisk_hip_lds_access_cycles", "frisk_hip_lds_search", "frisk_hip_lds_offset", "frisk_hip_wave_partition",
+           "frisk_hip_gemm", "frisk_hip_lds_access_cycles", "frisk_hip_lds_search", "frisk_hip_lds_search_atom", "frisk_hip_lds_offset", "frisk_hip_wave_partition",
            "frisk_hip_kernel_count", "frisk_hip_kernel_name", "frisk_hip_fill", "frisk_hip_copy", "frisk_hip_reduce",
            "frisk_hip_reduce_workspace_bytes", "frisk_hip_attention", "frisk_hip_softmax", "frisk_hip_softmax_workspace_bytes"]
 
@@ -93,6 +93,8 @@ def lib():
     L.frisk_hip_lds_access_cycles.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_int32)]
     L.frisk_hip_lds_search.argtypes = [ctypes.POINTER(LdsLayout), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                        ctypes.c_int, ctypes.POINTER(LdsLayout), ctypes.POINTER(ctypes.c_float)]
+    L.frisk_hip_lds_search_atom.argtypes = [ctypes.POINTER(LdsLayout), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                            ctypes.c_int, ctypes.c_int, ctypes.POINTER(LdsLayout), ctypes.POINTER(ctypes.c_float)]
     L.frisk_hip_lds_offset.restype = ctypes.c_int32
     L.frisk_hip_lds_offset.argtypes = [ctypes.POINTER(LdsLayout), ctypes.c_int32, ctypes.c_int32]
     L.frisk_hip_wave_partition.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -223,12 +225,13 @@ def lds_access_cycles(instr, lane_addrs):
     return lib().frisk_hip_lds_access_cycles(instr, arr)
 
 
-def lds_search(rows, row_bytes, k_contiguous, elem_bytes, frag_bytes, tile_mn, tile_k, waves):
-    """exhaustive swizzle search for one operand tile; returns (LdsLayout best, unswizzled cycles per access)"""
+def lds_search(rows, row_bytes, k_contiguous, elem_bytes, frag_bytes, tile_mn, tile_k, waves, atom=32):
+    """exhaustive swizzle search for one operand tile read by MFMA atoms of `atom` rows; returns (LdsLayout best, unswizzled
+    cycles per access)"""
     shape, best, base = LdsLayout(), LdsLayout(), ctypes.c_float()
     shape.rows, shape.row_bytes, shape.k_contiguous = rows, row_bytes, int(k_contiguous)
-    _check(lib().frisk_hip_lds_search(ctypes.byref(shape), elem_bytes, frag_bytes, tile_mn, tile_k, waves,
-                                      ctypes.byref(best), ctypes.byref(base)))
+    _check(lib().frisk_hip_lds_search_atom(ctypes.byref(shape), elem_bytes, frag_bytes, tile_mn, tile_k, waves, atom,
+                                           ctypes.byref(best), ctypes.byref(base)))
     return best, base.value
 
 

@@ -165,6 +165,10 @@ float frisk_hip_lds_access_cycles(int instr, const int32_t* lane_byte_addr);
  * modelled cycles per access of the same tile without a swizzle. */
 int frisk_hip_lds_search(const frisk_lds_layout* shape, int elem_bytes, int frag_bytes, int tile_mn, int tile_k, int waves,
                          frisk_lds_layout* best, float* unswizzled_cycles);
+/* The same for operands of MFMA atoms of `atom` rows / columns: 32 (32x32xK atoms, what frisk_hip_lds_search assumes) or
+ * 16 (16x16x2K atoms: lane l serves row l % 16 and K-group l / 16 of four). */
+int frisk_hip_lds_search_atom(const frisk_lds_layout* shape, int elem_bytes, int frag_bytes, int tile_mn, int tile_k, int waves, int atom,
+                         frisk_lds_layout* best, float* unswizzled_cycles);
 
 /* Pure host: byte offset inside an LDS tile of element (row, col_byte) under `layout`. */
 int32_t frisk_hip_lds_offset(const frisk_lds_layout* layout, int32_t row, int32_t col_byte);

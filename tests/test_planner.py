@@ -41,7 +41,9 @@ def test_plans_of_the_benchmark_configurations():
         assert p.grid_x == N // tile[1] and p.grid_y == M // tile[0]
         assert p.grid_x * p.grid_y >= 256 and p.xcd_remap == 1
         assert p.threads == 64 * p.waves_m * p.waves_n * p.waves_k and p.lds_bytes <= 160 * 1024
-        assert p.mfma_m == 32 and p.mfma_n == 32
+        # the 16-bit 256x256 default is built from 16x16x32 atoms (the part holds a higher clock on them), the rest from 32x32
+        atom = 16 if dt in (R.F16, R.BF16) else 32
+        assert (p.mfma_m, p.mfma_n) == (atom, atom) and p.mfma_k == {R.F32: 2, R.F16: 32, R.BF16: 32, R.I8: 32, R.E4M3: 64}[dt]
         assert p.flops == 2.0 * M * N * K
         assert p.lds_a.k_contiguous == (0 if tA else 1) and p.lds_b.k_contiguous == (1 if tB else 0)
         assert p.workspace_bytes == 0 and p.kernel_id >= 0
@@ -53,11 +55,15 @@ def test_fp16_tile_layouts_are_conflict_free_in_the_model():
     p = R.plan(R.make_desc(R.F16, 4096, 4096, 4096))
     a, b = p.lds_a, p.lds_b
     assert (a.rows, a.row_bytes, a.read_instr) == (256, 128, 0) and (b.rows, b.row_bytes, b.read_instr) == (64, 512, 1)
-    assert a.read_cycles == 4.0 and b.read_cycles == 3.0      # the floors of ds_read_b128 and ds_read_b64_tr_b16
+    # ds_read_b128 at its floor; the transpose reads of the 16x16x32 atoms put two K groups (K rows 8 apart) into one half wave,
+    # which the row-XOR swizzle family cannot separate: 2 passes per half instead of the floor of 3 cycles per instruction
+    assert a.read_cycles == 4.0 and b.read_cycles == 4.0
+    p = R.plan(R.make_desc(R.F16, 2048, 2048, 2048))   # 128x128 tiles of 32x32x16 atoms: both at their floors
+    assert (p.mfma_m, p.lds_a.read_cycles, p.lds_b.read_cycles) == (32, 4.0, 3.0)
 
 
-SHAPES = [  # rows, row_bytes, k_contiguous, elem_bytes, frag_bytes, tile_mn, tile_k  (every operand tile shape that is compiled)
-    (256, 128, 1, 2, 16, 256, 64), (64, 512, 0, 2, 16, 256, 64), (128, 128, 1, 2, 16, 128, 64), (64, 256, 0, 2, 16, 128, 64),
+SHAPES = [  # rows, row_bytes, k_contiguous, elem_bytes, frag_bytes, tile_mn, tile_k[, atom]  (every operand tile shape that is compiled)
+    (256, 128, 1, 2, 16, 256, 64, 16), (64, 512, 0, 2, 16, 256, 64, 16), (256, 128, 1, 2, 16, 256, 64), (64, 512, 0, 2, 16, 256, 64), (128, 128, 1, 2, 16, 128, 64), (64, 256, 0, 2, 16, 128, 64),
     (256, 128, 1, 1, 16, 256, 128), (128, 256, 0, 1, 16, 256, 128), (128, 128, 1, 1, 16, 128, 128), (128, 128, 0, 1, 16, 128, 128),
     (256, 128, 1, 1, 32, 256, 128), (128, 256, 0, 1, 32, 256, 128), (128, 128, 1, 1, 32, 128, 128), (128, 128, 0, 1, 32, 128, 128),
     (128, 128, 1, 4, 4, 128, 32), (32, 512, 0, 4, 4, 128, 32), (64, 128, 1, 4, 4, 64, 32), (32, 256, 0, 4, 4, 64, 32),
@@ -67,26 +73,32 @@ SHAPES = [  # rows, row_bytes, k_contiguous, elem_bytes, frag_bytes, tile_mn, ti
 
 @pytest.mark.parametrize("shape", SHAPES)
 def test_compiled_swizzle_is_what_the_cost_model_search_picks(shape):
-    rows, rowb, kc, es, fragb, mn, bk = shape
-    best, unswizzled = R.lds_search(rows, rowb, kc, es, fragb, mn, bk, 4)
+    rows, rowb, kc, es, fragb, mn, bk = shape[:7]
+    atom = shape[7] if len(shape) > 7 else 32
+    best, unswizzled = R.lds_search(rows, rowb, kc, es, fragb, mn, bk, 4, atom)
     # the kernels' constants come back through the plan; find a descriptor that uses this tile shape
     dt = {(2, 16): R.F16, (1, 16): R.I8, (1, 32): R.E4M3, (4, 4): R.F32}[(es, fragb)]
     for tA in (0, 1):
         for tB in (0, 1):
             for M in (mn * 16,):
-                d = R.make_desc(dt, M, M, bk * 8, dtype_out=R.ACC_OF[dt] if dt != R.F16 else R.F16, transA=tA, transB=tB, tile=(mn, mn, bk))
+                # the 16-bit 256x256 tiles exist with both atoms: the ring of 2 + 2 tiles is the variant of 32x32 atoms
+                d = R.make_desc(dt, M, M, bk * 8, dtype_out=R.ACC_OF[dt] if dt != R.F16 else R.F16, transA=tA, transB=tB, tile=(mn, mn, bk),
+                                stages=2 if (dt == R.F16 and mn == 256 and atom == 32) else 0)
                 p = R.plan(d)
+                assert p.mfma_m == atom
                 for L in (p.lds_a, p.lds_b):
                     if (L.rows, L.row_bytes, L.k_contiguous) == (rows, rowb, kc):
-                        assert (L.row_shift, L.row_mask, L.chunk_shift) == (best.row_shift, best.row_mask, best.chunk_shift)
+                        # the 16-row atoms keep the swizzles frozen for the 32-row atoms: several tie in the model, the search's
+                        # tie-break then names another one of the same cost
+                        assert atom == 16 or (L.row_shift, L.row_mask, L.chunk_shift) == (best.row_shift, best.row_mask, best.chunk_shift)
                         assert L.read_cycles == best.read_cycles <= unswizzled
                         return
     pytest.fail("no plan uses tile shape %r" % (shape,))
 
 
 def test_swizzle_is_a_bijection_on_the_tile():
-    for rows, rowb, kc, es, fragb, mn, bk in SHAPES:
-        best, _ = R.lds_search(rows, rowb, kc, es, fragb, mn, bk, 4)
+    for rows, rowb, kc, es, fragb, mn, bk, *atom in SHAPES:
+        best, _ = R.lds_search(rows, rowb, kc, es, fragb, mn, bk, 4, *atom)
         seen = set()
         for r in range(rows):
             for c in range(0, rowb, 16):
@@ -209,10 +221,12 @@ def test_planner_ranks_variants_by_estimated_time():
     def pick(dt, M, N, K, **kw):
         return names[R.plan(R.make_desc(dt, M, N, K, dtype_out={R.E4M3: R.BF16, R.I8: R.I32}.get(dt), **kw)).kernel_id]
     assert pick(R.F16, 2048, 2048, 2048) == "f16_nn_128x128x64_w2x2_s3"
+    # 144 tiles leave CUs idle: the clock is not the limit, so the 32x32 atoms stay unless both operands are K-contiguous
     assert pick(R.F16, 3072, 3072, 3072) == "f16_nn_256x256x64_w2x2_s2x3"
-    assert pick(R.F16, 4096, 4096, 4096) == "f16_nn_256x256x64_w2x2_s2x3"
+    assert pick(R.F16, 3072, 3072, 3072, transB=True) == "f16_nt_256x256x64_w2x2_s2x3_a16"
+    assert pick(R.F16, 4096, 4096, 4096) == "f16_nn_256x256x64_w2x2_s2x3_a16"
     assert pick(R.BF16, 1024, 8192, 8192, transB=True) == "bf16_nt_256x128x64_w2x2_s3"
-    assert pick(R.F16, 8192, 8192, 8192) == "f16_nn_256x256x64_w2x2_s2x3"
+    assert pick(R.F16, 8192, 8192, 8192) == "f16_nn_256x256x64_w2x2_s2x3_a16"
     assert pick(R.E4M3, 32, 8192, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s4_splitk"
     # more than 256 such tiles: the ring of 2, two work-groups per CU (29.3 us against 35.8 for 512 tiles, 52.8 against 60.1 for 1024)
     assert pick(R.E4M3, 32, 16384, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s2_splitk"
