@@ -122,13 +122,16 @@ static int validate(const frisk_gemm_desc* d) {
 
 static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, int mn, int bk, int nw, bool with_model, int atom) {
   TileShape t{kcontig ? mn : bk, (kcontig ? bk : mn) * es, kcontig, es, fragb, mn, bk, atom};
-  Swizzle s = default_swizzle(kcontig, es, t.rowb);
+  Swizzle s = default_swizzle(kcontig, es, t.rowb, atom);
   L->rows = t.rows;
   L->row_bytes = t.rowb;
   L->k_contiguous = kcontig;
   L->row_shift = s.sh;
   L->row_mask = s.mk;
   L->chunk_shift = s.cs;
+  L->row_shift2 = s.sh2;
+  L->row_mask2 = s.mk2;
+  L->chunk_shift2 = s.cs2;
   L->read_instr = es == 4 ? 3 : (kcontig ? 0 : (es == 2 ? 1 : 2));
   int atoms = mn / atom < 4 ? mn / atom : 4;
   int n_access = atoms * ((bk * es) / frag_kstep_bytes(fragb, atom)) * frag_instr_count(kcontig, es, fragb);
@@ -452,6 +455,7 @@ int frisk_hip_lds_search_atom(const frisk_lds_layout* shape, int elem_bytes, int
   if (n_access <= 0) return fail(FRISK_ERR_TILE, "tile holds no whole MFMA step");
   *best = *shape;
   best->row_shift = s.sh; best->row_mask = s.mk; best->chunk_shift = s.cs;
+  best->row_shift2 = s.sh2; best->row_mask2 = s.mk2; best->chunk_shift2 = s.cs2;
   best->read_instr = elem_bytes == 4 ? 3 : (kc ? 0 : (elem_bytes == 2 ? 1 : 2));
   best->read_cycles = (float)swizzle_read_cycles(t, s) / (float)n_access;
   best->write_cycles = 16.f;
@@ -461,7 +465,7 @@ int frisk_hip_lds_search_atom(const frisk_lds_layout* shape, int elem_bytes, int
 
 int32_t frisk_hip_lds_offset(const frisk_lds_layout* L, int32_t row, int32_t col_byte) {
   if (!L) return -1;
-  return lds_offset(L->row_bytes, Swizzle{L->row_shift, L->row_mask, L->chunk_shift}, row, col_byte);
+  return lds_offset(L->row_bytes, Swizzle{L->row_shift, L->row_mask, L->chunk_shift, L->row_shift2, L->row_mask2, L->chunk_shift2}, row, col_byte);
 }
 
 int frisk_hip_wave_partition(int policy, int tile_m, int tile_n, int num_waves, int* waves_m, int* waves_n) {

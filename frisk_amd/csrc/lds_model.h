@@ -37,12 +37,22 @@ namespace frisk {
 
 enum LdsInstr { LDS_READ_B128 = 0, LDS_READ_B64 = 1, LDS_READ_B64_TR16 = 1, LDS_READ_B64_TR8 = 1, LDS_READ_B32 = 3 };
 
-// XOR swizzle: 16-byte chunk c of row r is stored at chunk c ^ (((r >> sh) & mk) << cs)
+// XOR swizzle: 16-byte chunk c of row r is stored at chunk
+//   c ^ (((r >> sh) & mk) << cs) ^ (((r >> sh2) & mk2) << cs2)
+// The second term (absent when mk2 == 0) lets row bits that are not adjacent to
+// those of the first term take part: the transpose reads of a 16-row MFMA atom
+// put K rows r .. r+3 and r+8 .. r+11 into one half wave.
 struct Swizzle {
   int sh, mk, cs;
+  int sh2 = 0, mk2 = 0, cs2 = 0;
 };
 
-FRISK_HD int lds_swz(Swizzle s, int row) { return ((row >> s.sh) & s.mk) << s.cs; }
+FRISK_HD int lds_swz(Swizzle s, int row) { return (((row >> s.sh) & s.mk) << s.cs) ^ (((row >> s.sh2) & s.mk2) << s.cs2); }
+// rows after which the swizzle repeats
+FRISK_HD int lds_swz_period(Swizzle s) {
+  int p1 = s.mk == 0 ? 1 : ((s.mk + 1) << s.sh), p2 = s.mk2 == 0 ? 1 : ((s.mk2 + 1) << s.sh2);
+  return p1 > p2 ? p1 : p2;
+}
 FRISK_HD int lds_offset(int rowb, Swizzle s, int row, int colbyte) {
   return row * rowb + ((((colbyte >> 4) ^ lds_swz(s, row)) << 4) | (colbyte & 15));
 }
@@ -155,25 +165,41 @@ FRISK_HD int swizzle_read_cycles(TileShape t, Swizzle s) {
 FRISK_HD bool swizzle_usable(TileShape t, Swizzle s, int nw) {
   int chunks = t.rowb / 16;
   if ((s.mk << s.cs) >= chunks && s.mk != 0) return false;
+  if ((s.mk2 << s.cs2) >= chunks && s.mk2 != 0) return false;
   int rpc = 1024 / t.rowb;
-  int period = (s.mk + 1) << s.sh;
-  return s.mk == 0 || ((nw * rpc) % period) == 0;
+  int period = lds_swz_period(s);
+  return period == 1 || ((nw * rpc) % period) == 0 || (period % (nw * rpc)) == 0;
 }
 
 // Exhaustive search over (sh, mk, cs); ties go to the smaller mask, then the
 // smaller chunk shift, then the smaller row shift (the least surprising layout).
+// A second, one-bit term (sh2, 1, cs2) on a row bit the first term does not use
+// is tried on top of every first term and taken only when it is strictly cheaper.
 FRISK_HD Swizzle choose_swizzle(TileShape t, int nw) {
   Swizzle best = {0, 0, 0};
   int best_cost = swizzle_read_cycles(t, best);
-  const int masks[4] = {1, 3, 7, 15};
-  for (int mi = 0; mi < 4; ++mi)
-    for (int cs = 0; cs < 4; ++cs)
-      for (int sh = 0; sh < 4; ++sh) {
-        Swizzle s = {sh, masks[mi], cs};
-        if (!swizzle_usable(t, s, nw)) continue;
-        int c = swizzle_read_cycles(t, s);
-        if (c < best_cost) { best_cost = c; best = s; }
-      }
+  const int masks[5] = {0, 1, 3, 7, 15};
+  for (int second = 0; second < 2; ++second)
+    for (int mi = 0; mi < 5; ++mi)
+      for (int cs = 0; cs < 4; ++cs)
+        for (int sh = 0; sh < 4; ++sh) {
+          if (masks[mi] == 0 && (cs || sh)) continue;
+          if (!second) {
+            Swizzle s = {sh, masks[mi], cs};
+            if (masks[mi] == 0 || !swizzle_usable(t, s, nw)) continue;
+            int c = swizzle_read_cycles(t, s);
+            if (c < best_cost) { best_cost = c; best = s; }
+            continue;
+          }
+          for (int sh2 = 0; sh2 < 6; ++sh2)
+            for (int cs2 = 0; cs2 < 4; ++cs2) {
+              if ((((masks[mi] << sh) >> sh2) & 1) != 0) continue;
+              Swizzle s = {sh, masks[mi], cs, sh2, 1, cs2};
+              if (!swizzle_usable(t, s, nw)) continue;
+              int c = swizzle_read_cycles(t, s);
+              if (c < best_cost) { best_cost = c; best = s; }
+            }
+        }
   return best;
 }
 
@@ -184,7 +210,7 @@ FRISK_HD Swizzle choose_swizzle(TileShape t, int nw) {
 // (row >> 1).  Tiles whose rows run along M or N are read by transpose reads
 // that touch 4 (16-bit) or 8 (8-bit) consecutive K rows per half wave, 64 or
 // 32 bytes wide: XOR with the K row in units of that width.
-FRISK_HD Swizzle default_swizzle(bool kcontig, int es, int rowb) {
+FRISK_HD Swizzle default_swizzle(bool kcontig, int es, int rowb, int at = 32) {
   int chunks = rowb / 16;
   if (kcontig) {
     // 16 consecutive rows must cover the 16 bank groups of 16 bytes: rows of 128 B
@@ -198,6 +224,8 @@ FRISK_HD Swizzle default_swizzle(bool kcontig, int es, int rowb) {
   if (es == 4) return Swizzle{0, 0, 0};
   if (es == 2) {
     int units = chunks >> 2;  // 64-byte units
+    // 16-row atoms: a half wave holds two K groups (K rows 8 apart), 32 bytes wide each; K-row bit 3 picks the 32-byte half
+    if (at == 16 && units >= 4) return Swizzle{0, 3, 2, 3, 1, 1};
     return Swizzle{0, units >= 4 ? 3 : (units >= 2 ? 1 : 0), 2};
   }
   if (rowb >= 256) return Swizzle{0, 7, 1};

@@ -115,18 +115,22 @@ std::string lds_layout_debug(const frisk_lds_layout& L, int elem_bytes) {
   AffineExpr i = AffineExpr::dim(0), j = AffineExpr::dim(1);
   AffineExpr chunk = j.floor_div(AffineExpr::constant(vec));
   AffineExpr stored = chunk;
-  if (L.row_mask) {
-    const int64_t lo = (int64_t)1 << L.chunk_shift, span = (int64_t)L.row_mask + 1;
-    AffineExpr field = chunk.floor_div(AffineExpr::constant(lo)).mod(AffineExpr::constant(span));  // the chunk bits the swizzle touches
-    AffineExpr key = i.floor_div(AffineExpr::constant((int64_t)1 << L.row_shift)).mod(AffineExpr::constant(span));
+  // one XOR term applied to the chunk index as stored so far
+  auto apply = [&](int row_shift, int row_mask, int chunk_shift) {
+    if (!row_mask) return;
+    const int64_t lo = (int64_t)1 << chunk_shift, span = (int64_t)row_mask + 1;
+    AffineExpr field = stored.floor_div(AffineExpr::constant(lo)).mod(AffineExpr::constant(span));  // the chunk bits the swizzle touches
+    AffineExpr key = i.floor_div(AffineExpr::constant((int64_t)1 << row_shift)).mod(AffineExpr::constant(span));
     AffineExpr x = AffineExpr::constant(0);
     for (int64_t b = 1; b < span; b *= 2) {
       AffineExpr fb = field.floor_div(AffineExpr::constant(b)).mod(AffineExpr::constant(2));
       AffineExpr kb = key.floor_div(AffineExpr::constant(b)).mod(AffineExpr::constant(2));
       x = x + (fb + kb).mod(AffineExpr::constant(2)) * b;
     }
-    stored = chunk + (x - field) * lo;
-  }
+    stored = stored + (x - field) * lo;
+  };
+  apply(L.row_shift, L.row_mask, L.chunk_shift);
+  apply(L.row_shift2, L.row_mask2, L.chunk_shift2);
   AffineExpr index = i * cols + stored * vec + j.mod(AffineExpr::constant(vec));
   AffineMap map(2, 0, {index});
   return "Layout(shape=[" + std::to_string(L.rows) + ", " + std::to_string(cols) + "], index=affine_map<" + map.str() + ">)";
@@ -223,18 +227,23 @@ void init_ffi_runtime(py::module_&& m) {
     out["lds_b"] = lds_layout_debug(p.lds_b, es);
     out["lds_swizzle"] = py::make_tuple(py::make_tuple(p.lds_a.row_shift, p.lds_a.row_mask, p.lds_a.chunk_shift),
                                         py::make_tuple(p.lds_b.row_shift, p.lds_b.row_mask, p.lds_b.chunk_shift));
+    out["lds_swizzle2"] = py::make_tuple(py::make_tuple(p.lds_a.row_shift2, p.lds_a.row_mask2, p.lds_a.chunk_shift2),
+                                         py::make_tuple(p.lds_b.row_shift2, p.lds_b.row_mask2, p.lds_b.chunk_shift2));
     out["flops"] = p.flops;
     out["bytes"] = p.bytes;
     return out;
   }, py::arg("kernel"), py::arg("module") = py::none(), py::arg("epilogue") = "none");
 
-  m.def("lds_layout_string", [](int rows, int row_bytes, int elem_bytes, int row_shift, int row_mask, int chunk_shift) {
+  m.def("lds_layout_string", [](int rows, int row_bytes, int elem_bytes, int row_shift, int row_mask, int chunk_shift,
+                                int row_shift2, int row_mask2, int chunk_shift2) {
     frisk_lds_layout L{};
     L.rows = rows; L.row_bytes = row_bytes; L.row_shift = row_shift; L.row_mask = row_mask; L.chunk_shift = chunk_shift;
+    L.row_shift2 = row_shift2; L.row_mask2 = row_mask2; L.chunk_shift2 = chunk_shift2;
     if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) throw std::invalid_argument("element size must be 1, 2 or 4 bytes");
     return lds_layout_debug(L, elem_bytes);
   }, py::arg("rows"), py::arg("row_bytes"), py::arg("elem_bytes"), py::arg("row_shift"), py::arg("row_mask"), py::arg("chunk_shift"),
-     "Layout(shape=[...], index=affine_map<...>) of an LDS tile with the XOR swizzle (row_shift, row_mask, chunk_shift); pure host");
+     py::arg("row_shift2") = 0, py::arg("row_mask2") = 0, py::arg("chunk_shift2") = 0,
+     "Layout(shape=[...], index=affine_map<...>) of an LDS tile with the XOR swizzle (row_shift, row_mask, chunk_shift) and the optional second term; pure host");
   m.def("accumulator_layout_string", &accumulator_layout_debug, py::arg("tile_m"), py::arg("tile_n"), py::arg("waves_m"), py::arg("waves_n"),
         "Fragment(shape, index, thread, replicate) of the MFMA accumulators of a work-group tile; pure host");
 

@@ -27,9 +27,11 @@ def operand_entry(R, ffi_runtime, label, rows, cols, k_contiguous, es, frag, til
         degree = max(1.0, cycles / ideal)
         return {"avg_max_conflict": round(degree, 3), "max_conflict": int(math.ceil(degree - 1e-9)), "samples": 64,
                 "cycles_per_access": round(cycles, 3), "read_instruction": name}
-    text = ffi_runtime.lds_layout_string(rows, cols * es, es, best.row_shift, best.row_mask, best.chunk_shift)
+    text = ffi_runtime.lds_layout_string(rows, cols * es, es, best.row_shift, best.row_mask, best.chunk_shift,
+                                         best.row_shift2, best.row_mask2, best.chunk_shift2)
     return {"operand": label, "shape": [rows, cols], "element_bits": es * 8, "memory_space": "Shared",
-            "forward_index": text[text.index("index=") + 6:-1], "swizzle": {"row_shift": best.row_shift, "row_mask": best.row_mask, "chunk_shift": best.chunk_shift},
+            "forward_index": text[text.index("index=") + 6:-1], "swizzle": {"row_shift": best.row_shift, "row_mask": best.row_mask, "chunk_shift": best.chunk_shift,
+                        "row_shift2": best.row_shift2, "row_mask2": best.row_mask2, "chunk_shift2": best.chunk_shift2},
             "bank_stats": stats(best.read_cycles), "baseline_row_major": stats(unswizzled)}
 
 

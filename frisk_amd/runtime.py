@@ -37,7 +37,8 @@ class GemmDesc(ctypes.Structure):
 class LdsLayout(ctypes.Structure):
     _fields_ = [("rows", ctypes.c_int32), ("row_bytes", ctypes.c_int32), ("k_contiguous", ctypes.c_int32),
                 ("row_shift", ctypes.c_int32), ("row_mask", ctypes.c_int32), ("chunk_shift", ctypes.c_int32),
-                ("read_instr", ctypes.c_int32), ("read_cycles", ctypes.c_float), ("write_cycles", ctypes.c_float)]
+                ("read_instr", ctypes.c_int32), ("read_cycles", ctypes.c_float), ("write_cycles", ctypes.c_float),
+                ("row_shift2", ctypes.c_int32), ("row_mask2", ctypes.c_int32), ("chunk_shift2", ctypes.c_int32)]
 
 
 class GemmPlan(ctypes.Structure):

@@ -93,7 +93,10 @@ typedef struct frisk_gemm_desc {
 } frisk_gemm_desc;
 
 /* XOR swizzle of an LDS tile: 16-byte chunk index c of row r is stored at
- * chunk  c ^ (((r >> row_shift) & row_mask) << chunk_shift).  This is the
+ * chunk  c ^ (((r >> row_shift) & row_mask) << chunk_shift)
+ *          ^ (((r >> row_shift2) & row_mask2) << chunk_shift2)
+ * (the second term is absent when row_mask2 == 0; the tiles read by transpose
+ * reads for 16-row MFMA atoms use it).  This is the
  * representation of the reference's makeQuarter/Half/FullBankSwizzle layouts
  * (lib/Dialect/Frisk/IR/FriskOps.cpp:500-558), with the parameters chosen for
  * the gfx950 LDS instead of by the column-count rule of :560-618. */
@@ -104,6 +107,7 @@ typedef struct frisk_lds_layout {
   int32_t read_instr;      /* 0 ds_read_b128, 1 ds_read_b64_tr_b16, 2 ds_read_b64_tr_b8, 3 ds_read_b32 */
   float read_cycles;       /* modelled LDS cycles per wave-wide fragment read */
   float write_cycles;      /* modelled LDS cycles per KiB staged */
+  int32_t row_shift2, row_mask2, chunk_shift2; /* second XOR term, all 0 when unused */
 } frisk_lds_layout;
 
 typedef struct frisk_gemm_plan {

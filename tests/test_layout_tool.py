@@ -38,7 +38,8 @@ def test_report_has_the_reference_schema_and_consistent_maps(argv):
         i, j = L.grid(rows, cols)
         (idx,) = L.eval_affine_map(e["forward_index"], i, j)
         sw = e["swizzle"]
-        lay = R.LdsLayout(rows=rows, row_bytes=cols * es, k_contiguous=1, row_shift=sw["row_shift"], row_mask=sw["row_mask"], chunk_shift=sw["chunk_shift"])
+        lay = R.LdsLayout(rows=rows, row_bytes=cols * es, k_contiguous=1, row_shift=sw["row_shift"], row_mask=sw["row_mask"], chunk_shift=sw["chunk_shift"],
+                          row_shift2=sw["row_shift2"], row_mask2=sw["row_mask2"], chunk_shift2=sw["chunk_shift2"])
         for rr, cc in zip(np.random.default_rng(2).integers(0, rows, 200), np.random.default_rng(3).integers(0, cols, 200)):
             assert R.lds_offset(lay, int(rr), int(cc) * es) == int(idx[rr, cc]) * es
         assert len(np.unique(idx)) == rows * cols

@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), "libfrisk_hip.so does not export %s" % name
     assert sorted(R.EXPORTS) == declared
     assert lib.frisk_hip_abi_version() == R.ABI_VERSION
-    assert ctypes.sizeof(R.GemmDesc) == 104 and ctypes.sizeof(R.LdsLayout) == 36
+    assert ctypes.sizeof(R.GemmDesc) == 104 and ctypes.sizeof(R.LdsLayout) == 48
 
 
 def test_plans_of_the_benchmark_configurations():
@@ -56,8 +56,10 @@ def test_fp16_tile_layouts_are_conflict_free_in_the_model():
     a, b = p.lds_a, p.lds_b
     assert (a.rows, a.row_bytes, a.read_instr) == (256, 128, 0) and (b.rows, b.row_bytes, b.read_instr) == (64, 512, 1)
     # ds_read_b128 at its floor; the transpose reads of the 16x16x32 atoms put two K groups (K rows 8 apart) into one half wave,
-    # which the row-XOR swizzle family cannot separate: 2 passes per half instead of the floor of 3 cycles per instruction
-    assert a.read_cycles == 4.0 and b.read_cycles == 4.0
+    # which a single row-XOR term cannot separate (2 passes per half, 4 cycles); the second term on K-row bit 3 sends the
+    # groups to the two 32-byte halves of a 64-byte unit: the floor of 3 cycles per instruction
+    assert a.read_cycles == 4.0 and b.read_cycles == 3.0
+    assert (b.row_shift, b.row_mask, b.chunk_shift, b.row_shift2, b.row_mask2, b.chunk_shift2) == (0, 3, 2, 3, 1, 1)
     p = R.plan(R.make_desc(R.F16, 2048, 2048, 2048))   # 128x128 tiles of 32x32x16 atoms: both at their floors
     assert (p.mfma_m, p.lds_a.read_cycles, p.lds_b.read_cycles) == (32, 4.0, 3.0)
 
