@@ -174,10 +174,11 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
     c = k->wk > 1 ? 0.8 : (elem_size(k->dtype) == 1 ? 0.85 : 0.25);
   } else if (area >= 256 * 256) {
     c = k->wm * k->wn > 4 ? 1.56 : (k->stages_b > k->stages ? 1.5 : 1.55);  // 2 + 3 ring < 2 + 2 < 8 waves
-    // 16x16 atoms: the same cycles at a higher clock when every CU is busy (fp16 4096^3 NT 100 against 112 us); with an operand
-    // read by transpose reads (2-way bank conflicts there) less of it is left (NN 104 against 108), and a grid below one
-    // round is not limited by the clock (3072^3 NN 68 against 65)
-    if (k->atom == 16) c *= (!k->transA && k->transB) ? 0.93 : (tiles >= 256 ? 0.97 : 1.06);
+    // 16x16 atoms: the same cycles at a higher clock when most CUs are busy (fp16 4096^3 NT 100 against 112 us); with an operand
+    // read by transpose reads (twice the LDS instructions) less of it is left (NN 104 against 108).  How full the round is decides:
+    // 192 or 196 tiles, NN 78 against 82 us (3584^3) and 164 against 172 (4096x3072x8192), TN 79 against 85 and 169 against 182;
+    // 144 tiles (3072^3), where the clock is not the limit, NN 61 against 59, TN even
+    if (k->atom == 16) c *= (!k->transA && k->transB) ? 0.93 : (tiles >= 176 ? 0.96 : 1.06);
   } else if (area >= 256 * 128) {
     c = 0.93;
   } else {
