@@ -18,9 +18,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "i8": 5033.2, "e4m3": 5033.2, "f32": 157.3}
-# L2-miss bytes of one fp16 4096^3 launch from rocprofv3 counters: FETCH_SIZE 98 451.0 KiB x 2.00 (the factor a 1 GiB
-# copy shows for this counter) + WRITE_SIZE 37 388.3 KiB x 1.00; see profiles/bench_kernels_f16_4096_i8_4096_fp8_skinny.md
-TRAFFIC_BYTES_F16_4096 = int((98451.0 * 2.0 + 37388.3) * 1024)
+# L2-miss bytes of one fp16 4096^3 launch from rocprofv3 counters: FETCH_SIZE 98 458.0 KiB x 2.00 (the factor a 1 GiB
+# copy shows for this counter) + WRITE_SIZE 36 371.4 KiB x 1.00; see profiles/bench_kernels_f16_4096_i8_4096_fp8_skinny.md
+TRAFFIC_BYTES_F16_4096 = int((98458.0 * 2.0 + 36371.4) * 1024)
 
 
 SETTLE_MS = 100.0
