@@ -243,3 +243,14 @@ def test_planner_ranks_variants_by_estimated_time():
         p = R.plan(R.make_desc(R.F16, *shape, **kw))
         assert (p.tail_tiles, p.tail_split) == (0, 1) and p.workspace_bytes == 0, shape
     assert not pick(R.F16, 64, 384, 2048).endswith("_guard") and pick(R.F16, 65, 384, 2048).endswith("_guard")
+
+
+def test_atom_choice_follows_the_fill_of_the_round():
+    """16-bit 256x256 tiles: K-contiguous operands (NT) always take the 16x16x32 atoms; layouts with a transpose-read operand
+    take them from 176 tiles of a round of 256 up (measured crossover between 144 and 192 tiles)"""
+    for dt in (R.F16, R.BF16):
+        for (M, N, K), tA, tB, atom in (((3072, 3072, 3072), 0, 0, 32), ((3072, 3072, 3072), 1, 0, 32), ((3072, 3072, 3072), 0, 1, 16),
+                                        ((3584, 3584, 3584), 0, 0, 16), ((3584, 3584, 3584), 1, 1, 16), ((4096, 3072, 8192), 1, 0, 16),
+                                        ((4096, 4096, 4096), 0, 0, 16), ((8192, 8192, 8192), 0, 1, 16)):
+            p = R.plan(R.make_desc(dt, M, N, K, transA=tA, transB=tB))
+            assert (p.tile_m, p.tile_n, p.mfma_m) == (256, 256, atom), (dt, M, N, K, tA, tB, p.mfma_m)
