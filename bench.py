@@ -3,62 +3,121 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One step = one launch of the fp16 4096^3 NN GEMM (fp32 accumulate, fp16 out,
-inputs N(0,1)/sqrt(K), seed 1) through the C ABI, inputs resident in HBM.
-Prints ONE JSON line: whole-job TFLOP/s, the MFMA roofline of the kernel and
-the CPU oracle timed on the host cores beside it.
+One step = one launch of the fp16 4096^3 NN GEMM (fp32 accumulate, fp16 out, inputs N(0,1)/sqrt(K)) through the C ABI,
+inputs resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s, the MFMA roofline of the kernel (against the nominal
+peak and against the rate an MFMA-only loop sustains on this box in the same run), the other configurations of the
+metric timed the same way, and the CPU oracle timed on the host cores beside them.
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+# MI355X published dense peaks (TFLOP/s or TOP/s) and what one CU does per clock for each type (256 CUs x 2.4 GHz)
 PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "i8": 5033.2, "e4m3": 5033.2, "f32": 157.3}
-# L2-miss bytes of one fp16 4096^3 launch from rocprofv3 counters: FETCH_SIZE 98 458.0 KiB x 2.00 (the factor a 1 GiB
-# copy shows for this counter) + WRITE_SIZE 36 371.4 KiB x 1.00; see profiles/bench_kernels_f16_4096_i8_4096_fp8_skinny.md
+FLOPS_PER_CU_CLK = {"f16": 4096, "bf16": 4096, "i8": 8192, "e4m3": 8192, "f32": 256}
+# L2-miss bytes of one fp16 4096^3 launch, a constant taken from rocprofv3 counters (not measured by this run):
+# FETCH_SIZE 98 458.0 KiB x 2.00 (the factor a 1 GiB copy shows for this counter) + WRITE_SIZE 36 371.4 KiB x 1.00
 TRAFFIC_BYTES_F16_4096 = int((98458.0 * 2.0 + 36371.4) * 1024)
-
+TRAFFIC_SOURCE = "constant from profiles/bench_kernels_f16_4096_i8_4096_fp8_skinny.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE), not measured by this run"
 
 SETTLE_MS = 100.0
 
 
-def settle(torch, launch, stream):
-    """Untimed launches until SETTLE_MS of GPU time have passed.  After an idle period the part's power management
-    first overshoots and then takes about 50 ms of continuous load to reach its steady clocks (launch time goes
+def settle(torch, launch, stream, ms=SETTLE_MS):
+    """Untimed launches until `ms` of GPU time have passed.  After an idle period the part's power management first
+    overshoots and then takes about 50 ms of continuous load to reach its steady clocks (launch time goes
     122 -> 145 -> 116 us over the first 400 launches of the fp16 4096^3 kernel; the vendor library shows the same
     curve), so a short warm-up would time the transient, not the kernel."""
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     spent = 0.0
-    while spent < SETTLE_MS:
+    while spent < ms:
         e0.record(stream)
-        for _ in range(50):
+        for _ in range(20):
             launch()
         e1.record(stream)
         e1.synchronize()
         spent += e0.elapsed_time(e1)
 
 
-def gpu_time_gemm(R, torch, desc, ptrs, steps, warmup):
-    """returns (wall seconds for `steps` launches, mean kernel ms from HIP events on the launch stream)"""
-    stream = torch.cuda.current_stream()
-    s = stream.cuda_stream
-    settle(torch, lambda: R.gemm(desc, *ptrs, None, 0, s), stream)
+def time_launches(torch, launch, steps, warmup, stream):
+    """`launch` is timed three ways on `stream` (the stream the kernels are launched on), after the settle period:
+    wall clock around `steps` back-to-back launches (bracketed by synchronize), one HIP event pair around the same
+    launches (mean kernel time), and one HIP event pair per launch in a second pass (median and min)."""
+    settle(torch, launch, stream)
     for _ in range(warmup):
-        R.gemm(desc, *ptrs, None, 0, s)
+        launch()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record(stream)
     for _ in range(steps):
-        R.gemm(desc, *ptrs, None, 0, s)
+        launch()
     e1.record(stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    return wall, e0.elapsed_time(e1) / steps
+    mean_ms = e0.elapsed_time(e1) / steps
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in pairs:
+        a.record(stream)
+        launch()
+        b.record(stream)
+    torch.cuda.synchronize()
+    each = [a.elapsed_time(b) for a, b in pairs]
+    return {"wall_s": wall, "mean_ms": mean_ms, "median_ms": statistics.median(each), "min_ms": min(each)}
+
+
+def mfma_leg(name, dtype_key, flops, t, extra=None):
+    """one MFMA-bound configuration: achieved rate from the mean kernel time, fraction of the nominal peak"""
+    achieved = flops / (t["mean_ms"] * 1e-3) / 1e12
+    out = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS[dtype_key], "unit": "TOP/s" if dtype_key == "i8" else "TFLOP/s",
+           "frac": round(achieved / PEAK_TFLOPS[dtype_key], 4), "kernel_ms": round(t["mean_ms"], 5),
+           "kernel_ms_median": round(t["median_ms"], 5), "kernel_ms_min": round(t["min_ms"], 5), "workload": name}
+    if extra:
+        out.update(extra)
+    return out
+
+
+def mfma_ceiling(torch, HW, stream, cus):
+    """The rate a loop of nothing but MFMAs sustains on this box, per instruction kind, with pseudo-random operand
+    registers (the values matter: the part is power-limited and constant operands draw less).  One wave per SIMD,
+    accumulators of a 128 x 128 wave tile.  Also the shader clock that rate implies: the loop needs a known number of
+    matrix-pipe cycles."""
+    out = {}
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for kind, (name, dtype_key) in HW.LOOP_KINDS.items():
+        iters = 4000
+        run = lambda: HW.mfma_loop(kind, iters, True, cus, stream.cuda_stream)
+        settle(torch, run, stream, 60.0)
+        times = []
+        for _ in range(5):
+            e0.record(stream)
+            run()
+            e1.record(stream)
+            e1.synchronize()
+            times.append(e0.elapsed_time(e1))
+        ms = statistics.median(times)
+        rate = HW.mfma_loop_flops(kind, iters, cus) / (ms * 1e-3) / 1e12
+        out[name] = {"dtype": dtype_key, "rate": round(rate, 1), "frac_of_nominal": round(rate / PEAK_TFLOPS[dtype_key], 4),
+                     "implied_clock_mhz": round(HW.mfma_loop_cycles(kind, iters) / (ms * 1e3), 1), "ms": round(ms, 4)}
+    e0.record(stream)
+    HW.mfma_loop(0, 4000, False, cus, stream.cuda_stream)
+    e1.record(stream)
+    e1.synchronize()
+    ms = e0.elapsed_time(e1)
+    out["f16 32x32x16, constant operands"] = {"dtype": "f16", "rate": round(HW.mfma_loop_flops(0, 4000, cus) / (ms * 1e-3) / 1e12, 1),
+                                              "implied_clock_mhz": round(HW.mfma_loop_cycles(0, 4000) / (ms * 1e3), 1), "ms": round(ms, 4)}
+    return out
+
+
+def sustained_peak(ceiling, dtype_key):
+    """best MFMA-only rate any atom of this element type sustained in this run"""
+    return max(v["rate"] for k, v in ceiling.items() if v["dtype"] == dtype_key and "constant" not in k)
 
 
 def cpu_baseline(M, N, K):
@@ -84,6 +143,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only-headline", action="store_true", help="time the fp16 and int8 4096^3 kernels only (for profiler runs)")
     ap.add_argument("--copy-mib", type=int, default=0,
                     help="also run 3 plain device copies of this many MiB first: a kernel of known traffic to scale profiler byte counters by")
     a = ap.parse_args()
@@ -92,10 +152,16 @@ def main():
 
     import torch
     from frisk_amd import runtime as R
+    from frisk_amd import hwcheck as HW
 
     R.lib()
     assert torch.cuda.is_available(), "bench.py needs an MI355X"
     dev = torch.device("cuda:0")
+    prop = torch.cuda.get_device_properties(0)
+    cus = prop.multi_processor_count
+    clock_khz = getattr(prop, "clock_rate", 0) or 0
+    stream = torch.cuda.current_stream()
+    cs = stream.cuda_stream
     if a.copy_mib:
         src = torch.empty(a.copy_mib << 20, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)
@@ -103,147 +169,202 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    M = N = K = 4096
     g = torch.Generator(device=dev)
     g.manual_seed(1)
+
+    def gemm_launcher(desc, ptrs, ws=None, ws_bytes=0):
+        return lambda: R.gemm(desc, *ptrs, ws, ws_bytes, cs)
+
+    # ---------------------------------------------------------------- headline: fp16 4096^3 NN (BASELINE configs[1])
+    M = N = K = 4096
+    flops = 2.0 * M * N * K
     A = (torch.randn(M, K, device=dev, generator=g) / K ** 0.5).half()
     B = (torch.randn(K, N, device=dev, generator=g) / K ** 0.5).half()
     C = torch.empty(M, N, device=dev, dtype=torch.float16)
     desc = R.make_desc(R.F16, M, N, K, dtype_out=R.F16)
     plan = R.plan(desc)
-    ptrs = (A.data_ptr(), B.data_ptr(), C.data_ptr(), None, None)
-    wall, kern_ms = gpu_time_gemm(R, torch, desc, ptrs, a.steps, a.warmup)
-    flops = 2.0 * M * N * K
-    value = flops * a.steps / wall / 1e12
-    achieved = flops / (kern_ms * 1e-3) / 1e12
+    t16 = time_launches(torch, gemm_launcher(desc, (A.data_ptr(), B.data_ptr(), C.data_ptr(), None, None)), a.steps, a.warmup, stream)
+    value = flops * a.steps / t16["wall_s"] / 1e12
+    achieved = flops / (t16["mean_ms"] * 1e-3) / 1e12
 
-    # the same launch with operands rotating over 4 buffer sets (4 x 96 MiB > the 256 MiB last-level cache): every
-    # launch streams A and B from HBM instead of finding them cached
-    sets = [(A, B, C)] + [((torch.randn(M, K, device=dev, generator=g) / K ** 0.5).half(), (torch.randn(K, N, device=dev, generator=g) / K ** 0.5).half(),
-                           torch.empty(M, N, device=dev, dtype=torch.float16)) for _ in range(3)]
-    stream0 = torch.cuda.current_stream()
-
-    def cold(n):
-        for i in range(n):
-            a_, b_, c_ = sets[i % 4]
-            R.gemm(desc, a_.data_ptr(), b_.data_ptr(), c_.data_ptr(), None, None, None, 0, stream0.cuda_stream)
-    settle(torch, lambda: cold(4), stream0)
-    ce0, ce1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    ce0.record(stream0)
-    cold(a.steps)
-    ce1.record(stream0)
-    torch.cuda.synchronize()
-    cold_ms = ce0.elapsed_time(ce1) / a.steps
-    del sets
-
-    # second headline shape of the metric: W8A8 int8 4096^3 with the dequant epilogue (reported, not the timed value)
+    # second headline shape of the metric: W8A8 int8 4096^3 with the dequant epilogue
     A8 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
     B8 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev, generator=g)
     sA = torch.rand(M, device=dev, generator=g) * 0.019 + 0.001
     sB = torch.rand(N, device=dev, generator=g) * 0.019 + 0.001
     C8 = torch.empty(M, N, device=dev, dtype=torch.float16)
     d8 = R.make_desc(R.I8, M, N, K, dtype_out=R.F16, epilogue=R.EPI_ROW_COL_SCALE)
-    _, i8_ms = gpu_time_gemm(R, torch, d8, (A8.data_ptr(), B8.data_ptr(), C8.data_ptr(), sA.data_ptr(), sB.data_ptr()),
-                             a.steps, a.warmup)
-    i8_tops = flops / (i8_ms * 1e-3) / 1e12
-
-    # HBM-bound shape of the configuration list: fp8 e4m3 M=32, N=K=8192 (B stored [N][K]), per-tensor scales, bf16 out.
-    # B rotates over 6 buffers (384 MiB > the 256 MiB last-level cache) so every launch streams it from HBM.
-    Ms, Ns, Ks = 32, 8192, 8192
-    Af = torch.randn(Ms, Ks, device=dev, generator=g).to(torch.float8_e4m3fn)
-    Bf = [torch.randn(Ns, Ks, device=dev, generator=g).to(torch.float8_e4m3fn) for _ in range(6)]
-    Cf = torch.empty(Ms, Ns, device=dev, dtype=torch.bfloat16)
-    one = torch.ones(1, device=dev)
-    df = R.make_desc(R.E4M3, Ms, Ns, Ks, dtype_out=R.BF16, transB=True, epilogue=R.EPI_TENSOR_SCALE)
-    pf = R.plan(df)
-    ws_bytes = R.workspace_bytes(df)
-    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
-    stream = torch.cuda.current_stream()
-
-    def skinny(n):
-        for i in range(n):
-            R.gemm(df, Af.data_ptr(), Bf[i % len(Bf)].data_ptr(), Cf.data_ptr(), one.data_ptr(), one.data_ptr(),
-                   ws.data_ptr() if ws_bytes else None, ws_bytes, stream.cuda_stream)
-    settle(torch, lambda: skinny(1), stream)
-    skinny(a.warmup)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    skinny(a.steps)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    sk_ms = e0.elapsed_time(e1) / a.steps
-    sk_bytes = Ms * Ks + Ns * Ks + 2 * Ms * Ns + 8
-    sk_gbs = sk_bytes / (sk_ms * 1e-3) / 1e9
-    del Bf
-
-    # the dialect's data-movement ops on a 32768 x 8192 f16 view (512 MiB per array: twice the last-level cache)
-    def time_op(fn):
-        settle(torch, fn, stream)
-        e0.record(stream)
-        for _ in range(20):
-            fn()
-        e1.record(stream)
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / 20
-
-    orows, ocols = 32768, 8192
-    src16 = torch.randn(orows, ocols, device=dev, generator=g).half()
-    dst16 = torch.empty_like(src16)
-    red = torch.empty(orows, device=dev, dtype=torch.float16)
-    rws_bytes = R.reduce_workspace_bytes(R.F16, orows, ocols, 0)
-    rws = torch.empty(max(rws_bytes, 16), dtype=torch.uint8, device=dev)
-    cs = stream.cuda_stream
-    nbytes = orows * ocols * 2
-    ops = {}
-    for name, moved, fn in (
-            ("fill", nbytes, lambda: R.fill(R.F16, dst16.data_ptr(), orows, ocols, ocols, 1.5, cs)),
-            ("copy", 2 * nbytes, lambda: R.copy(R.F16, src16.data_ptr(), ocols, R.F16, dst16.data_ptr(), ocols, orows, ocols, cs)),
-            ("reduce_dim1_add", nbytes, lambda: R.reduce(R.F16, src16.data_ptr(), orows, ocols, ocols, 1, "add", True, red.data_ptr(), None, 0, cs)),
-            ("reduce_dim0_max", nbytes, lambda: R.reduce(R.F16, src16.data_ptr(), orows, ocols, ocols, 0, "max", True, red.data_ptr(), rws.data_ptr(),
-                                                         rws_bytes, cs))):
-        ms = time_op(fn)
-        ops[name] = {"GB/s": round(moved / (ms * 1e-3) / 1e9, 1), "frac_of_8TB/s": round(moved / (ms * 1e-3) / 8e12, 4), "kernel_ms": round(ms, 5)}
-    # the reference's @online_softmax sketch at the same size class: one read and one write of every element
-    ms = time_op(lambda: R.softmax(R.F16, src16.data_ptr(), ocols, dst16.data_ptr(), ocols, orows, ocols, 1.25, None, cs))
-    ops["softmax_rows"] = {"GB/s": round(2 * nbytes / (ms * 1e-3) / 1e9, 1), "frac_of_8TB/s": round(2 * nbytes / (ms * 1e-3) / 8e12, 4), "kernel_ms": round(ms, 5)}
-    del src16, dst16
-
-    # fused attention forward at the shape of the reference's sketch: 1 x 32 heads x 4096 x 128, fp16
-    ab, ah, aseq, ad = 1, 32, 4096, 128
-    aq, ak, av = (torch.randn(ab * ah, aseq, ad, device=dev, generator=g).half() for _ in range(3))
-    ao = torch.empty_like(aq)
-    adesc = R.make_attention_desc(R.F16, ab, ah, aseq, aseq, ad)
-    attn_ms = time_op(lambda: R.attention(adesc, aq.data_ptr(), ak.data_ptr(), av.data_ptr(), ao.data_ptr(), None, cs))
-    attn_tflops = 4.0 * ab * ah * aseq * aseq * ad / (attn_ms * 1e-3) / 1e12
-    del aq, ak, av, ao
+    t8 = time_launches(torch, gemm_launcher(d8, (A8.data_ptr(), B8.data_ptr(), C8.data_ptr(), sA.data_ptr(), sB.data_ptr())), a.steps, a.warmup, stream)
+    legs = {"int8_4096": mfma_leg("W8A8 int8 4096^3 NN, int32 accumulate, per-row/per-column fp32 scales, fp16 out (configs[3])", "i8", flops, t8,
+                                  {"kernel": R.kernel_names()[R.plan(d8).kernel_id]})}
+    del A8, B8, C8
 
     line = {
         "metric": "GEMM TFLOP/s at 4096^3 fp16 (fp32 accumulate), 1 GPU",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": round(wall / a.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": round(t16["wall_s"] / a.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic", "settle_ms": SETTLE_MS,
-        "config": {"workload": "fp16 GEMM M=N=K=4096 NN row-major, N(0,1)/sqrt(K) seed 1, fp32 accumulate, fp16 out",
-                   "kernel": R.kernel_names()[plan.kernel_id], "grid": [plan.grid_x, plan.grid_y],
-                   "lds_bytes": plan.lds_bytes},
+        "config": {"workload": "fp16 GEMM M=N=K=4096 NN row-major, N(0,1)/sqrt(K), fp32 accumulate, fp16 out; values drawn on the device by "
+                               "torch's generator (seed 1), not by the parity tests' counter-based generator",
+                   "kernel": R.kernel_names()[plan.kernel_id], "grid": [plan.grid_x, plan.grid_y], "lds_bytes": plan.lds_bytes,
+                   "library": R.LIB_PATH},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_TFLOPS["f16"], 4), "traffic": TRAFFIC_BYTES_F16_4096, "traffic_unit": "bytes per launch",
-                     "kernel_ms": round(kern_ms, 5), "kernel_ms_rotating_4_buffer_sets": round(cold_ms, 5)},
-        "int8_4096": {"value": round(i8_tops, 2), "unit": "TOPS", "peak": PEAK_TFLOPS["i8"],
-                      "frac": round(i8_tops / PEAK_TFLOPS["i8"], 4), "kernel_ms": round(i8_ms, 5),
-                      "workload": "W8A8 int8 4096^3 NN, int32 accumulate, per-row/per-column fp32 scales, fp16 out"},
-        "fp8_skinny_32x8192x8192": {"bound": "hbm", "achieved": round(sk_gbs, 1), "peak": 8000.0, "unit": "GB/s",
-                                    "frac": round(sk_gbs / 8000.0, 4), "kernel_ms": round(sk_ms, 5),
-                                    "kernel": R.kernel_names()[pf.kernel_id], "split_k": pf.split_k,
-                                    "workload": "fp8 e4m3 M=32 N=K=8192 NT, per-tensor scales, bf16 out; algorithmic bytes "
-                                                "|A|+|B|+|C|+scales per launch, B rotating over 6 buffers"},
-        "tile_ops_32768x8192_f16": ops,
-        "attention_1x32x4096x128_f16": {"bound": "mfma", "achieved": round(attn_tflops, 2), "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
-                                        "frac": round(attn_tflops / PEAK_TFLOPS["f16"], 4), "kernel_ms": round(attn_ms, 5),
-                                        "workload": "softmax(Q K^T / sqrt(128)) V, 32 heads, 4096 queries x 4096 keys, head_dim 128, "
-                                                    "fp16 in / out, fp32 accumulate; 4 * heads * seq^2 * head_dim flops per launch"},
+                     "traffic_source": TRAFFIC_SOURCE, "kernel_ms": round(t16["mean_ms"], 5), "kernel_ms_median": round(t16["median_ms"], 5),
+                     "kernel_ms_min": round(t16["min_ms"], 5)},
+        "device": {"name": prop.name, "compute_units": cus, "clock_mhz_reported": round(clock_khz / 1e3, 1),
+                   "peak_from_device_properties": {k: round(cus * clock_khz * 1e3 * v / 1e12, 1) for k, v in FLOPS_PER_CU_CLK.items()},
+                   "peak_nominal": PEAK_TFLOPS, "note": "CUs x reported clock x flops per CU and clock (4096 16-bit, 8192 8-bit, 256 fp32)"},
     }
-    if not a.no_cpu:
+
+    if not a.only_headline:
+        # the same launch with operands rotating over 4 buffer sets (4 x 96 MiB > the 256 MiB last-level cache): every
+        # launch streams A and B from HBM instead of finding them cached
+        sets = [(A, B, C)] + [((torch.randn(M, K, device=dev, generator=g) / K ** 0.5).half(), (torch.randn(K, N, device=dev, generator=g) / K ** 0.5).half(),
+                               torch.empty(M, N, device=dev, dtype=torch.float16)) for _ in range(3)]
+        turn = [0]
+
+        def cold():
+            a_, b_, c_ = sets[turn[0] % 4]
+            turn[0] += 1
+            R.gemm(desc, a_.data_ptr(), b_.data_ptr(), c_.data_ptr(), None, None, None, 0, cs)
+        line["roofline"]["kernel_ms_rotating_4_buffer_sets"] = round(time_launches(torch, cold, a.steps, a.warmup, stream)["mean_ms"], 5)
+        del sets
+
+        # the same problem with B stored [N][K]: both operands K-contiguous in LDS, no transpose reads
+        Bt = B.t().contiguous()
+        dnt = R.make_desc(R.F16, M, N, K, dtype_out=R.F16, transB=True)
+        tnt = time_launches(torch, gemm_launcher(dnt, (A.data_ptr(), Bt.data_ptr(), C.data_ptr(), None, None)), a.steps, a.warmup, stream)
+        legs["fp16_4096_nt"] = mfma_leg("fp16 4096^3 NT (B stored [N][K])", "f16", flops, tnt, {"kernel": R.kernel_names()[R.plan(dnt).kernel_id]})
+        del Bt
+
+        # what the matrix pipe sustains on this box when nothing else runs
+        ceiling = mfma_ceiling(torch, HW, stream, cus)
+        line["mfma_ceiling"] = ceiling
+        sp = sustained_peak(ceiling, "f16")
+        line["roofline"]["sustained_peak"] = sp
+        line["roofline"]["frac_of_sustained"] = round(achieved / sp, 4)
+        for key, dk in (("int8_4096", "i8"), ("fp16_4096_nt", "f16")):
+            legs[key]["sustained_peak"] = sustained_peak(ceiling, dk)
+            legs[key]["frac_of_sustained"] = round(legs[key]["achieved"] / legs[key]["sustained_peak"], 4)
+
+        # configs[0]: fp32 1024^3 built through the IR builder, lowered by frisk_ffi.runtime, launched through the C ABI
+        import frisk_amd  # noqa: F401  (puts the builder package on the path)
+        import frisk as F
+        M1 = 1024
+        h = F.create_session()
+        kern = h.tiled_gemm("matmul", M1, M1, M1, "fp32", tile=(128, 128, 32), threads=256)
+        A1 = torch.rand(M1, M1, device=dev, generator=g) * 2 - 1
+        B1 = torch.rand(M1, M1, device=dev, generator=g) * 2 - 1
+        C1 = torch.empty(M1, M1, device=dev)
+        p1 = [A1.data_ptr(), B1.data_ptr(), C1.data_ptr()]
+        t1 = time_launches(torch, lambda: F.runtime.launch(kern, p1, cs), a.steps, a.warmup, stream)
+        legs["fp32_1024_builder"] = mfma_leg("fp32 1024^3 NN, U[-1,1], built with the IR builder and launched by frisk_ffi.runtime (configs[0]); "
+                                             "the time includes the builder's matching and planning on the host", "f32", 2.0 * M1 ** 3, t1)
+        d1 = R.make_desc(R.F32, M1, M1, M1)
+        t1c = time_launches(torch, gemm_launcher(d1, (A1.data_ptr(), B1.data_ptr(), C1.data_ptr(), None, None)), a.steps, a.warmup, stream)
+        legs["fp32_1024"] = mfma_leg("fp32 1024^3 NN through the C ABI, planner's choice of tile", "f32", 2.0 * M1 ** 3, t1c,
+                                     {"kernel": R.kernel_names()[R.plan(d1).kernel_id]})
+
+        # configs[2]: bf16 8192^3 NT; configs[4], square part: fp8 e4m3 8192^3 NT with per-tensor scales, bf16 out
+        Mb = 8192
+        big_steps = max(5, min(a.steps, 40))
+        Ab = (torch.randn(Mb, Mb, device=dev, generator=g) * 0.02).bfloat16()
+        Bb = (torch.randn(Mb, Mb, device=dev, generator=g) * 0.02).bfloat16()
+        Cb = torch.empty(Mb, Mb, device=dev, dtype=torch.bfloat16)
+        db = R.make_desc(R.BF16, Mb, Mb, Mb, dtype_out=R.BF16, transB=True)
+        tb = time_launches(torch, gemm_launcher(db, (Ab.data_ptr(), Bb.data_ptr(), Cb.data_ptr(), None, None)), big_steps, 3, stream)
+        legs["bf16_8192_nt"] = mfma_leg("bf16 8192^3 NT, N(0,1)*0.02, fp32 accumulate, bf16 out (configs[2])", "bf16", 2.0 * Mb ** 3, tb,
+                                        {"kernel": R.kernel_names()[R.plan(db).kernel_id], "steps": big_steps,
+                                         "sustained_peak": sustained_peak(ceiling, "bf16")})
+        legs["bf16_8192_nt"]["frac_of_sustained"] = round(legs["bf16_8192_nt"]["achieved"] / legs["bf16_8192_nt"]["sustained_peak"], 4)
+        A8f = (torch.randn(Mb, Mb, device=dev, generator=g) * 100).clamp(-448, 448).to(torch.float8_e4m3fn)
+        B8f = (torch.randn(Mb, Mb, device=dev, generator=g) * 100).clamp(-448, 448).to(torch.float8_e4m3fn)
+        one = torch.full((1,), 0.01, device=dev)
+        d8f = R.make_desc(R.E4M3, Mb, Mb, Mb, dtype_out=R.BF16, transB=True, epilogue=R.EPI_TENSOR_SCALE)
+        t8f = time_launches(torch, gemm_launcher(d8f, (A8f.data_ptr(), B8f.data_ptr(), Cb.data_ptr(), one.data_ptr(), one.data_ptr())), big_steps, 3, stream)
+        legs["fp8_8192_nt"] = mfma_leg("fp8 e4m3 8192^3 NT, N(0,1) scaled to the e4m3 range, per-tensor fp32 scales, bf16 out (configs[4], square part)",
+                                       "e4m3", 2.0 * Mb ** 3, t8f, {"kernel": R.kernel_names()[R.plan(d8f).kernel_id], "steps": big_steps,
+                                                                    "sustained_peak": sustained_peak(ceiling, "e4m3")})
+        legs["fp8_8192_nt"]["frac_of_sustained"] = round(legs["fp8_8192_nt"]["achieved"] / legs["fp8_8192_nt"]["sustained_peak"], 4)
+        del Ab, Bb, Cb, A8f, B8f
+
+        # HBM-bound shape of the configuration list: fp8 e4m3 M=32, N=K=8192 (B stored [N][K]), per-tensor scales, bf16 out.
+        # B rotates over 6 buffers (384 MiB > the 256 MiB last-level cache) so every launch streams it from HBM.
+        Ms, Ns, Ks = 32, 8192, 8192
+        Af = torch.randn(Ms, Ks, device=dev, generator=g).to(torch.float8_e4m3fn)
+        Bf = [torch.randn(Ns, Ks, device=dev, generator=g).to(torch.float8_e4m3fn) for _ in range(6)]
+        Cf = torch.empty(Ms, Ns, device=dev, dtype=torch.bfloat16)
+        df = R.make_desc(R.E4M3, Ms, Ns, Ks, dtype_out=R.BF16, transB=True, epilogue=R.EPI_TENSOR_SCALE)
+        pf = R.plan(df)
+        ws_bytes = R.workspace_bytes(df)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        sk_turn = [0]
+
+        def skinny():
+            b_ = Bf[sk_turn[0] % len(Bf)]
+            sk_turn[0] += 1
+            R.gemm(df, Af.data_ptr(), b_.data_ptr(), Cf.data_ptr(), one.data_ptr(), one.data_ptr(), ws.data_ptr() if ws_bytes else None, ws_bytes, cs)
+        tsk = time_launches(torch, skinny, a.steps, a.warmup, stream)
+        sk_bytes = Ms * Ks + Ns * Ks + 2 * Ms * Ns + 8
+        sk_gbs = sk_bytes / (tsk["mean_ms"] * 1e-3) / 1e9
+        legs["fp8_skinny_32x8192x8192"] = {"bound": "hbm", "achieved": round(sk_gbs, 1), "peak": 8000.0, "unit": "GB/s", "frac": round(sk_gbs / 8000.0, 4),
+                                           "kernel_ms": round(tsk["mean_ms"], 5), "kernel_ms_median": round(tsk["median_ms"], 5),
+                                           "kernel_ms_min": round(tsk["min_ms"], 5), "kernel": R.kernel_names()[pf.kernel_id], "split_k": pf.split_k,
+                                           "workload": "fp8 e4m3 M=32 N=K=8192 NT, per-tensor scales, bf16 out (configs[4], decode part); algorithmic bytes "
+                                                       "|A|+|B|+|C|+scales per launch, B rotating over 6 buffers"}
+        del Bf
+
+        # the dialect's data-movement ops on a 32768 x 8192 f16 view (512 MiB per array: twice the last-level cache)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+        def time_op(fn):
+            settle(torch, fn, stream)
+            e0.record(stream)
+            for _ in range(20):
+                fn()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / 20
+
+        orows, ocols = 32768, 8192
+        src16 = torch.randn(orows, ocols, device=dev, generator=g).half()
+        dst16 = torch.empty_like(src16)
+        red = torch.empty(orows, device=dev, dtype=torch.float16)
+        rws_bytes = R.reduce_workspace_bytes(R.F16, orows, ocols, 0)
+        rws = torch.empty(max(rws_bytes, 16), dtype=torch.uint8, device=dev)
+        nbytes = orows * ocols * 2
+        ops = {}
+        for name, moved, fn in (
+                ("fill", nbytes, lambda: R.fill(R.F16, dst16.data_ptr(), orows, ocols, ocols, 1.5, cs)),
+                ("copy", 2 * nbytes, lambda: R.copy(R.F16, src16.data_ptr(), ocols, R.F16, dst16.data_ptr(), ocols, orows, ocols, cs)),
+                ("reduce_dim1_add", nbytes, lambda: R.reduce(R.F16, src16.data_ptr(), orows, ocols, ocols, 1, "add", True, red.data_ptr(), None, 0, cs)),
+                ("reduce_dim0_max", nbytes, lambda: R.reduce(R.F16, src16.data_ptr(), orows, ocols, ocols, 0, "max", True, red.data_ptr(), rws.data_ptr(),
+                                                             rws_bytes, cs))):
+            ms = time_op(fn)
+            ops[name] = {"GB/s": round(moved / (ms * 1e-3) / 1e9, 1), "frac_of_8TB/s": round(moved / (ms * 1e-3) / 8e12, 4), "kernel_ms": round(ms, 5)}
+        # the reference's @online_softmax sketch at the same size class: one read and one write of every element
+        ms = time_op(lambda: R.softmax(R.F16, src16.data_ptr(), ocols, dst16.data_ptr(), ocols, orows, ocols, 1.25, None, cs))
+        ops["softmax_rows"] = {"GB/s": round(2 * nbytes / (ms * 1e-3) / 1e9, 1), "frac_of_8TB/s": round(2 * nbytes / (ms * 1e-3) / 8e12, 4), "kernel_ms": round(ms, 5)}
+        del src16, dst16
+        line["tile_ops_32768x8192_f16"] = ops
+
+        # fused attention forward at the shape of the reference's sketch: 1 x 32 heads x 4096 x 128, fp16
+        ab, ah, aseq, ad = 1, 32, 4096, 128
+        aq, ak, av = (torch.randn(ab * ah, aseq, ad, device=dev, generator=g).half() for _ in range(3))
+        ao = torch.empty_like(aq)
+        adesc = R.make_attention_desc(R.F16, ab, ah, aseq, aseq, ad)
+        attn_ms = time_op(lambda: R.attention(adesc, aq.data_ptr(), ak.data_ptr(), av.data_ptr(), ao.data_ptr(), None, cs))
+        attn_tflops = 4.0 * ab * ah * aseq * aseq * ad / (attn_ms * 1e-3) / 1e12
+        del aq, ak, av, ao
+        line["attention_1x32x4096x128_f16"] = {"bound": "mfma", "achieved": round(attn_tflops, 2), "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
+                                               "frac": round(attn_tflops / PEAK_TFLOPS["f16"], 4), "frac_of_sustained": round(attn_tflops / sp, 4),
+                                               "kernel_ms": round(attn_ms, 5),
+                                               "workload": "softmax(Q K^T / sqrt(128)) V, 32 heads, 4096 queries x 4096 keys, head_dim 128, "
+                                                           "fp16 in / out, fp32 accumulate; 4 * heads * seq^2 * head_dim flops per launch"}
+
+    line.update(legs)
+    if not a.no_cpu and not a.only_headline:
         line["cpu_baseline"] = cpu_baseline(M, N, K)
     print(json.dumps(line))
 

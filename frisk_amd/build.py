@@ -1,6 +1,6 @@
 """Builds libfrisk_hip.so (HIP kernels + C ABI) for gfx950, in-tree.
 
-    python -m frisk_amd.build          # rebuild everything (HIP library + frisk_ffi extension)
+    python -m frisk_amd.build          # rebuild everything (HIP library, the device-check library, frisk_ffi extension)
     python -m frisk_amd.build --if-missing
 
 hipcc cross-compiles without a GPU; the resulting library is loaded from
@@ -18,6 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(CSRC, "build")
 LIB = os.path.join(LIBDIR, "libfrisk_hip.so")
+HWCHECK_LIB = os.path.join(LIBDIR, "libfrisk_hwcheck.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = [
@@ -59,6 +60,19 @@ def build(jobs=None, verbose=True):
     return LIB
 
 
+def build_hwcheck(verbose=True):
+    """libfrisk_hwcheck.so: device-side checks of the MFMA fragment conventions and the MFMA-only loop the benchmark times
+    (csrc/hwcheck.hip); used by the GPU tests and bench.py, never by the product library"""
+    os.makedirs(LIBDIR, exist_ok=True)
+    cmd = [HIPCC] + COMMON + ["-shared", os.path.join(CSRC, "hwcheck.hip"), "-o", HWCHECK_LIB]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building libfrisk_hwcheck.so failed:\n" + r.stderr)
+    if verbose:
+        print("built", HWCHECK_LIB)
+    return HWCHECK_LIB
+
+
 FFI_DIR = os.path.join(HERE, "ffi")
 FFI_SOURCES = ["ffi.cpp", "ir.cpp", "runtime.cpp"]
 
@@ -80,37 +94,16 @@ def build_ffi(verbose=True):
     return out
 
 
-def build_tools(verbose=True):
-    """the hardware probes the kernel designs rest on: the LDS cost model's (csrc/tools/lds_probe.hip -> lib/lds_probe) and the
-    matrix / vector pipe's (csrc/tools/pipe_probe.hip -> lib/pipe_probe)"""
-    os.makedirs(LIBDIR, exist_ok=True)
-    outs = []
-    for name in ("lds_probe", "pipe_probe"):
-        out = os.path.join(LIBDIR, name)
-        cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-               "-Wno-unused-value", os.path.join(CSRC, "tools", name + ".hip"), "-o", out]
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError("building %s failed:\n%s" % (name, r.stderr))
-        if verbose:
-            print("built", out)
-        outs.append(out)
-    return outs
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--if-missing", action="store_true")
     ap.add_argument("-j", type=int, default=None)
-    ap.add_argument("--tools", action="store_true", help="build only the hardware probes")
     a = ap.parse_args()
-    if a.tools:
-        build_tools()
-        return
     if a.if_missing and os.path.exists(LIB):
         print("present", LIB)
         return
     build(a.j)
+    build_hwcheck()
     build_ffi()
 
 

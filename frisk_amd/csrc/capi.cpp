@@ -400,9 +400,6 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
   p.M = (int)desc->M; p.N = (int)desc->N; p.K = (int)desc->K;
   p.tiles_m = plan.grid_y; p.tiles_n = plan.grid_x;
   p.group_m = group_rows(p.tiles_m, p.tiles_n);
-#ifdef FRISK_DEV_GROUP_ENV
-  if (const char* e = getenv("FRISK_GROUP_M")) p.group_m = std::max(1, std::min(atoi(e), p.tiles_m));
-#endif
   p.xcd_remap = plan.xcd_remap;
   p.epilogue = desc->epilogue; p.dtype_out = desc->dtype_out; p.accumulate = desc->clear_accum ? 0 : 1;
   const KernelEntry* k = kernels()[plan.kernel_id];

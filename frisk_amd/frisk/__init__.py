@@ -8,6 +8,6 @@ from .frisk_ffi.ir import *  # noqa: F401,F403
 from .frisk_ffi import ir, runtime  # noqa: F401
 from .common.utils import FriskHelper, create_context, create_session  # noqa: F401
 
-runtime.set_library(_os.environ.get("FRISK_HIP_LIB") or _os.path.join(_os.path.dirname(_os.path.dirname(_os.path.abspath(__file__))), "lib", "libfrisk_hip.so"))
+runtime.set_library(_os.path.join(_os.path.dirname(_os.path.dirname(_os.path.abspath(__file__))), "lib", "libfrisk_hip.so"))
 
 __all__ = [name for name in globals().keys() if not name.startswith("_")]

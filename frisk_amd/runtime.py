@@ -8,8 +8,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# FRISK_HIP_LIB points kernel developers at another build of the same library
-LIB_PATH = os.environ.get("FRISK_HIP_LIB") or os.path.join(_HERE, "lib", "libfrisk_hip.so")
+LIB_PATH = os.path.join(_HERE, "lib", "libfrisk_hip.so")
 
 ABI_VERSION = 1
 F32, F16, BF16, I8, E4M3, I32 = 0, 1, 2, 3, 4, 5

@@ -2,8 +2,8 @@
 """Writes tests/golden/lds_probe_gfx950.json: lane-address patterns and the LDS cycles per
 wave-wide instruction measured for them on an MI355X (16 waves of one work-group issuing the
 same access in a loop, time per instruction converted to cycles with the all-conflict case as the
-clock reference).  The measured numbers are copied from the output of the LDS probe
-(frisk_amd/csrc/tools/lds_probe.hip); the patterns are regenerated here from their definitions.
+clock reference).  The measured numbers are copied from the output of a stand-alone micro-benchmark run on the
+device (not kept in the tree); the patterns are regenerated here from their definitions.
 """
 import json
 import os

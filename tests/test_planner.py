@@ -25,6 +25,17 @@ def test_library_exports_every_declared_symbol():
     assert ctypes.sizeof(R.GemmDesc) == 104 and ctypes.sizeof(R.LdsLayout) == 48
 
 
+def test_device_check_library_loads_and_exports_its_entry_points():
+    from frisk_amd import hwcheck
+    lib = hwcheck.lib()
+    for name in hwcheck.EXPORTS:
+        assert hasattr(lib, name), "libfrisk_hwcheck.so does not export %s" % name
+    # pure host helpers: flops and matrix-pipe cycles of the MFMA-only loop (64 MFMAs of 32 cycles and 32768 flops per iteration)
+    assert hwcheck.mfma_loop_flops(0, 10, 256) == 10 * 64 * 32768 * 4 * 256
+    assert hwcheck.mfma_loop_cycles(0, 10) == 10 * 64 * 32 and hwcheck.mfma_loop_cycles(1, 10) == 10 * 128 * 16
+    assert hwcheck.mfma_loop_flops(4, 1, 1) == 2 * hwcheck.mfma_loop_flops(0, 1, 1) == hwcheck.mfma_loop_flops(6, 1, 1)
+
+
 def test_plans_of_the_benchmark_configurations():
     cases = [
         (R.F32, 1024, 1024, 1024, 0, 0, R.F32, (64, 64, 128)),   # 8 waves: two sets of four share each K tile
