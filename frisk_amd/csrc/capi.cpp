@@ -111,6 +111,7 @@ static int validate(const frisk_gemm_desc* d) {
     return fail(FRISK_ERR_EPILOGUE, "int32 output carries the raw accumulators; scales need a floating output type");
   if (d->policy < FRISK_POLICY_SQUARE || d->policy > FRISK_POLICY_FULL_COL)
     return fail(FRISK_ERR_TILE, "unknown wave policy %d", d->policy);
+  if (d->atom != 0 && d->atom != 16 && d->atom != 32) return fail(FRISK_ERR_TILE, "MFMA atoms have 32 or 16 rows, not %d", d->atom);
   if (d->M < 0 || d->N < 0 || d->K < 0) return fail(FRISK_ERR_SHAPE, "negative extent M=%lld N=%lld K=%lld", (long long)d->M, (long long)d->N, (long long)d->K);
   if (d->M > INT32_MAX || d->N > INT32_MAX || d->K > INT32_MAX) return fail(FRISK_ERR_SHAPE, "extent exceeds 2^31-1");
   const int64_t a_cols = d->transA ? d->M : d->K, b_cols = d->transB ? d->K : d->N;
@@ -227,7 +228,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   const auto& ks = kernels();
   int best = -1;
   double best_cost = 0.0;
-  bool any_layout = false, tile_requested = d->tile_m || d->tile_n || d->tile_k || d->waves_m || d->waves_n || d->stages;
+  bool any_layout = false, tile_requested = d->tile_m || d->tile_n || d->tile_k || d->waves_m || d->waves_n || d->stages || d->atom;
   auto search = [&](bool want_split) {
     for (size_t i = 0; i < ks.size(); ++i) {
       const KernelEntry* k = ks[i];
@@ -239,6 +240,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
       if (d->waves_m && d->waves_m != k->wm) continue;
       if (d->waves_n && d->waves_n != k->wn) continue;
       if (d->stages && d->stages != k->stages_b) continue;  // the deeper ring names the variant
+      if (d->atom && d->atom != k->atom) continue;
       if (want_split && !k->splitk) continue;
       // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
       if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
@@ -260,8 +262,8 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   if (best < 0) {
     if (!any_layout) return fail(FRISK_ERR_DTYPE, "no kernel compiled for dtype %d transA=%d transB=%d", d->dtype_ab, d->transA, d->transB);
     if (tile_requested)
-      return fail(FRISK_ERR_TILE, "no compiled kernel with tile %dx%dx%d waves %dx%d divides M=%lld N=%lld K=%lld", d->tile_m, d->tile_n,
-                  d->tile_k, d->waves_m, d->waves_n, (long long)d->M, (long long)d->N, (long long)d->K);
+      return fail(FRISK_ERR_TILE, "no compiled kernel with tile %dx%dx%d waves %dx%d atom %d divides M=%lld N=%lld K=%lld", d->tile_m, d->tile_n,
+                  d->tile_k, d->waves_m, d->waves_n, d->atom, (long long)d->M, (long long)d->N, (long long)d->K);
     return fail(FRISK_ERR_SHAPE, "M=%lld N=%lld K=%lld is not a multiple of any compiled tile", (long long)d->M, (long long)d->N, (long long)d->K);
   }
   const KernelEntry* k = ks[best];

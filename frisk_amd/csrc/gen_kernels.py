@@ -51,7 +51,7 @@ def square(bk, atom16=False):
 VARIANTS = {
     "f16": ("FRISK_F16", "F16", square(64, atom16=True)),
     "bf16": ("FRISK_BF16", "BF16", square(64, atom16=True)),
-    "i8": ("FRISK_I8", "I8", square(128)),
+    "i8": ("FRISK_I8", "I8", square(128, atom16=True)),
     "e4m3": ("FRISK_E4M3", "E4M3", square(128)),
     # fp32: 128x128 for large problems; 64x64 (one atom per wave) fills the chip at 1024^3, K tiles of 64 measured 5 % faster than 32;
     # the same tile with K tiles of 128 shared by two sets of four waves (8 waves, two per SIMD) another 9 % at 1024^3 (21.6 against

@@ -321,7 +321,7 @@ int frisk_hwcheck_mfma_atom(int id, const float* A, const float* B, float* D, vo
 }
 
 // One K tile through the product's LDS layout, fragment reader and MFMA wrapper.  dtype: frisk_dtype of A and B; atom 32 or
-// 16 (16 only for F16 / BF16).  The tile is 256 x 256 x (64 | 128 for 8-bit), 128 x 128 x 32 for F32.  A and B are the
+// 16 (16 only for F16 / BF16 / I8).  The tile is 256 x 256 x (64 | 128 for 8-bit), 128 x 128 x 32 for F32.  A and B are the
 // stored tiles, dense: A [BM][BK] (transA: [BK][BM]), B [BK][BN] (transB: [BN][BK]).  D: BM x BN raw 32-bit accumulators.
 // Returns a hipError_t, or -1 for a combination that is not compiled.
 int frisk_hwcheck_fragment_path(int dtype, int atom, int transA, int transB, const void* A, const void* B, void* D, void* stream) {
@@ -331,6 +331,7 @@ int frisk_hwcheck_fragment_path(int dtype, int atom, int transA, int transB, con
   if (dtype == FRISK_BF16 && atom == 32) return (int)PathCfg<FRISK_BF16, 32, 256, 64>::launch(transA, transB, A, B, D, s);
   if (dtype == FRISK_BF16 && atom == 16) return (int)PathCfg<FRISK_BF16, 16, 256, 64>::launch(transA, transB, A, B, D, s);
   if (dtype == FRISK_I8 && atom == 32) return (int)PathCfg<FRISK_I8, 32, 256, 128>::launch(transA, transB, A, B, D, s);
+  if (dtype == FRISK_I8 && atom == 16) return (int)PathCfg<FRISK_I8, 16, 256, 128>::launch(transA, transB, A, B, D, s);
   if (dtype == FRISK_E4M3 && atom == 32) return (int)PathCfg<FRISK_E4M3, 32, 256, 128>::launch(transA, transB, A, B, D, s);
   if (dtype == FRISK_F32 && atom == 32) return (int)PathCfg<FRISK_F32, 32, 128, 32>::launch(transA, transB, A, B, D, s);
   return -1;

@@ -228,6 +228,9 @@ FRISK_HD Swizzle default_swizzle(bool kcontig, int es, int rowb, int at = 32) {
     if (at == 16 && units >= 4) return Swizzle{0, 3, 2, 3, 1, 1};
     return Swizzle{0, units >= 4 ? 3 : (units >= 2 ? 1 : 0), 2};
   }
+  // 8-bit, 16-row atoms: a half wave holds two K groups (K rows 16 apart), 16 bytes wide each; K-row bit 4 picks the 16-byte half
+  // of the 32-byte unit that rows r .. r+7 choose
+  if (at == 16 && rowb >= 256) return Swizzle{0, 7, 1, 4, 1, 0};
   if (rowb >= 256) return Swizzle{0, 7, 1};
   return Swizzle{1, 3, 1};
 }

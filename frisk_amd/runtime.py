@@ -30,7 +30,7 @@ class GemmDesc(ctypes.Structure):
                 ("transA", ctypes.c_uint8), ("transB", ctypes.c_uint8), ("clear_accum", ctypes.c_uint8),
                 ("split_k", ctypes.c_uint8), ("epilogue", ctypes.c_int32), ("policy", ctypes.c_int32),
                 ("tile_m", ctypes.c_int32), ("tile_n", ctypes.c_int32), ("tile_k", ctypes.c_int32),
-                ("waves_m", ctypes.c_int32), ("waves_n", ctypes.c_int32), ("stages", ctypes.c_int32)]
+                ("waves_m", ctypes.c_int32), ("waves_n", ctypes.c_int32), ("stages", ctypes.c_int32), ("atom", ctypes.c_int32)]
 
 
 class LdsLayout(ctypes.Structure):
@@ -124,7 +124,7 @@ def _check(status):
 
 
 def make_desc(dtype_ab, M, N, K, dtype_out=None, transA=False, transB=False, lda=None, ldb=None, ldc=None,
-              clear_accum=True, epilogue=EPI_NONE, policy=POLICY_SQUARE, tile=(0, 0, 0), waves=(0, 0), stages=0, split_k=0):
+              clear_accum=True, epilogue=EPI_NONE, policy=POLICY_SQUARE, tile=(0, 0, 0), waves=(0, 0), stages=0, split_k=0, atom=0):
     d = GemmDesc()
     d.abi_version = ABI_VERSION
     d.dtype_ab = dtype_ab
@@ -139,6 +139,7 @@ def make_desc(dtype_ab, M, N, K, dtype_out=None, transA=False, transB=False, lda
     d.tile_m, d.tile_n, d.tile_k = tile
     d.waves_m, d.waves_n = waves
     d.stages = stages
+    d.atom = atom
     d.split_k = split_k
     return d
 

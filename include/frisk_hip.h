@@ -90,6 +90,8 @@ typedef struct frisk_gemm_desc {
   int32_t tile_m, tile_n, tile_k; /* block tile = the M,N,K attrs of the tile-level frisk.gemm */
   int32_t waves_m, waves_n;       /* wave grid inside the work-group */
   int32_t stages;                 /* LDS stages of the global->LDS pipeline (of B when A and B differ), 0 = planner's choice */
+  int32_t atom;                   /* rows of the MFMA atom: 32 (32x32xK), 16 (16x16x2K), 0 = planner's choice.  Occupies what was
+                                     tail padding of the structure: its size is unchanged and zero-initialised callers keep working */
 } frisk_gemm_desc;
 
 /* XOR swizzle of an LDS tile: 16-byte chunk index c of row r is stored at

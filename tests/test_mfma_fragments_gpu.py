@@ -50,7 +50,7 @@ def test_single_mfma_atom_against_host_product(hw, atom_id):
     assert np.array_equal(dD.cpu().numpy().astype(np.float64), want), name
 
 
-PATHS = [(O.F16, 32), (O.F16, 16), (O.BF16, 32), (O.BF16, 16), (O.I8, 32), (O.E4M3, 32), (O.F32, 32)]
+PATHS = [(O.F16, 32), (O.F16, 16), (O.BF16, 32), (O.BF16, 16), (O.I8, 32), (O.I8, 16), (O.E4M3, 32), (O.F32, 32)]
 
 
 @pytest.mark.parametrize("dtype,atom", PATHS)

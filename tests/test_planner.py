@@ -52,9 +52,10 @@ def test_plans_of_the_benchmark_configurations():
         assert p.grid_x == N // tile[1] and p.grid_y == M // tile[0]
         assert p.grid_x * p.grid_y >= 256 and p.xcd_remap == 1
         assert p.threads == 64 * p.waves_m * p.waves_n * p.waves_k and p.lds_bytes <= 160 * 1024
-        # the 16-bit 256x256 default is built from 16x16x32 atoms (the part holds a higher clock on them), the rest from 32x32
-        atom = 16 if dt in (R.F16, R.BF16) else 32
-        assert (p.mfma_m, p.mfma_n) == (atom, atom) and p.mfma_k == {R.F32: 2, R.F16: 32, R.BF16: 32, R.I8: 32, R.E4M3: 64}[dt]
+        # the 16-bit and int8 256x256 defaults are built from 16-row atoms of twice the K depth (the part holds a higher clock on
+        # them), the rest from 32x32
+        atom = 16 if dt in (R.F16, R.BF16, R.I8) else 32
+        assert (p.mfma_m, p.mfma_n) == (atom, atom) and p.mfma_k == {R.F32: 2, R.F16: 32, R.BF16: 32, R.I8: 64, R.E4M3: 64}[dt]
         assert p.flops == 2.0 * M * N * K
         assert p.lds_a.k_contiguous == (0 if tA else 1) and p.lds_b.k_contiguous == (1 if tB else 0)
         assert p.workspace_bytes == 0 and p.kernel_id >= 0
@@ -77,6 +78,7 @@ def test_fp16_tile_layouts_are_conflict_free_in_the_model():
 
 SHAPES = [  # rows, row_bytes, k_contiguous, elem_bytes, frag_bytes, tile_mn, tile_k[, atom]  (every operand tile shape that is compiled)
     (256, 128, 1, 2, 16, 256, 64, 16), (64, 512, 0, 2, 16, 256, 64, 16), (256, 128, 1, 2, 16, 256, 64), (64, 512, 0, 2, 16, 256, 64), (128, 128, 1, 2, 16, 128, 64), (64, 256, 0, 2, 16, 128, 64),
+    (256, 128, 1, 1, 16, 256, 128, 16), (128, 256, 0, 1, 16, 256, 128, 16),
     (256, 128, 1, 1, 16, 256, 128), (128, 256, 0, 1, 16, 256, 128), (128, 128, 1, 1, 16, 128, 128), (128, 128, 0, 1, 16, 128, 128),
     (256, 128, 1, 1, 32, 256, 128), (128, 256, 0, 1, 32, 256, 128), (128, 128, 1, 1, 32, 128, 128), (128, 128, 0, 1, 32, 128, 128),
     (128, 128, 1, 4, 4, 128, 32), (32, 512, 0, 4, 4, 128, 32), (64, 128, 1, 4, 4, 64, 32), (32, 256, 0, 4, 4, 64, 32),
@@ -94,9 +96,8 @@ def test_compiled_swizzle_is_what_the_cost_model_search_picks(shape):
     for tA in (0, 1):
         for tB in (0, 1):
             for M in (mn * 16,):
-                # the 16-bit 256x256 tiles exist with both atoms: the ring of 2 + 2 tiles is the variant of 32x32 atoms
-                d = R.make_desc(dt, M, M, bk * 8, dtype_out=R.ACC_OF[dt] if dt != R.F16 else R.F16, transA=tA, transB=tB, tile=(mn, mn, bk),
-                                stages=2 if (dt == R.F16 and mn == 256 and atom == 32) else 0)
+                # the 16-bit and int8 256x256 tiles exist with both atoms: the descriptor names the one wanted
+                d = R.make_desc(dt, M, M, bk * 8, dtype_out=R.ACC_OF[dt] if dt != R.F16 else R.F16, transA=tA, transB=tB, tile=(mn, mn, bk), atom=atom)
                 p = R.plan(d)
                 assert p.mfma_m == atom
                 for L in (p.lds_a, p.lds_b):
@@ -246,7 +247,7 @@ def test_planner_ranks_variants_by_estimated_time():
     assert pick(R.E4M3, 32, 32768, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s2_splitk"
     assert pick(R.F16, 1024, 1024, 1024) == "f16_nn_32x128x64_w1x4_s3_splitk"
     # 576 tiles = 2 rounds + 64: the variant with the split-K store path, its last 64 tiles as 4 work-groups each
-    assert pick(R.I8, 6144, 6144, 6144) == "i8_nn_256x256x128_w2x2_s2x3_splitk"
+    assert pick(R.I8, 6144, 6144, 6144) == "i8_nn_256x256x128_w2x2_s2x3_a16_splitk"
     p = R.plan(R.make_desc(R.I8, 6144, 6144, 6144, dtype_out=R.I32))
     assert (p.tail_tiles, p.tail_split, p.split_k) == (64, 4, 1) and p.workspace_bytes == 4 * 64 * 256 * 256 * 4
     # whole rounds, more than half a round left over, or a descriptor that forbids splitting: no tail
