@@ -1,6 +1,6 @@
 // C ABI of libfrisk_hip.so: descriptor validation, the planner (tile / wave
 // grid / LDS layout choice) and kernel dispatch.  Host code only.
-#include <hip/hip_runtime_api.h>
+#include <hip/hip_runtime.h>
 
 #include <atomic>
 #include <cmath>
@@ -16,9 +16,32 @@
 #include "tile_ops.h"
 #include "attention.h"
 
+// Scratch memory of frisk_hip_gemm_static_ws: the split-K / tail-split partial sums of callers that cannot allocate.
+// Every GPU the library runs on holds its own copy of this array, at its own address, until the process ends.  In host
+// code the name below is only a handle for hipGetSymbolAddress; kernels and copies get the device address it returns.
+static __device__ __align__(256) unsigned char scratch[FRISK_HIP_STATIC_WS_BYTES];
+
 namespace frisk {
 
 static thread_local std::string g_last_error;
+
+// device address of `scratch` on each device, resolved once per device with that device current
+static constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+static hipError_t scratch_of_current_device(void** out) {
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)); e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing threads resolve the same address
+  }
+  *out = p;
+  return hipSuccess;
+}
 
 static int fail(int status, const char* fmt, ...) {
   char buf[512];
@@ -359,6 +382,8 @@ int frisk_hip_init(void) {
   for (const KernelEntry* k : kernels())
     if (hipError_t e = k->prepare(); e != hipSuccess) return fail(FRISK_ERR_DEVICE, "preparing %s failed: %s", k->name, hipGetErrorString(e));
   if (hipError_t e = prepare_attention(); e != hipSuccess) return fail(FRISK_ERR_DEVICE, "preparing the attention kernels failed: %s", hipGetErrorString(e));
+  void* ws = nullptr;
+  if (hipError_t e = scratch_of_current_device(&ws); e != hipSuccess) return fail(FRISK_ERR_DEVICE, "resolving the static workspace failed: %s", hipGetErrorString(e));
   return FRISK_OK;
 }
 
@@ -424,6 +449,25 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
     if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "launch of the tail reduction failed: %s", hipGetErrorString(e));
   }
   return FRISK_OK;
+}
+
+size_t frisk_hip_static_workspace_bytes(void) { return (size_t)FRISK_HIP_STATIC_WS_BYTES; }
+
+int frisk_hip_gemm_static_ws(const frisk_gemm_desc* desc, const void* A, const void* B, void* C, const float* scaleA, const float* scaleB,
+                             void* stream) {
+  frisk_gemm_plan plan;
+  int st = make_plan(desc, &plan, false);
+  if (st != FRISK_OK) return st;
+  if (plan.workspace_bytes > (size_t)FRISK_HIP_STATIC_WS_BYTES)
+    return fail(FRISK_ERR_WORKSPACE, "this problem's partial sums need %zu bytes, the static workspace holds %zu: pass split_k = 1 or use frisk_hip_gemm with a workspace",
+                plan.workspace_bytes, (size_t)FRISK_HIP_STATIC_WS_BYTES);
+  void* ws = nullptr;
+  if (plan.workspace_bytes > 0) {
+    if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
+    if (hipError_t e = scratch_of_current_device(&ws); e != hipSuccess) return fail(FRISK_ERR_DEVICE, "resolving the static workspace failed: %s", hipGetErrorString(e));
+  }
+  // every slice of a split stores its whole share of the partial sums before the reduction reads it: nothing to clear
+  return frisk_hip_gemm(desc, A, B, C, scaleA, scaleB, ws, ws ? (size_t)FRISK_HIP_STATIC_WS_BYTES : 0, stream);
 }
 
 float frisk_hip_lds_access_cycles(int instr, const int32_t* lane_byte_addr) {

@@ -71,7 +71,8 @@ _lib = None
 EXPORTS = ["frisk_hip_init", "frisk_hip_abi_version", "frisk_hip_last_error", "frisk_hip_plan", "frisk_hip_workspace_bytes",
            "frisk_hip_gemm", "frisk_hip_lds_access_cycles", "frisk_hip_lds_search", "frisk_hip_lds_search_atom", "frisk_hip_lds_offset", "frisk_hip_wave_partition",
            "frisk_hip_kernel_count", "frisk_hip_kernel_name", "frisk_hip_fill", "frisk_hip_copy", "frisk_hip_reduce",
-           "frisk_hip_reduce_workspace_bytes", "frisk_hip_attention", "frisk_hip_softmax", "frisk_hip_softmax_workspace_bytes"]
+           "frisk_hip_reduce_workspace_bytes", "frisk_hip_attention", "frisk_hip_softmax", "frisk_hip_softmax_workspace_bytes",
+           "frisk_hip_gemm_static_ws", "frisk_hip_static_workspace_bytes"]
 
 
 def lib():
@@ -89,6 +90,9 @@ def lib():
     L.frisk_hip_workspace_bytes.argtypes = [ctypes.POINTER(GemmDesc)]
     L.frisk_hip_gemm.argtypes = [ctypes.POINTER(GemmDesc), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                  ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    L.frisk_hip_gemm_static_ws.argtypes = [ctypes.POINTER(GemmDesc), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                           ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    L.frisk_hip_static_workspace_bytes.restype = ctypes.c_size_t
     L.frisk_hip_lds_access_cycles.restype = ctypes.c_float
     L.frisk_hip_lds_access_cycles.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_int32)]
     L.frisk_hip_lds_search.argtypes = [ctypes.POINTER(LdsLayout), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -164,6 +168,17 @@ def gemm(desc, A_ptr, B_ptr, C_ptr, scaleA_ptr=None, scaleB_ptr=None, workspace_
     """Asynchronous launch on `stream` (a raw hipStream_t value or None). Pointers are raw device addresses."""
     _check(lib().frisk_hip_gemm(ctypes.byref(desc), A_ptr, B_ptr, C_ptr, scaleA_ptr, scaleB_ptr, workspace_ptr,
                                 workspace_bytes, stream))
+
+
+def static_workspace_bytes():
+    """size of the library's own scratch array, the most a plan run by gemm_static_ws may need"""
+    return int(lib().frisk_hip_static_workspace_bytes())
+
+
+def gemm_static_ws(desc, A_ptr, B_ptr, C_ptr, scaleA_ptr=None, scaleB_ptr=None, stream=None):
+    """`gemm` for callers that cannot allocate: split-K / tail-split partial sums go to the library's own scratch array.
+    Calls that may overlap on one GPU race on that array."""
+    _check(lib().frisk_hip_gemm_static_ws(ctypes.byref(desc), A_ptr, B_ptr, C_ptr, scaleA_ptr, scaleB_ptr, stream))
 
 
 REDUCE_KINDS = {"add": 0, "sum": 0, "mul": 1, "min": 2, "max": 3}

@@ -157,6 +157,19 @@ size_t frisk_hip_workspace_bytes(const frisk_gemm_desc* desc);
 int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, void* C, const float* scaleA,
                    const float* scaleB, void* workspace, size_t workspace_bytes, void* stream);
 
+/* frisk_hip_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc) and therefore have no workspace to pass.  No counterpart in the reference.  The
+ * partial sums of a split-K or tail-split plan go to a fixed array of FRISK_HIP_STATIC_WS_BYTES that lives in the
+ * library's device image (one copy per GPU, held until the process ends); neither this call nor anything it calls
+ * allocates or frees.  Same planner, kernels and results as frisk_hip_gemm with a large enough workspace.  A
+ * descriptor whose plan needs more than the array holds (a large explicit split_k) is refused with
+ * FRISK_ERR_WORKSPACE.  All calls on one GPU share the array: calls that may overlap on that GPU (different streams,
+ * different host threads) race on it and must be serialised by the caller; calls on one stream are ordered. */
+#define FRISK_HIP_STATIC_WS_BYTES (32u << 20)
+size_t frisk_hip_static_workspace_bytes(void);
+int frisk_hip_gemm_static_ws(const frisk_gemm_desc* desc, const void* A, const void* B, void* C, const float* scaleA,
+                             const float* scaleB, void* stream);
+
 /* Pure host: modelled LDS cycles for one wave-wide access given the 64 byte
  * addresses the lanes present.  instr: 0 ds_read_b128, 1 ds_read_b64 /
  * ds_read_b64_tr_b16 / ds_read_b64_tr_b8, 3 ds_read_b32.  Replaces the bank
