@@ -1,25 +1,60 @@
-"""Convenience layer over the builder: context + builder + module in one object.
+"""Session helper of the `frisk` package: one object that owns a context, a builder and a module.
 
-Same surface as the reference's python/frisk/common/utils.py:18-163
-(create_context, create_session, FriskHelper with memref_type, new_kernel,
-alloc_buffer, create_gemm, ensure_insertion_block, dump), plus `tiled_gemm`,
-which writes the whole tiled GEMM program of the reference's design sketch
-(tmp/ir.mlir:1-17) in one call.
+The public names and keyword arguments are those the reference's scripts use
+(test/python/helper_test.py:4-24: `create_session`, `.builder`, `.module`, `memref_type(shape, type, space=)`,
+`new_kernel(name, types) -> (kernel, entry block)`, `create_gemm(A, B, C)`, `alloc_buffer(shape, "fp16", space=, alignment=)`;
+`create_context`, `ensure_insertion_block` and `dump` complete the surface of python/frisk/common/utils.py).  Everything
+behind those names is this build's own: element types live in one table, and `tiled_gemm` writes the whole tiled GEMM
+program of the reference's design sketch (tmp/ir.mlir:1-17) that `frisk.runtime` lowers to the gfx950 kernels.
 """
-from __future__ import annotations
-
-from dataclasses import dataclass
-from typing import Sequence, Tuple, Union
-
 from ..frisk_ffi import ir
-
-DTypeLike = Union[str, ir.type]
-ShapeLike = Sequence[int]
 
 __all__ = ["create_context", "create_session", "FriskHelper"]
 
 
-def create_context(*, load_dialects: bool = True, disable_multithreading: bool = True) -> ir.context:
+class _Element:
+    """one row of the element-type table: how the builder makes the type, how a type object is recognised, and the type a
+    GEMM on such operands accumulates in"""
+
+    def __init__(self, name, getter, probe=None, accumulator=None):
+        self.name, self.getter, self.probe, self.accumulator = name, getter, probe, accumulator
+
+    def make(self, builder):
+        return getattr(builder, self.getter)()
+
+    def matches(self, ty):
+        return self.probe is not None and getattr(ty, self.probe)()
+
+
+_ELEMENTS = [
+    _Element("fp16", "get_f16_ty", "is_f16", "fp32"),
+    _Element("bf16", "get_bf16_ty", "is_bf16", "fp32"),
+    _Element("fp32", "get_f32_ty", "is_f32", "fp32"),
+    _Element("fp64", "get_f64_ty", "is_f64"),
+    _Element("e4m3fn", "get_f8e4m3fn_ty", None, "fp32"),
+    _Element("int8", "get_int8_ty", None, "int32"),
+    _Element("int32", "get_int32_ty"),
+    _Element("int64", "get_int64_ty"),
+]
+_BY_NAME = {e.name: e for e in _ELEMENTS}
+
+
+def _element_named(name):
+    try:
+        return _BY_NAME[str(name).strip().lower()]
+    except KeyError:
+        raise ValueError("element type %r is not one of %s" % (name, ", ".join(sorted(_BY_NAME)))) from None
+
+
+def _name_of_type(ty):
+    for e in _ELEMENTS:
+        if e.matches(ty):
+            return e.name
+    raise ValueError("alloc_buffer takes the element type as a string or as an f16 / bf16 / f32 / f64 type object, got %s" % (ty,))
+
+
+def create_context(*, load_dialects=True, disable_multithreading=True):
+    """a fresh IR context, single-threaded and with the Frisk dialect registered unless told otherwise"""
     ctx = ir.context()
     if disable_multithreading:
         ctx.disable_multithreading()
@@ -28,135 +63,105 @@ def create_context(*, load_dialects: bool = True, disable_multithreading: bool =
     return ctx
 
 
-def create_session(*, load_dialects: bool = True, disable_multithreading: bool = True) -> "FriskHelper":
+def create_session(*, load_dialects=True, disable_multithreading=True):
     return FriskHelper.create(load_dialects=load_dialects, disable_multithreading=disable_multithreading)
 
 
-_DTYPES = {"fp16": "get_f16_ty", "bf16": "get_bf16_ty", "fp32": "get_f32_ty", "fp64": "get_f64_ty", "int64": "get_int64_ty",
-           "int32": "get_int32_ty", "int8": "get_int8_ty", "e4m3fn": "get_f8e4m3fn_ty"}
-_ACCUMULATOR = {"fp16": "fp32", "bf16": "fp32", "fp32": "fp32", "e4m3fn": "fp32", "int8": "int32"}
-
-
-@dataclass
 class FriskHelper:
-    context: ir.context
-    builder: ir.builder
-    module: ir.module
+    """context + builder + module.  The module keeps a reference to the context (`module.context`), which owns every IR
+    object, so handing the module around is enough to keep the IR alive."""
+
+    def __init__(self, context, builder, module):
+        self.context, self.builder, self.module = context, builder, module
 
     @classmethod
-    def create(cls, *, load_dialects: bool = True, disable_multithreading: bool = True) -> "FriskHelper":
-        ctx = create_context(load_dialects=load_dialects, disable_multithreading=disable_multithreading)
-        builder = ir.builder(ctx)
+    def create(cls, *, load_dialects=True, disable_multithreading=True):
+        context = create_context(load_dialects=load_dialects, disable_multithreading=disable_multithreading)
+        builder = ir.builder(context)
         module = builder.create_module()
-        module.context = ctx  # the context owns every IR object: keep it alive with the module
-        return cls(ctx, builder, module)
+        module.context = context
+        return cls(context, builder, module)
 
-    # ------------------------------------------------------------------ types
-    def memref_type(self, shape: ShapeLike, dtype: DTypeLike = "fp16", *, space: ir.MemorySpace = ir.MemorySpace.GLOBAL,
-                    layout: ir.AffineMap | None = None) -> ir.memref_buffer:
-        element_type = self._as_type(dtype)
-        dims = [int(dim) for dim in shape]
-        affine_map = layout if layout is not None else ir.AffineMap()
-        return self.builder.get_memref_ty(element_type, dims, affine_map, space)
+    def __repr__(self):
+        return "FriskHelper(%d top-level ops)" % str(self.module).count("frisk.kernel")
 
-    # ------------------------------------------------------------------ ops
-    def new_kernel(self, name: str, arg_types: Sequence[ir.type]) -> Tuple[ir.KernelOp, ir.block]:
-        kernel_type = self.builder.get_kernel_ty(list(arg_types))
-        kernel = self.builder.create_kernel_op(self.module, name, kernel_type)
+    # ---------------------------------------------------------------- types
+    def element_type(self, dtype):
+        """`dtype` as a type object: a name from the element table or a type that is passed through"""
+        return dtype if isinstance(dtype, ir.type) else _element_named(dtype).make(self.builder)
+
+    def memref_type(self, shape, dtype="fp16", *, space=ir.MemorySpace.GLOBAL, layout=None):
+        return self.builder.get_memref_ty(self.element_type(dtype), [int(extent) for extent in shape],
+                                          ir.AffineMap() if layout is None else layout, space)
+
+    # ---------------------------------------------------------------- ops
+    def new_kernel(self, name, arg_types):
+        """appends `frisk.kernel @name(arg_types...)` to the module and leaves the builder at the start of its body"""
+        kernel = self.builder.create_kernel_op(self.module, name, self.builder.get_kernel_ty(list(arg_types)))
         self.module.push_back(kernel)
         entry = kernel.add_entry_block()
         self.builder.set_insertion_point_to_start(entry)
         return kernel, entry
 
-    def alloc_buffer(self, shape: ShapeLike, dtype: DTypeLike = "fp16", *, space: ir.MemorySpace = ir.MemorySpace.LOCAL,
-                     alignment: int = 0) -> ir.value:
-        dtype_str = self._as_dtype_str(dtype)
-        op = self.builder.create_alloc_buffer_op(list(shape), dtype_str, space, alignment)
-        return ir.OpState.get_result(op, 0)
+    def alloc_buffer(self, shape, dtype="fp16", *, space=ir.MemorySpace.LOCAL, alignment=0):
+        """the value of a `frisk.alloc_buffer`"""
+        name = dtype if isinstance(dtype, str) else _name_of_type(dtype)
+        return ir.OpState.get_result(self.builder.create_alloc_buffer_op([int(extent) for extent in shape], name, space, alignment), 0)
 
-    def create_gemm(self, A: ir.value, B: ir.value, C: ir.value, *, trans_a: bool = False, trans_b: bool = False,
-                    clear_accum: bool = False) -> ir.GemmOp:
+    def create_gemm(self, A, B, C, *, trans_a=False, trans_b=False, clear_accum=False):
         return self.builder.create_gemm_op(A, B, C, trans_a, trans_b, clear_accum)
 
-    def tiled_gemm(self, name: str, M: int, N: int, K: int, dtype: str = "fp16", *, out_dtype: str | None = None,
-                   tile: Tuple[int, int, int] = (256, 256, 64), threads: int = 512, trans_a: bool = False,
-                   trans_b: bool = False) -> ir.KernelOp:
+    def tiled_gemm(self, name, M, N, K, dtype="fp16", *, out_dtype=None, tile=(256, 256, 64), threads=512, trans_a=False, trans_b=False):
         """kernel(A, B, C) { parallel (by, bx) { sA, sB, acc; fill acc 0; for k { copy A, copy B, gemm }; copy acc -> C } }"""
         b = self.builder
         bm, bn, bk = tile
         if M % bm or N % bn or K % bk:
             raise ValueError("tile %r does not divide the problem %r" % (tile, (M, N, K)))
-        acc_dtype = _ACCUMULATOR[dtype]
-        out_dtype = out_dtype or dtype
+        acc_dtype = _element_named(dtype).accumulator
+        if acc_dtype is None:
+            raise ValueError("no GEMM on operands of type %r" % (dtype,))
         a_shape = (K, M) if trans_a else (M, K)
         b_shape = (N, K) if trans_b else (K, N)
-        tys = [self.memref_type(a_shape, dtype), self.memref_type(b_shape, dtype), self.memref_type((M, N), out_dtype)]
-        kernel, entry = self.new_kernel(name, tys)
+        kernel, entry = self.new_kernel(name, [self.memref_type(a_shape, dtype), self.memref_type(b_shape, dtype),
+                                               self.memref_type((M, N), out_dtype or dtype)])
         gA, gB, gC = (entry.get_argument(i) for i in range(3))
-        par = b.create_parallel_op([M // bm, N // bn], threads)
-        body = par.add_entry_block()
+        body = b.create_parallel_op([M // bm, N // bn], threads).add_entry_block()
         b.set_insertion_point_to_start(body)
         by, bx = body.get_argument(0), body.get_argument(1)
-        sa_shape = (bk, bm) if trans_a else (bm, bk)
-        sb_shape = (bn, bk) if trans_b else (bk, bn)
+        sa_shape = [bk, bm] if trans_a else [bm, bk]
+        sb_shape = [bn, bk] if trans_b else [bk, bn]
         sA = self.alloc_buffer(sa_shape, dtype, space=ir.MemorySpace.SHARED, alignment=1024)
         sB = self.alloc_buffer(sb_shape, dtype, space=ir.MemorySpace.SHARED, alignment=1024)
         acc = self.alloc_buffer((bm, bn), acc_dtype, space=ir.MemorySpace.LOCAL)
         b.create_fill_op(acc, 0.0, acc_dtype)
         d0, d1 = b.get_affine_dim_expr(0), b.get_affine_dim_expr(1)
-        ident = ir.AffineMap.get_multi_dim_identity_map(2)
 
-        def tile_map(e0, e1):
-            return ir.AffineMap.get(2, 0, [e0, e1])
+        def scaled(s0, s1):  # (i, j) -> (i * s0, j * s1): tile indices to element offsets
+            return ir.AffineMap.get(2, 0, [d0 * s0, d1 * s1])
+
+        def origin(bb):  # () -> (0, 0)
+            return ir.AffineMap.get(0, 0, [bb.get_affine_constant_expr(0)] * 2)
 
         def k_body(bb, k):
-            a_map = tile_map(d0 * bk, d1 * bm) if trans_a else tile_map(d0 * bm, d1 * bk)
-            b_map = tile_map(d0 * bn, d1 * bk) if trans_b else tile_map(d0 * bk, d1 * bn)
-            bb.create_copy_op(gA, sA, [k, by] if trans_a else [by, k], [], a_map, ir.AffineMap.get(0, 0, [bb.get_affine_constant_expr(0)] * 2),
-                              list(sa_shape), list(sa_shape))
-            bb.create_copy_op(gB, sB, [bx, k] if trans_b else [k, bx], [], b_map, ir.AffineMap.get(0, 0, [bb.get_affine_constant_expr(0)] * 2),
-                              list(sb_shape), list(sb_shape))
+            bb.create_copy_op(gA, sA, [k, by] if trans_a else [by, k], [], scaled(*sa_shape), origin(bb), sa_shape, sa_shape)
+            bb.create_copy_op(gB, sB, [bx, k] if trans_b else [k, bx], [], scaled(*sb_shape), origin(bb), sb_shape, sb_shape)
             bb.create_gemm_op(sA, sB, acc, trans_a, trans_b, False)
 
         b.create_for_op(0, K // bk, 1, k_body)
-        b.create_copy_op(acc, gC, [], [by, bx], ir.AffineMap.get(0, 0, [b.get_affine_constant_expr(0)] * 2), tile_map(d0 * bm, d1 * bn),
-                         [bm, bn], [bm, bn])
-        del ident
+        b.create_copy_op(acc, gC, [], [by, bx], origin(b), scaled(bm, bn), [bm, bn], [bm, bn])
         return kernel
 
-    # ------------------------------------------------------------------ utilities
-    def ensure_insertion_block(self) -> ir.block:
+    # ---------------------------------------------------------------- utilities
+    def ensure_insertion_block(self):
+        """the block the builder inserts into; when it has none yet, a new block at the end of the module's body"""
         block = self.builder.get_insertion_block()
-        if block is not None:
-            return block
-        new_block = self.builder.new_block()
-        self.module.get_region(0).push_back(new_block)
-        self.builder.set_insertion_point_to_start(new_block)
-        return new_block
+        if block is None:
+            block = self.builder.new_block()
+            self.module.get_region(0).push_back(block)
+            self.builder.set_insertion_point_to_start(block)
+        return block
 
-    def dump(self, msg: str | None = None) -> None:
+    def dump(self, msg=None):
         if msg:
             print(msg)
         print(self.module)
-
-    # ------------------------------------------------------------------ internal
-    def _as_type(self, dtype: DTypeLike) -> ir.type:
-        if isinstance(dtype, ir.type):
-            return dtype
-        key = dtype.lower()
-        if key in _DTYPES:
-            return getattr(self.builder, _DTYPES[key])()
-        raise ValueError(f"Unsupported dtype '{dtype}'.")
-
-    def _as_dtype_str(self, dtype: DTypeLike) -> str:
-        if isinstance(dtype, str):
-            return dtype
-        if dtype.is_f16():
-            return "fp16"
-        if dtype.is_bf16():
-            return "bf16"
-        if dtype.is_f32():
-            return "fp32"
-        if dtype.is_f64():
-            return "fp64"
-        raise ValueError("Unsupported type for allocation helper.")
