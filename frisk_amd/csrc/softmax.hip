@@ -25,6 +25,8 @@ template <> struct SElem<FRISK_BF16> { typedef __bf16 T; static __device__ float
 struct MaxSum {
   float m, l;
   __device__ void add(float v) {
+    // a masked element (-inf) adds nothing; without the test an all-masked prefix would compute 2^(-inf - -inf)
+    if (v == -INFINITY) return;
     if (v > m) { l = l * __builtin_amdgcn_exp2f(m - v) + 1.f; m = v; }
     else l += __builtin_amdgcn_exp2f(v - m);
   }

@@ -564,15 +564,28 @@ void init_ffi_ir(py::module_&& m) {
         };
         const TypeImpl *a = require_memref(A, "A"), *bt = require_memref(B, "B"), *c = require_memref(C, "C");
         if (a->shape.size() != 2 || bt->shape.size() != 2 || c->shape.size() != 2) throw std::invalid_argument("create_gemm_op expects rank-2 memrefs");
-        // Without transpose flags: M, K from A and N from B as stored (ffi/ir.cpp:346-355).  The reference
-        // applies the same reading when a flag is set, which no transposed operand can satisfy; here a set
-        // flag means the operand is stored transposed ([K][M] for A, [N][K] for B).
-        int64_t mm = require_static(a->shape[transA ? 1 : 0], "M dimension of A"), k = require_static(a->shape[transA ? 0 : 1], "K dimension of A");
-        int64_t kb = require_static(bt->shape[transB ? 1 : 0], "K dimension of B");
-        if (k != kb) throw std::invalid_argument("create_gemm_op expects A and B inner dimensions to match");
-        int64_t n = require_static(bt->shape[transB ? 0 : 1], "N dimension of B");
-        int64_t cm = require_static(c->shape[0], "M dimension of C"), cn = require_static(c->shape[1], "N dimension of C");
-        if (mm != cm || n != cn) throw std::invalid_argument("create_gemm_op expects C shape to match A/B product");
+        // The reference reads A as [M][K] and B as [K][N] whatever the flags say (ffi/ir.cpp:346-355, GemmOp::verify
+        // FriskOps.cpp:1264-1283); its flags only pick the shared-memory layout (FriskOps.cpp:1359, 1376).  A path that
+        // executes the GEMM needs operands that really are stored transposed (B as [N][K]), so here a set flag first
+        // means "stored transposed" ([K][M] for A, [N][K] for B).  When the shapes do not fit that reading but fit the
+        // reference's, the reference's is taken: the flag is then a layout hint without effect on the arithmetic.
+        for (int d = 0; d < 2; ++d) {
+          require_static(a->shape[(size_t)d], d == 0 ? "M dimension of A" : "K dimension of A");
+          require_static(bt->shape[(size_t)d], d == 0 ? "K dimension of B" : "N dimension of B");
+          require_static(c->shape[(size_t)d], d == 0 ? "M dimension of C" : "N dimension of C");
+        }
+        const int64_t cm = c->shape[0], cn = c->shape[1];
+        int64_t mm = 0, n = 0, k = 0;
+        auto reading = [&](bool ta, bool tb) {
+          mm = a->shape[ta ? 1 : 0]; k = a->shape[ta ? 0 : 1];
+          n = bt->shape[tb ? 0 : 1];
+          return k == bt->shape[tb ? 1 : 0] && mm == cm && n == cn;
+        };
+        if (!reading(transA, transB) && !((transA || transB) && reading(false, false))) {
+          reading(transA, transB);
+          if (k != bt->shape[transB ? 1 : 0]) throw std::invalid_argument("create_gemm_op expects A and B inner dimensions to match");
+          throw std::invalid_argument("create_gemm_op expects C shape to match A/B product");
+        }
         Type ea(a->element), eb(bt->element), ec(c->element);
         // same element type for all three as in the reference (ffi/ir.cpp:357-359), or C in the accumulator
         // type of the inputs (f32 for floating inputs, i32 for i8), which the MFMA path needs

@@ -804,11 +804,15 @@ inline bool verify_operation(const Operation* op, Diagnostics& d) {
     if (a && b && c) {
       if (a->shape.size() != 2 || b->shape.size() != 2 || c->shape.size() != 2) fail("expects rank-2 memrefs");
       else {
-        // FriskOps.cpp:1274-1281 checks the shapes as stored; a set transpose flag swaps the operand's two extents
+        // The reference's verifier (FriskOps.cpp:1264-1283) reads A as [M][K] and B as [K][N] and ignores the transpose
+        // flags.  Here a set flag may also mean the operand is stored transposed ([K][M], [N][K]): either reading that
+        // fits the op's M, N, K is accepted.
         const bool ta = op->bool_attr("transA"), tb = op->bool_attr("transB");
-        if (a->shape[ta ? 1 : 0] != op->int_attr("M") || a->shape[ta ? 0 : 1] != op->int_attr("K")) fail("A shape does not match M x K");
-        if (b->shape[tb ? 1 : 0] != op->int_attr("K") || b->shape[tb ? 0 : 1] != op->int_attr("N")) fail("B shape does not match K x N");
-        if (c->shape[0] != op->int_attr("M") || c->shape[1] != op->int_attr("N")) fail("C shape does not match M x N");
+        const int64_t M = op->int_attr("M"), N = op->int_attr("N"), K = op->int_attr("K");
+        auto fits = [](const TypeImpl* t, bool swapped, int64_t r, int64_t cc) { return t->shape[swapped ? 1 : 0] == r && t->shape[swapped ? 0 : 1] == cc; };
+        if (!fits(a, ta, M, K) && !fits(a, false, M, K)) fail("A shape does not match M x K");
+        if (!fits(b, tb, K, N) && !fits(b, false, K, N)) fail("B shape does not match K x N");
+        if (c->shape[0] != M || c->shape[1] != N) fail("C shape does not match M x N");
       }
       if (!Type(a->element).equals(Type(b->element))) fail("A and B must have the same element type");
     }
@@ -878,6 +882,46 @@ inline int kernel_arg_index(const Operation* kernel, Value v) {
   return -1;
 }
 
+// The window origin one side of a frisk.copy addresses, as an affine function of (grid index along M, grid index along N,
+// K induction variable): origin[r] = cm[r] * by + cn[r] * bx + ck[r] * k + c0[r] for result r of the side's index map.
+// Index operands must be those three values; the map must be linear in them.
+struct CopyOrigin {
+  std::vector<int64_t> cm, cn, ck, c0;
+};
+
+inline CopyOrigin copy_origin(const Operation* cp, bool dst_side, Value by, Value bx, Value k) {
+  const AffineMap& map = cp->attr(dst_side ? "dstMap" : "srcMap")->map;
+  const int ns = cp->src_index_count, first = dst_side ? 2 + ns : 2;
+  const int count = dst_side ? (int)cp->operands.size() - 2 - ns : ns;
+  if (count != map.num_inputs()) throw std::invalid_argument("not a tiled GEMM kernel: a copy's index operands do not match its index map");
+  std::vector<int> which((size_t)count);  // 0 by, 1 bx, 2 k
+  for (int i = 0; i < count; ++i) {
+    const Value v = cp->operands[(size_t)(first + i)];
+    if (v == by) which[(size_t)i] = 0;
+    else if (v == bx) which[(size_t)i] = 1;
+    else if (k && v == k) which[(size_t)i] = 2;
+    else throw std::invalid_argument("not a tiled GEMM kernel: a copy is indexed by something other than the grid indices and the K induction variable");
+  }
+  auto at = [&](int64_t vby, int64_t vbx, int64_t vk) {
+    const int64_t val[3] = {vby, vbx, vk};
+    std::vector<int64_t> dims, syms;
+    for (int i = 0; i < count; ++i) (i < map.num_dims() ? dims : syms).push_back(val[which[(size_t)i]]);
+    std::vector<int64_t> out;
+    for (int r = 0; r < map.num_results(); ++r) out.push_back(map.impl->results[(size_t)r].eval(dims, syms));
+    return out;
+  };
+  CopyOrigin o;
+  o.c0 = at(0, 0, 0);
+  const std::vector<int64_t> m1 = at(1, 0, 0), n1 = at(0, 1, 0), k1 = at(0, 0, 1), probe = at(2, 3, 5);
+  for (size_t r = 0; r < o.c0.size(); ++r) {
+    o.cm.push_back(m1[r] - o.c0[r]);
+    o.cn.push_back(n1[r] - o.c0[r]);
+    o.ck.push_back(k1[r] - o.c0[r]);
+    if (probe[r] != o.c0[r] + 2 * o.cm[r] + 3 * o.cn[r] + 5 * o.ck[r]) throw std::invalid_argument("not a tiled GEMM kernel: a copy's index map is not linear in the grid and K indices");
+  }
+  return o;
+}
+
 inline GemmProgram match_tiled_gemm(Operation* kernel, Operation* module = nullptr) {
   auto bad = [](const std::string& m) -> GemmProgram { throw std::invalid_argument("not a tiled GEMM kernel: " + m); };
   if (!kernel || kernel->name != "frisk.kernel") return bad("expected a frisk.kernel");
@@ -904,7 +948,7 @@ inline GemmProgram match_tiled_gemm(Operation* kernel, Operation* module = nullp
   std::vector<Operation*> allocs;
   for (Operation* op : body->ops) {
     if (op->name == "frisk.alloc_buffer") allocs.push_back(op);
-    else if (op->name == "frisk.fill") fill = op;
+    else if (op->name == "frisk.fill") { if (fill) return bad("more than one frisk.fill"); if (loop) return bad("frisk.fill after the K loop"); fill = op; }
     else if (op->name == "frisk.for") { if (loop) return bad("more than one frisk.for"); loop = op; }
     else if (op->name == "frisk.copy") { if (store) return bad("more than one copy after the K loop"); if (!loop) return bad("copy before the K loop"); store = op; }
     else if (op->name != "frisk.end") return bad("unexpected '" + op->name + "' in frisk.parallel");
@@ -938,15 +982,25 @@ inline GemmProgram match_tiled_gemm(Operation* kernel, Operation* module = nullp
   for (Value v : {gA, gB, gC}) if (space_of(v) != (int)MemorySpace::Global) return bad("kernel arguments must be global memrefs");
 
   g.transA = gemm->bool_attr("transA"); g.transB = gemm->bool_attr("transB");
+  {
+    // A set flag means the operand is stored transposed; when the op's M, N, K fit only the un-transposed reading of its
+    // operand shapes (the reference's reading, where the flag is a layout hint), the operand is taken as stored.
+    const auto& ha = sA.type().impl->shape; const auto& hb = sB.type().impl->shape;
+    const int64_t gm = gemm->int_attr("M"), gn = gemm->int_attr("N"), gk = gemm->int_attr("K");
+    if (g.transA && ha.size() == 2 && ha[0] != ha[1] && ha[0] == gm && ha[1] == gk) g.transA = false;
+    if (g.transB && hb.size() == 2 && hb[0] != hb[1] && hb[0] == gk && hb[1] == gn) g.transB = false;
+  }
   g.policy = (GemmWarpPolicy)gemm->attr("policy")->i;
   // clear_accum on the gemm restarts the sum every K step; the tiled program clears once with fill 0
   if (gemm->bool_attr("clear_accum")) return bad("gemm inside the K loop must accumulate (clear_accum = false)");
-  g.clear_accum = fill && fill->operands[0] == acc && fill->attr("value")->f == 0.0;
+  // The program only ever copies the accumulator to C, so C is never read: the result is (fill value) + A.B.  Only the
+  // fill value 0 has a kernel here; without a fill the accumulator would start undefined.
+  if (!fill || !(fill->operands[0] == acc)) return bad("the accumulator must be cleared by a frisk.fill before the K loop");
+  if (fill->attr("value")->f != 0.0) return bad("the accumulator must be filled with 0 (a GEMM on top of another fill value is not lowered)");
+  g.clear_accum = true;
   g.tile_m = gemm->int_attr("M"); g.tile_n = gemm->int_attr("N"); g.tile_k = gemm->int_attr("K");
   const auto& sa = sA.type().impl->shape; const auto& sb = sB.type().impl->shape; const auto& sc = acc.type().impl->shape;
-  // with a transposed operand the staged tile is stored transposed, like the global operand
-  if (g.transA) { if (sa[0] != g.tile_k && sa[1] != g.tile_k) return bad("shared A tile does not match the gemm K"); }
-  (void)sb; (void)sc;
+  if (sa.size() != 2 || sb.size() != 2) return bad("the shared tiles of A and B must be rank-2");
   const auto& ga = gA.type().impl->shape; const auto& gb = gB.type().impl->shape; const auto& gc = gC.type().impl->shape;
   if (ga.size() != 2 || gb.size() != 2 || gc.size() != 2) return bad("A, B and C must be rank-2");
   g.M = gc[0]; g.N = gc[1];
@@ -961,8 +1015,38 @@ inline GemmProgram match_tiled_gemm(Operation* kernel, Operation* module = nullp
   g.tile_m = tm; g.tile_n = tn; g.tile_k = tkA;
   if (g.grid_m * g.tile_m != g.M || g.grid_n * g.tile_n != g.N) return bad("grid x tile does not cover C exactly");
   int64_t lo = loop->int_attr("lower"), hi = loop->int_attr("upper"), step = loop->int_attr("step");
+  if (step <= 0 || hi < lo) return bad("the K loop must count upwards");
   int64_t trips = (hi - lo + step - 1) / step;
-  if (trips * g.tile_k != g.K && (hi - lo) != g.K) return bad("the K loop does not cover K exactly");
+  if (trips * g.tile_k != g.K) return bad("the K loop does not cover K exactly");
+  // The kernels compute the canonical tiling: tile (by, bx) of C from row band by of op(A) and column band bx of op(B),
+  // K tile t of both in iteration t.  Check that the copies address exactly those windows.
+  Block* loop_body = loop->regions[0]->blocks[0];
+  if (body->args.size() != 2 || loop_body->args.size() != 1) return bad("unexpected block arguments");
+  const Value by{body->args[0]}, bx{body->args[1]}, kv{loop_body->args[0]};
+  auto window = [&](const Operation* cp, bool dst_side, bool is_global, int64_t rows, int64_t cols, int m_axis, int n_axis, int k_axis, const char* what) {
+    const CopyOrigin o = copy_origin(cp, dst_side, by, bx, cp == store ? Value{} : kv);
+    if (o.c0.size() != 2) throw std::invalid_argument(std::string("not a tiled GEMM kernel: ") + what + " is not addressed with two indices");
+    const std::vector<int64_t>& ext = cp->attr(dst_side ? "dstExtents" : "srcExtents")->ints;
+    if (!(ext.size() == 2 && ext[0] == rows && ext[1] == cols)) throw std::invalid_argument(std::string("not a tiled GEMM kernel: the window of ") + what + " is not one whole tile");
+    for (int r = 0; r < 2; ++r) {
+      const int64_t want_m = (is_global && r == m_axis) ? (m_axis == 0 ? rows : cols) : 0;
+      const int64_t want_n = (is_global && r == n_axis) ? (n_axis == 0 ? rows : cols) : 0;
+      const bool k_here = is_global && r == k_axis;
+      const bool ok = o.cm[(size_t)r] == want_m && o.cn[(size_t)r] == want_n &&
+                      (k_here ? (o.ck[(size_t)r] * step == g.tile_k && o.c0[(size_t)r] + o.ck[(size_t)r] * lo == 0) : (o.ck[(size_t)r] == 0 && o.c0[(size_t)r] == 0));
+      if (!ok) throw std::invalid_argument(std::string("not a tiled GEMM kernel: ") + what + " is not the window of the canonical tiling (tile (by, bx) of C, K tile of the loop iteration)");
+    }
+  };
+  for (Operation* cp : loads) {
+    const bool is_a = cp->operands[1] == sA;
+    const auto& sh = is_a ? sa : sb;
+    // stored [M][K] / [K][M] for A, [K][N] / [N][K] for B
+    const bool k_first = is_a ? g.transA : !g.transB;
+    window(cp, false, true, sh[0], sh[1], is_a ? (k_first ? 1 : 0) : -1, is_a ? -1 : (k_first ? 1 : 0), k_first ? 0 : 1, is_a ? "the source of A" : "the source of B");
+    window(cp, true, false, sh[0], sh[1], -1, -1, -1, is_a ? "the shared tile of A" : "the shared tile of B");
+  }
+  window(store, false, false, g.tile_m, g.tile_n, -1, -1, -1, "the accumulator");
+  window(store, true, true, g.tile_m, g.tile_n, 0, 1, -1, "the destination in C");
   g.elem_ab = sA.type().element();
   if (!g.elem_ab.equals(sB.type().element()) || !g.elem_ab.equals(gA.type().element()) || !g.elem_ab.equals(gB.type().element()))
     return bad("A and B element types differ between global and shared memory");

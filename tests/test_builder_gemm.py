@@ -176,6 +176,73 @@ def test_matcher_rejects_what_is_not_a_tiled_gemm():
     assert F.runtime.match(kernel)["target"] == "gfx950"
 
 
+def _reparsed_kernel(text):
+    ctx = F.create_context()
+    module = F.parse_module(ctx, text)
+    module.context = ctx
+    return module, module.get_kernel("g")
+
+
+def test_matcher_checks_what_the_program_computes_not_only_its_shape():
+    """A kernel that has the ops of a tiled GEMM but addresses other windows, clears the accumulator with another value or not
+    at all, would be silently run as the canonical GEMM: the matcher refuses each of them"""
+    h = F.create_session()
+    h.tiled_gemm("g", 512, 768, 256, "fp16", tile=(256, 256, 64))
+    text = str(h.module)
+    assert F.runtime.match(_reparsed_kernel(text)[1])["tile"] == (256, 256, 64)       # the unchanged text is accepted
+    # equivalent forms are accepted: the K loop counting elements instead of tiles
+    by_elements = text.replace("frisk.for %arg5 = 0 to 4 {", "frisk.for %arg5 = 0 to 256 step = 64 {").replace("%arg5 * 64", "%arg5")
+    assert F.runtime.match(_reparsed_kernel(by_elements)[1])["K"] == 256
+    variants = {
+        "fill value": (text.replace("value = 0.000000e+00", "value = 1.000000e+00"), "filled with 0"),
+        "no fill": ("\n".join(l for l in text.splitlines() if "frisk.fill" not in l), "cleared by a frisk.fill"),
+        "swapped grid indices in the store": (text.replace("%arg2[%arg3 * 256, %arg4 * 256]", "%arg2[%arg4 * 256, %arg3 * 256]"), "canonical tiling"),
+        "offset window of A": (text.replace("%arg0[%arg3 * 256, %arg5 * 64]", "%arg0[%arg3 * 256, %arg5 * 64 + 64]"), "canonical tiling"),
+        "A indexed by the wrong grid index": (text.replace("%arg0[%arg3 * 256,", "%arg0[%arg4 * 256,"), "canonical tiling"),
+        "wrong K stride of B": (text.replace("%arg1[%arg5 * 64,", "%arg1[%arg5 * 32,"), "canonical tiling"),
+        "offset inside the shared tile": (text.replace("%0[0, 0] {src_extents = [256, 64]", "%0[0, 8] {src_extents = [256, 64]"), "canonical tiling"),
+        "window smaller than the tile": (text.replace("{src_extents = [256, 64], dst_extents = [256, 64]}", "{src_extents = [128, 64], dst_extents = [128, 64]}"), "whole tile"),
+        "K loop short of K": (text.replace("frisk.for %arg5 = 0 to 4 {", "frisk.for %arg5 = 0 to 3 {"), "cover K"),
+    }
+    for name, (changed, message) in variants.items():
+        assert changed != text, name
+        module, kernel = _reparsed_kernel(changed)
+        with pytest.raises(ValueError, match=message):
+            F.runtime.match(kernel)
+    # a rank-1 shared buffer is refused before its shape is indexed
+    h2 = F.create_session()
+    b = h2.builder
+    tys = [h2.memref_type((256, 64), "fp16"), h2.memref_type((64, 256), "fp16"), h2.memref_type((256, 256), "fp16")]
+    kernel, entry = h2.new_kernel("g", tys)
+    body = b.create_parallel_op([1, 1], 256).add_entry_block()
+    b.set_insertion_point_to_start(body)
+    flat = h2.alloc_buffer((256 * 64,), "fp16", space=F.MemorySpace.SHARED)
+    sB = h2.alloc_buffer((64, 256), "fp16", space=F.MemorySpace.SHARED)
+    with pytest.raises(ValueError):
+        h2.create_gemm(flat, sB, h2.alloc_buffer((256, 256), "fp32", space=F.MemorySpace.LOCAL))      # the builder already refuses rank 1
+
+
+def test_transpose_flags_stored_transposed_first_then_the_references_reading():
+    """ffi/ir.cpp:346-355 reads A as [M][K] and B as [K][N] whatever the flags say; this build reads a flagged operand as stored
+    transposed when the shapes allow it, and falls back to the reference's reading (flag = layout hint) when only that fits"""
+    h = F.create_session()
+    mk = lambda shape, space=F.MemorySpace.SHARED, dt="fp16": h.alloc_buffer(shape, dt, space=space)
+    h.new_kernel("k", [])
+    acc = mk((128, 256), F.MemorySpace.LOCAL, "fp32")
+    stored_t = h.create_gemm(mk((128, 64)), mk((256, 64)), acc, trans_b=True)          # B stored [N][K]
+    assert "K = 64 : i64, M = 128 : i64, N = 256 : i64" in str(stored_t) and "transB = true" in str(stored_t)
+    hint = h.create_gemm(mk((128, 64)), mk((64, 256)), acc, trans_a=True, trans_b=True)  # the reference's reading: shapes un-transposed
+    assert "K = 64 : i64, M = 128 : i64, N = 256 : i64" in str(hint) and hint.verify()
+    with pytest.raises(ValueError, match="inner dimensions"):
+        h.create_gemm(mk((128, 64)), mk((256, 32)), acc, trans_b=True)                  # fits neither reading
+    # in a tiled program the hint form runs as the un-transposed GEMM
+    h2 = F.create_session()
+    h2.tiled_gemm("g", 512, 768, 256, "fp16", tile=(256, 256, 64))
+    text = str(h2.module).replace("transA = false, transB = false", "transA = true, transB = true")
+    p = F.runtime.match(_reparsed_kernel(text)[1])
+    assert not p["transA"] and not p["transB"] and (p["M"], p["N"], p["K"]) == (512, 768, 256)
+
+
 def test_plan_goes_through_the_hip_library():
     h = F.create_session()
     kernel = h.tiled_gemm("g", 4096, 4096, 4096, "fp16", tile=(256, 256, 64), trans_b=True)

@@ -274,3 +274,23 @@ def test_softmax_gpu(hip, dt):
     torch.cuda.synchronize()
     g = O.decode(dt, _host(d, st)).astype(np.float64).reshape(4, 512)
     assert np.all(g[:, 17] == 0.0) and np.allclose(g.sum(axis=1), 1.0, atol=64 * tol)
+    # the same on the streaming paths, whose running (maximum, sum) meets the mask first: masked columns incl. column 0 in a
+    # row of two sweeps (over 16384 elements per row), an odd-length long row (element by element) and a row split over work-groups
+    for rows, cols, use_ws in ((3, 20480, False), (2, 18001, False), (2, 65536, True)):
+        vals = O.encode(dt, O.normal(rows * cols, 45, 0, 1.0)).reshape(rows, cols)
+        masked = [0, 1, 7, cols // 2, cols - 1]
+        vals[:, masked] = O.encode(dt, np.array([-np.inf], dtype=np.float32))[0]
+        ref, lse = T.softmax_f64(dt, vals, 1.25)
+        dS = _dev(vals)
+        dD = torch.zeros_like(dS)
+        dL = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
+        ws_bytes = hip.softmax_workspace_bytes(dt, rows, cols) if use_ws else 0
+        assert ws_bytes > 0 or not use_ws
+        ws = torch.full((max(ws_bytes, 4),), 0xFF, dtype=torch.uint8, device="cuda")
+        hip.softmax(dt, dS.data_ptr(), cols, dD.data_ptr(), cols, rows, cols, 1.25, dL.data_ptr(), stream, ws.data_ptr() if ws_bytes else None, ws_bytes)
+        torch.cuda.synchronize()
+        g = O.decode(dt, _host(dD, st)).astype(np.float64).reshape(rows, cols)
+        scale = np.maximum(np.abs(ref), np.sqrt(np.mean(ref * ref)))
+        assert np.all(np.isfinite(g)) and np.all(g[:, masked] == 0.0), (rows, cols)
+        assert np.all(np.abs(g - ref) <= tol * scale + floor), (rows, cols, float(np.max(np.abs(g - ref) / scale)))
+        assert np.abs(dL.cpu().numpy() - lse).max() <= 1e-4 * max(1.0, np.abs(lse).max()), (rows, cols)
