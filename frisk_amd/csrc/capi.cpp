@@ -251,6 +251,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   const auto& ks = kernels();
   int best = -1;
   double best_cost = 0.0;
+  bool policy_excluded = false;
   bool any_layout = false, tile_requested = d->tile_m || d->tile_n || d->tile_k || d->waves_m || d->waves_n || d->stages || d->atom;
   auto search = [&](bool want_split) {
     for (size_t i = 0; i < ks.size(); ++i) {
@@ -264,6 +265,13 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
       if (d->waves_n && d->waves_n != k->wn) continue;
       if (d->stages && d->stages != k->stages_b) continue;  // the deeper ring names the variant
       if (d->atom && d->atom != k->atom) continue;
+      // frisk.gemm's wave policy (FriskOps.td:248-289) decides the wave grid unless the descriptor names one: only variants
+      // whose compiled grid is what computeWarpPartition gives for their tile and wave count under that policy qualify
+      if (!d->waves_m && !d->waves_n) {
+        int pm = 0, pn = 0;
+        wave_partition(d->policy, k->bm, k->bn, k->wm * k->wn, k->atom, k->atom, &pm, &pn);
+        if (pm != k->wm || pn != k->wn) { policy_excluded = true; continue; }
+      }
       if (want_split && !k->splitk) continue;
       // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
       if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
@@ -284,6 +292,9 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   }
   if (best < 0) {
     if (!any_layout) return fail(FRISK_ERR_DTYPE, "no kernel compiled for dtype %d transA=%d transB=%d", d->dtype_ab, d->transA, d->transB);
+    if (policy_excluded && d->policy != FRISK_POLICY_SQUARE)
+      return fail(FRISK_ERR_TILE, "wave policy %s: no compiled kernel for M=%lld N=%lld K=%lld has the wave grid that policy gives (compiled grids: 2x2, 1x4, 2x4, 1x1)",
+                  d->policy == FRISK_POLICY_FULL_ROW ? "FullRow" : "FullCol", (long long)d->M, (long long)d->N, (long long)d->K);
     if (tile_requested)
       return fail(FRISK_ERR_TILE, "no compiled kernel with tile %dx%dx%d waves %dx%d atom %d divides M=%lld N=%lld K=%lld", d->tile_m, d->tile_n,
                   d->tile_k, d->waves_m, d->waves_n, d->atom, (long long)d->M, (long long)d->N, (long long)d->K);

@@ -86,7 +86,9 @@ typedef struct frisk_gemm_desc {
   uint8_t split_k; /* slices of K computed by separate work-groups and summed through the workspace:
                       0 = planner's choice (splits only skinny problems, and only if a workspace is passed), 1 = never */
   int32_t epilogue;
-  int32_t policy;                 /* frisk_wave_policy */
+  int32_t policy;                 /* frisk_wave_policy: only kernel variants whose wave grid is the policy's partition of their tile
+                                     (frisk_hip_wave_partition) qualify; FRISK_ERR_TILE when none is compiled.  Ignored when
+                                     waves_m / waves_n name a grid */
   int32_t tile_m, tile_n, tile_k; /* block tile = the M,N,K attrs of the tile-level frisk.gemm */
   int32_t waves_m, waves_n;       /* wave grid inside the work-group */
   int32_t stages;                 /* LDS stages of the global->LDS pipeline (of B when A and B differ), 0 = planner's choice */

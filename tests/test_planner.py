@@ -257,6 +257,34 @@ def test_planner_ranks_variants_by_estimated_time():
     assert not pick(R.F16, 64, 384, 2048).endswith("_guard") and pick(R.F16, 65, 384, 2048).endswith("_guard")
 
 
+def test_wave_policy_decides_the_wave_grid():
+    """frisk.gemm's policy (FriskOps.td:248-289, computeWarpPartition FriskOps.cpp:825-888) is honoured by the planner: among
+    the compiled variants only those whose wave grid is the policy's partition of their tile qualify, unless the descriptor
+    names a wave grid itself"""
+    names = R.kernel_names()
+    square = R.plan(R.make_desc(R.F16, 4096, 4096, 4096))
+    assert (square.tile_m, square.tile_n, square.waves_m, square.waves_n) == (256, 256, 2, 2)
+    assert (square.waves_m, square.waves_n) == R.wave_partition(R.POLICY_SQUARE, 256, 256, 4)
+    # FullCol puts all four waves side by side along N: the 32 x 128 tile is the compiled variant with that grid
+    col = R.plan(R.make_desc(R.F16, 4096, 4096, 4096, policy=R.POLICY_FULL_COL))
+    assert (col.tile_m, col.tile_n, col.waves_m, col.waves_n) == (32, 128, 1, 4) == (32, 128) + R.wave_partition(R.POLICY_FULL_COL, 32, 128, 4)
+    assert names[col.kernel_id] != names[square.kernel_id]
+    # on the 256 x 256 tile FullRow asks for 4 x 1 and FullCol for 1 x 4 waves: neither is compiled, the plan is refused
+    for policy, grid in ((R.POLICY_FULL_ROW, (4, 1)), (R.POLICY_FULL_COL, (1, 4))):
+        assert R.wave_partition(policy, 256, 256, 4) == grid
+        with pytest.raises(R.FriskHipError) as e:
+            R.plan(R.make_desc(R.F16, 4096, 4096, 4096, policy=policy, tile=(256, 256, 64)))
+        assert e.value.status == R.ERR_TILE and "wave policy" in str(e.value)
+    # an explicit wave grid overrides the policy
+    p = R.plan(R.make_desc(R.F16, 4096, 4096, 4096, policy=R.POLICY_FULL_ROW, waves=(2, 4)))
+    assert (p.waves_m, p.waves_n) == (2, 4)
+    # every variant the planner picks by itself carries the Square partition of its tile
+    for dt, M, N, K, kw in ((R.F16, 2048, 2048, 2048, {}), (R.BF16, 1024, 8192, 8192, {"transB": True}), (R.F32, 1024, 1024, 1024, {}),
+                            (R.F16, 100, 75, 40, {}), (R.I8, 64, 2048, 8192, {"dtype_out": R.I32}), (R.E4M3, 32, 8192, 8192, {"transB": True, "dtype_out": R.BF16})):
+        p = R.plan(R.make_desc(dt, M, N, K, **kw))
+        assert (p.waves_m, p.waves_n) == R.wave_partition(R.POLICY_SQUARE, p.tile_m, p.tile_n, p.waves_m * p.waves_n), names[p.kernel_id]
+
+
 def test_atom_choice_follows_the_fill_of_the_round():
     """16-bit 256x256 tiles: K-contiguous operands (NT) always take the 16x16x32 atoms; layouts with a transpose-read operand
     take them from 176 tiles of a round of 256 up (measured crossover between 144 and 192 tiles)"""
