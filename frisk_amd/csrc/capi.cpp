@@ -449,6 +449,7 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
   p.tail_from = p.tiles_m * p.tiles_n - plan.tail_tiles;
   p.tail_kt = plan.tail_split > 1 ? p.kt_per_slice / plan.tail_split : 0;
   p.tile_m = k->bm; p.tile_n = k->bn;
+  p.k_rotate = 1;
   hipError_t e = k->launch(p, (hipStream_t)stream);
   if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "launch of %s failed: %s", k->name, hipGetErrorString(e));
   if (plan.split_k > 1) {

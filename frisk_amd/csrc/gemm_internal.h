@@ -27,6 +27,7 @@ struct GemmParams {
   // partial[slice][tile - tail_from][BM][BN] and a second kernel sums them.  tail_split <= 1: no tail.
   int tail_from, tail_tiles, tail_split, tail_kt;
   int tile_m, tile_n;  // BM, BN of the kernel (for the tail reduction)
+  int k_rotate;        // 32-row kernels: work-groups start at different K tiles of their slice and wrap around
 };
 
 // Hardware hands consecutive work-group ids to the 8 XCDs round-robin.  Give each XCD a contiguous range of "compact"

@@ -74,6 +74,36 @@ struct Builder {
   }
   Operation* make_end() { return ctx->new_op("frisk.end"); }
   template <class T> T wrap(Operation* op) { T t; t.op = op; t.ctx = ctx; return t; }
+  // scalar ops of frisk.block bodies: one result each
+  Value constant(const Attribute& v) {
+    Operation* op = ctx->new_op("arith.constant");
+    op->attrs["value"] = v;
+    Value r = ctx->add_result(op, v.kind == Attribute::Float ? v.type : Type::scalar(TypeKind::I64));
+    insert(op);
+    return r;
+  }
+  Value scalar_op(const std::string& name, std::vector<Value> operands) {
+    const Type t = operands.at(0).type();
+    if (!t.is_float()) throw std::invalid_argument(name + " expects floating-point operands");
+    for (const Value& v : operands)
+      if (!v.type().equals(t)) throw std::invalid_argument(name + " expects operands of one type, got " + t.str() + " and " + v.type().str());
+    Operation* op = ctx->new_op(name);
+    op->operands = operands;
+    Value r = ctx->add_result(op, t);
+    insert(op);
+    return r;
+  }
+  Value cast_op(const std::string& name, Value x, const Type& to) {
+    const Type from = x.type();
+    if (!from.is_float() || !to.is_float()) throw std::invalid_argument(name + " casts between floating-point types");
+    if (name == "arith.extf" ? from.bit_width() >= to.bit_width() : from.bit_width() <= to.bit_width())
+      throw std::invalid_argument(name + ": " + from.str() + " to " + to.str() + " is not " + (name == "arith.extf" ? "a widening" : "a narrowing"));
+    Operation* op = ctx->new_op(name);
+    op->operands = {x};
+    Value r = ctx->add_result(op, to);
+    insert(op);
+    return r;
+  }
 };
 
 static Type parse_dtype(const std::string& dtype) {
@@ -728,7 +758,49 @@ void init_ffi_ir(py::module_&& m) {
         op->attrs["clear"] = Attribute::boolean(clear);
         b.insert(op);
         return b.wrap<ReduceOp>(op);
-      }, py::arg("src"), py::arg("dst"), py::arg("kind"), py::arg("dim"), py::arg("clear") = true);
+      }, py::arg("src"), py::arg("dst"), py::arg("kind"), py::arg("dim"), py::arg("clear") = true)
+      // ---- scalar values: the constants of the reference's builder (ffi/ir.cpp:178-193) ...
+      .def("get_f16", [](Builder& b, float v) { return b.constant(Attribute::floating((double)v, Type::scalar(TypeKind::F16))); })
+      .def("get_f32", [](Builder& b, float v) { return b.constant(Attribute::floating((double)v, Type::scalar(TypeKind::F32))); })
+      .def("get_f64", [](Builder& b, double v) { return b.constant(Attribute::floating(v, Type::scalar(TypeKind::F64))); })
+      .def("get_int64", [](Builder& b, int64_t v) { return b.constant(Attribute::integer(v, 64)); })
+      // ... and what the bodies of frisk.block need beyond them (tmp/ir.mlir:39-47, 114-147 use affine.load / affine.store,
+      // arith.mulf / subf / addf, math.exp2 / log2; the reference's builder has no creators for these)
+      .def("create_load_op", [](Builder& b, Value memref, std::vector<Value> indices, AffineMap map) {
+        if (!memref.type().is_memref()) throw std::invalid_argument("create_load_op expects a memref");
+        if (!map) map = AffineMap::identity((int)memref.type().impl->shape.size());
+        if ((int)indices.size() != map.num_inputs()) throw std::invalid_argument("create_load_op: the map takes " + std::to_string(map.num_inputs()) + " indices, got " + std::to_string(indices.size()));
+        if (map.num_results() != (int)memref.type().impl->shape.size()) throw std::invalid_argument("create_load_op: the map must give one index per memref dimension");
+        Operation* op = b.ctx->new_op("affine.load");
+        op->operands = {memref};
+        op->operands.insert(op->operands.end(), indices.begin(), indices.end());
+        op->attrs["map"] = Attribute::affine_map(map);
+        Value r = b.ctx->add_result(op, memref.type().element());
+        b.insert(op);
+        return r;
+      }, py::arg("memref"), py::arg("indices"), py::arg("map") = AffineMap())
+      .def("create_store_op", [](Builder& b, Value value, Value memref, std::vector<Value> indices, AffineMap map) {
+        if (!memref.type().is_memref()) throw std::invalid_argument("create_store_op expects a memref");
+        if (!map) map = AffineMap::identity((int)memref.type().impl->shape.size());
+        if ((int)indices.size() != map.num_inputs()) throw std::invalid_argument("create_store_op: the map takes " + std::to_string(map.num_inputs()) + " indices, got " + std::to_string(indices.size()));
+        if (map.num_results() != (int)memref.type().impl->shape.size()) throw std::invalid_argument("create_store_op: the map must give one index per memref dimension");
+        if (!value.type().equals(memref.type().element())) throw std::invalid_argument("create_store_op: the value's type is not the memref's element type");
+        Operation* op = b.ctx->new_op("affine.store");
+        op->operands = {value, memref};
+        op->operands.insert(op->operands.end(), indices.begin(), indices.end());
+        op->attrs["map"] = Attribute::affine_map(map);
+        b.insert(op);
+        return OpState{op, b.ctx};
+      }, py::arg("value"), py::arg("memref"), py::arg("indices"), py::arg("map") = AffineMap())
+      .def("create_mulf", [](Builder& b, Value l, Value r) { return b.scalar_op("arith.mulf", {l, r}); })
+      .def("create_addf", [](Builder& b, Value l, Value r) { return b.scalar_op("arith.addf", {l, r}); })
+      .def("create_subf", [](Builder& b, Value l, Value r) { return b.scalar_op("arith.subf", {l, r}); })
+      .def("create_divf", [](Builder& b, Value l, Value r) { return b.scalar_op("arith.divf", {l, r}); })
+      .def("create_maxnumf", [](Builder& b, Value l, Value r) { return b.scalar_op("arith.maxnumf", {l, r}); })
+      .def("create_exp2", [](Builder& b, Value x) { return b.scalar_op("math.exp2", {x}); })
+      .def("create_log2", [](Builder& b, Value x) { return b.scalar_op("math.log2", {x}); })
+      .def("create_extf", [](Builder& b, Value x, Type to) { return b.cast_op("arith.extf", x, to); })
+      .def("create_truncf", [](Builder& b, Value x, Type to) { return b.cast_op("arith.truncf", x, to); });
 
   // ---------------------------------------------------------------- dialect registration (ffi/ir.cpp:33-47)
   auto frisk = m.def_submodule("frisk");

@@ -371,6 +371,12 @@ class IrParser {
     if (!v.type().equals(t)) fail("use of value '" + name + "' expects different type than prior uses: '" + t.str() + "' vs '" + v.type().str() + "'");
   }
 
+  void one_result(Operation* op, std::vector<std::string>& results, const Type& t) {
+    if (results.size() != 1) fail("operation '" + op->name + "' defines one result");
+    define(results[0], ctx_.add_result(op, t).impl);
+    results.clear();
+  }
+
   void parse_operation(Block* block) {
     skip();
     std::vector<std::string> results;
@@ -507,6 +513,43 @@ class IrParser {
       }
     } else if (n == "frisk.end") {
       try_attr_dict(op);
+    } else if (n == "arith.constant") {
+      Attribute v = parse_attribute();
+      if (v.kind != Attribute::Float && v.kind != Attribute::Int) fail("arith.constant expects a number with its type");
+      op->attrs["value"] = v;
+      one_result(op, results, v.kind == Attribute::Float ? v.type : Type::scalar(v.int_width == 32 ? TypeKind::I32 : TypeKind::I64));
+    } else if (n == "affine.load" || n == "affine.store") {
+      std::string stored;
+      if (n == "affine.store") { stored = ssa_name(); expect(","); }
+      const std::string mem = ssa_name();
+      std::vector<Value> idx;
+      AffineMap map = parse_map_of_ssa_ids(idx);
+      expect(":");
+      Type mt = memref_type("the accessed buffer");
+      Value mv = use(mem);
+      check_operand_type(mv, mt, mem);
+      if (n == "affine.store") op->operands.push_back(use(stored));
+      op->operands.push_back(mv);
+      op->operands.insert(op->operands.end(), idx.begin(), idx.end());
+      op->attrs["map"] = Attribute::affine_map(map);
+      if (n == "affine.load") one_result(op, results, mt.element());
+    } else if (is_scalar_binary(n) || is_scalar_unary(n)) {
+      std::vector<std::string> names = {ssa_name()};
+      if (is_scalar_binary(n)) { expect(","); names.push_back(ssa_name()); }
+      expect(":");
+      Type t = parse_type();
+      for (auto& nm : names) { Value v = use(nm); check_operand_type(v, t, nm); op->operands.push_back(v); }
+      one_result(op, results, t);
+    } else if (is_scalar_cast(n)) {
+      const std::string nm = ssa_name();
+      expect(":");
+      Type from = parse_type();
+      expect_word("to");
+      Type to = parse_type();
+      Value v = use(nm);
+      check_operand_type(v, from, nm);
+      op->operands.push_back(v);
+      one_result(op, results, to);
     } else {
       fail("unknown operation '" + n + "'");
     }

@@ -584,6 +584,15 @@ struct Context {
   Value add_block_arg(Block* b, Type t) { ValueImpl* v = new_value(t); v->block = b; v->index = (int)b->args.size(); b->args.push_back(v); return Value{v}; }
 };
 
+// The scalar ops of frisk.block bodies (the element-wise steps of the reference's sketches, tmp/ir.mlir:39-47, 49-60,
+// 114-147): constants, affine.load / affine.store, floating binary and unary ops, width casts.  Upstream MLIR ops, printed
+// in their standard forms.
+inline bool is_scalar_binary(const std::string& n) {
+  return n == "arith.mulf" || n == "arith.addf" || n == "arith.subf" || n == "arith.divf" || n == "arith.maxnumf" || n == "arith.minnumf";
+}
+inline bool is_scalar_unary(const std::string& n) { return n == "math.exp2" || n == "math.log2" || n == "arith.negf"; }
+inline bool is_scalar_cast(const std::string& n) { return n == "arith.extf" || n == "arith.truncf"; }
+
 // ------------------------------------------------------------------ printer
 struct Printer {
   std::map<const ValueImpl*, std::string> names;
@@ -724,6 +733,22 @@ struct Printer {
       os << " : " << op->operands[0].type().str() << ", " << op->operands[1].type().str();
     } else if (n == "frisk.end") {
       os << "frisk.end";
+    } else if (n == "arith.constant") {
+      os << "arith.constant " << op->attr("value")->str();
+    } else if (n == "affine.load") {
+      os << "affine.load " << name(op->operands[0]) << "[";
+      map_of_ssa_ids(op->attr("map")->map, std::vector<Value>(op->operands.begin() + 1, op->operands.end()));
+      os << "] : " << op->operands[0].type().str();
+    } else if (n == "affine.store") {
+      os << "affine.store " << name(op->operands[0]) << ", " << name(op->operands[1]) << "[";
+      map_of_ssa_ids(op->attr("map")->map, std::vector<Value>(op->operands.begin() + 2, op->operands.end()));
+      os << "] : " << op->operands[1].type().str();
+    } else if (is_scalar_binary(n)) {
+      os << n << " " << name(op->operands[0]) << ", " << name(op->operands[1]) << " : " << op->results[0]->type.str();
+    } else if (is_scalar_unary(n)) {
+      os << n << " " << name(op->operands[0]) << " : " << op->results[0]->type.str();
+    } else if (is_scalar_cast(n)) {
+      os << n << " " << name(op->operands[0]) << " : " << op->operands[0].type().str() << " to " << op->results[0]->type.str();
     } else {
       os << "\"" << n << "\"(";
       for (size_t i = 0; i < op->operands.size(); ++i) os << (i ? ", " : "") << name(op->operands[i]);
@@ -836,6 +861,39 @@ inline bool verify_operation(const Operation* op, Diagnostics& d) {
     if (nd != dm.num_inputs()) fail("expected " + std::to_string(dm.num_inputs()) + " destination indices, but got " + std::to_string(nd));
     if (s && sm.num_results() != (int)s->shape.size()) fail("source map must produce one index per source dimension");
     if (t && dm.num_results() != (int)t->shape.size()) fail("destination map must produce one index per destination dimension");
+  } else if (n == "arith.constant") {
+    const Attribute* v = op->attr("value");
+    if (!v || (v->kind != Attribute::Float && v->kind != Attribute::Int)) fail("requires a numeric 'value' attribute");
+    else if (op->results.size() != 1) fail("defines one result");
+    else if (v->kind == Attribute::Float && !op->results[0]->type.equals(v->type)) fail("result type does not match the value's type");
+  } else if (n == "affine.load" || n == "affine.store") {
+    const size_t at = n == "affine.load" ? 0 : 1;
+    const TypeImpl* m = memref_operand(at, "memref");
+    const Attribute* map = op->attr("map");
+    if (!map || map->kind != Attribute::Map) fail("requires a 'map' attribute");
+    else if (m) {
+      if (map->map.num_results() != (int)m->shape.size()) fail("map must produce one index per memref dimension");
+      if ((int)op->operands.size() - (int)at - 1 != map->map.num_inputs()) fail("index operand count does not match the map");
+      for (size_t i = at + 1; i < op->operands.size(); ++i) if (op->operands[i].type().kind() != TypeKind::Index) fail("indices must have index type");
+      const Type elem(m->element);
+      if (n == "affine.load" && (op->results.size() != 1 || !op->results[0]->type.equals(elem))) fail("result type must be the memref element type");
+      if (n == "affine.store" && !op->operands[0].type().equals(elem)) fail("stored value type must be the memref element type");
+    }
+  } else if (is_scalar_binary(n) || is_scalar_unary(n)) {
+    const size_t want = is_scalar_binary(n) ? 2 : 1;
+    if (op->operands.size() != want || op->results.size() != 1) fail("wrong number of operands or results");
+    else {
+      const Type& t = op->results[0]->type;
+      if (!t.is_float()) fail("operates on floating-point values");
+      for (const Value& v : op->operands) if (!v.type().equals(t)) fail("operand and result types must be the same");
+    }
+  } else if (is_scalar_cast(n)) {
+    if (op->operands.size() != 1 || op->results.size() != 1) fail("wrong number of operands or results");
+    else {
+      const Type from = op->operands[0].type(), to = op->results[0]->type;
+      if (!from.is_float() || !to.is_float()) fail("casts between floating-point types");
+      else if (n == "arith.extf" ? from.bit_width() >= to.bit_width() : from.bit_width() <= to.bit_width()) fail(n == "arith.extf" ? "result must be wider than the operand" : "result must be narrower than the operand");
+    }
   } else if (n == "frisk.fill") {
     const TypeImpl* m = memref_operand(0, "memref");
     if (m && !Type(m->element).equals(op->attr("value")->type)) fail("fill value type does not match the memref element type");

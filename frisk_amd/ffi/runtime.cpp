@@ -13,6 +13,7 @@
 #include "frisk_hip.h"
 #include "mini_ir.h"
 #include "layout_infer.h"
+#include "programs.h"
 
 namespace frisk_ffi {
 
@@ -33,6 +34,9 @@ struct HipLibrary {
   decltype(&frisk_hip_copy) copy = nullptr;
   decltype(&frisk_hip_reduce) reduce = nullptr;
   decltype(&frisk_hip_reduce_workspace_bytes) reduce_workspace_bytes = nullptr;
+  decltype(&frisk_hip_softmax) softmax = nullptr;
+  decltype(&frisk_hip_softmax_workspace_bytes) softmax_workspace_bytes = nullptr;
+  decltype(&frisk_hip_attention) attention = nullptr;
 };
 
 HipLibrary g_lib;
@@ -57,7 +61,10 @@ HipLibrary& library() {
   lib.copy = (decltype(lib.copy))dlsym(h, "frisk_hip_copy");
   lib.reduce = (decltype(lib.reduce))dlsym(h, "frisk_hip_reduce");
   lib.reduce_workspace_bytes = (decltype(lib.reduce_workspace_bytes))dlsym(h, "frisk_hip_reduce_workspace_bytes");
-  if (!lib.plan || !lib.gemm || !lib.last_error || !lib.abi_version || !lib.kernel_name || !lib.fill || !lib.copy || !lib.reduce || !lib.reduce_workspace_bytes)
+  lib.softmax = (decltype(lib.softmax))dlsym(h, "frisk_hip_softmax");
+  lib.softmax_workspace_bytes = (decltype(lib.softmax_workspace_bytes))dlsym(h, "frisk_hip_softmax_workspace_bytes");
+  lib.attention = (decltype(lib.attention))dlsym(h, "frisk_hip_attention");
+  if (!lib.softmax || !lib.softmax_workspace_bytes || !lib.attention || !lib.plan || !lib.gemm || !lib.last_error || !lib.abi_version || !lib.kernel_name || !lib.fill || !lib.copy || !lib.reduce || !lib.reduce_workspace_bytes)
     throw std::runtime_error("frisk runtime: " + g_lib_path + " does not export the frisk_hip entry points");
   if (lib.abi_version() != FRISK_HIP_ABI_VERSION) throw std::runtime_error("frisk runtime: libfrisk_hip.so ABI version mismatch");
   g_lib = lib;
@@ -196,6 +203,51 @@ py::dict tile_op_dict(const TileOpDesc& d) {
   return o;
 }
 
+// Which of the recognised programs a kernel is, by the ops it holds: frisk.block bodies only occur in the softmax and
+// attention programs; two products make the attention program.
+enum class ProgramKind { TiledGemm, OnlineSoftmax, Attention };
+ProgramKind classify(Operation* kernel) {
+  int gemms = 0, blocks = 0;
+  std::function<void(Operation*)> walk = [&](Operation* op) {
+    if (op->name == "frisk.gemm") ++gemms;
+    if (op->name == "frisk.block") ++blocks;
+    for (Region* r : op->regions)
+      for (Block* b : r->blocks)
+        for (Operation* inner : b->ops) walk(inner);
+  };
+  if (kernel) walk(kernel);
+  if (blocks > 0 && gemms == 0) return ProgramKind::OnlineSoftmax;
+  if (blocks > 0 && gemms >= 2) return ProgramKind::Attention;
+  return ProgramKind::TiledGemm;
+}
+
+py::dict softmax_dict(const SoftmaxProgram& g) {
+  py::dict o;
+  o["program"] = "online_softmax";
+  o["kernel"] = g.kernel_name;
+  o["rows"] = g.rows; o["cols"] = g.cols; o["chunk"] = g.chunk;
+  o["scale_log2"] = g.cst;
+  o["dtype"] = g.elem.str();
+  o["args"] = py::make_tuple(g.arg_src, g.arg_dst);
+  o["target"] = g.target;
+  return o;
+}
+
+py::dict attention_dict(const AttentionProgram& g) {
+  py::dict o;
+  o["program"] = "attention";
+  o["kernel"] = g.kernel_name;
+  o["batch"] = g.batch; o["heads"] = g.heads; o["seq_q"] = g.seq_q; o["seq_k"] = g.seq_k; o["head_dim"] = g.head_dim;
+  o["tile"] = py::make_tuple(g.tile_q, g.tile_k);
+  o["k_transposed"] = g.k_transposed;
+  o["scale_log2"] = g.cst;
+  o["scale"] = g.cst / 1.4426950408889634;
+  o["dtype"] = g.elem.str();
+  o["args"] = py::make_tuple(g.arg_q, g.arg_k, g.arg_v, g.arg_o);
+  o["target"] = g.target;
+  return o;
+}
+
 }  // namespace
 
 void init_ffi_runtime(py::module_&& m) {
@@ -205,9 +257,20 @@ void init_ffi_runtime(py::module_&& m) {
   }, "path of libfrisk_hip.so; loaded on first use");
   m.def("library_path", []() { return g_lib_path; });
 
-  m.def("match", [](py::object kernel, py::object module) { return program_dict(program_of(kernel, module)); }, py::arg("kernel"),
-        py::arg("module") = py::none(),
-        "recognise kernel{parallel{alloc, alloc, alloc, fill, for{copy, copy, gemm}, copy}} and return the GEMM it describes; pure host");
+  m.def("match", [](py::object kernel, py::object module) {
+    Operation* k = op_of_handle(kernel);
+    Operation* mod = module.is_none() ? nullptr : op_of_handle(module);
+    switch (classify(k)) {
+      case ProgramKind::OnlineSoftmax: return softmax_dict(match_online_softmax(k, mod));
+      case ProgramKind::Attention: return attention_dict(match_attention(k, mod));
+      default: break;
+    }
+    py::dict d = program_dict(match_tiled_gemm(k, mod));
+    d["program"] = "tiled_gemm";
+    return d;
+  }, py::arg("kernel"), py::arg("module") = py::none(),
+        "recognise one of the programs of the reference's design sketches and return what it computes: the tiled GEMM "
+        "kernel{parallel{alloc x3, fill, for{copy, copy, gemm}, copy}}, the row softmax with a running log-sum, or the fused attention; pure host");
 
   m.def("plan", [](py::object kernel, py::object module, const std::string& epilogue) {
     GemmProgram g = program_of(kernel, module);
@@ -349,7 +412,43 @@ void init_ffi_runtime(py::module_&& m) {
 
   m.def("launch", [](py::object kernel, std::vector<uint64_t> args, uint64_t stream, py::object module, const std::string& epilogue,
                      uint64_t scale_a, uint64_t scale_b) {
-    GemmProgram g = program_of(kernel, module);
+    Operation* k = op_of_handle(kernel);
+    Operation* mod = module.is_none() ? nullptr : op_of_handle(module);
+    const ProgramKind kind = classify(k);
+    if (kind == ProgramKind::OnlineSoftmax) {
+      const SoftmaxProgram g = match_online_softmax(k, mod);
+      if (args.size() < (size_t)std::max(g.arg_src, g.arg_dst) + 1) throw std::invalid_argument("launch needs one device pointer per kernel argument");
+      HipLibrary& lib = library();
+      int st;
+      {
+        py::gil_scoped_release release;
+        st = lib.softmax(dtype_of(g.elem), (const void*)args[(size_t)g.arg_src], g.cols, (void*)args[(size_t)g.arg_dst], g.cols, g.rows, g.cols, (float)g.cst, nullptr,
+                         nullptr, 0, (void*)stream);
+      }
+      if (st) throw std::runtime_error(std::string("frisk_hip_softmax: ") + lib.last_error() + " (status " + std::to_string(st) + ")");
+      return;
+    }
+    if (kind == ProgramKind::Attention) {
+      const AttentionProgram g = match_attention(k, mod);
+      if (args.size() < (size_t)std::max(std::max(g.arg_q, g.arg_k), std::max(g.arg_v, g.arg_o)) + 1) throw std::invalid_argument("launch needs one device pointer per kernel argument");
+      if (!(g.cst > 0)) throw std::invalid_argument("the attention program's constant must be positive");
+      frisk_attention_desc d{};
+      d.abi_version = FRISK_HIP_ABI_VERSION;
+      d.dtype = dtype_of(g.elem);
+      d.batch = g.batch; d.heads = g.heads; d.seq_q = g.seq_q; d.seq_k = g.seq_k; d.head_dim = g.head_dim;
+      d.scale = (float)(g.cst / 1.4426950408889634);
+      d.k_transposed = g.k_transposed ? 1 : 0;
+      HipLibrary& lib = library();
+      int st;
+      {
+        py::gil_scoped_release release;
+        st = lib.attention(&d, (const void*)args[(size_t)g.arg_q], (const void*)args[(size_t)g.arg_k], (const void*)args[(size_t)g.arg_v], (void*)args[(size_t)g.arg_o],
+                           nullptr, (void*)stream);
+      }
+      if (st) throw std::runtime_error(std::string("frisk_hip_attention: ") + lib.last_error() + " (status " + std::to_string(st) + ")");
+      return;
+    }
+    GemmProgram g = match_tiled_gemm(k, mod);
     size_t need = (size_t)std::max(g.arg_a, std::max(g.arg_b, g.arg_c)) + 1;
     if (args.size() < need) throw std::invalid_argument("launch needs one device pointer per kernel argument");
     frisk_gemm_desc d = desc_of(g, epilogue_of(epilogue));
@@ -363,7 +462,8 @@ void init_ffi_runtime(py::module_&& m) {
     if (st) throw std::runtime_error(std::string("frisk_hip_gemm: ") + lib.last_error() + " (status " + std::to_string(st) + ")");
   }, py::arg("kernel"), py::arg("args"), py::arg("stream") = 0, py::arg("module") = py::none(), py::arg("epilogue") = "none",
      py::arg("scale_a") = 0, py::arg("scale_b") = 0,
-     "asynchronous launch on `stream` (a hipStream_t value); `args` holds one raw device pointer per kernel argument");
+     "asynchronous launch on `stream` (a hipStream_t value) of a recognised program (tiled GEMM, online softmax, fused attention); "
+     "`args` holds one raw device pointer per kernel argument");
 }
 
 }  // namespace frisk_ffi

@@ -151,6 +151,16 @@ class FriskHelper:
         b.create_copy_op(acc, gC, [], [by, bx], origin(b), scaled(bm, bn), [bm, bn], [bm, bn])
         return kernel
 
+    def online_softmax(self, name, rows, cols, dtype="fp16", **kw):
+        """the row softmax with a running log-sum of the reference's sketch (tmp/ir.mlir:21-75); see common/programs.py"""
+        from . import programs
+        return programs.online_softmax(self, name, rows, cols, dtype, **kw)
+
+    def attention(self, name, batch, heads, seq_q, seq_k, head_dim=128, dtype="fp16", **kw):
+        """the fused attention of the reference's sketch (tmp/ir.mlir:88-158); see common/programs.py"""
+        from . import programs
+        return programs.attention(self, name, batch, heads, seq_q, seq_k, head_dim, dtype, **kw)
+
     # ---------------------------------------------------------------- utilities
     def ensure_insertion_block(self):
         """the block the builder inserts into; when it has none yet, a new block at the end of the module's body"""
