@@ -259,8 +259,9 @@ def main():
         C1 = torch.empty(M1, M1, device=dev)
         p1 = [A1.data_ptr(), B1.data_ptr(), C1.data_ptr()]
         t1 = time_launches(torch, lambda: F.runtime.launch(kern, p1, cs), a.steps, a.warmup, stream)
-        legs["fp32_1024_builder"] = mfma_leg("fp32 1024^3 NN, U[-1,1], built with the IR builder and launched by frisk_ffi.runtime (configs[0]); "
-                                             "the time includes the builder's matching and planning on the host", "f32", 2.0 * M1 ** 3, t1)
+        legs["fp32_1024_builder"] = mfma_leg("fp32 1024^3 NN, U[-1,1], built with the IR builder (128x128x32 tiles as in the design sketch) and launched by "
+                                             "frisk_ffi.runtime, which matches the program and lets the planner pick the kernel (configs[0]); the time "
+                                             "includes that host work per launch", "f32", 2.0 * M1 ** 3, t1)
         d1 = R.make_desc(R.F32, M1, M1, M1)
         t1c = time_launches(torch, gemm_launcher(d1, (A1.data_ptr(), B1.data_ptr(), C1.data_ptr(), None, None)), a.steps, a.warmup, stream)
         legs["fp32_1024"] = mfma_leg("fp32 1024^3 NN through the C ABI, planner's choice of tile", "f32", 2.0 * M1 ** 3, t1c,

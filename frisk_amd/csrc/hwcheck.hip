@@ -141,6 +141,11 @@ template <class C> __global__ void __launch_bounds__(64) fragment_path_kernel(co
 #pragma unroll
       for (int r = 0; r < M::NACC; ++r) acc[i][j][r] = 0;
 #pragma unroll
+  for (int i = 0; i < C::AM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::AN; ++j) M::settle(acc[i][j]);
+  M::drain();
+#pragma unroll
   for (int ks = 0; ks < C::KSTEPS; ++ks) {
     int fa[C::AM][FI], fb[C::AN][FI];
 #pragma unroll
@@ -160,6 +165,7 @@ template <class C> __global__ void __launch_bounds__(64) fragment_path_kernel(co
         M::run(b, a, acc[i][j]);
       }
   }
+  M::drain();
   // accumulator convention of the epilogue: register 4q + e of lane l in atom (i, j) is
   // C[i * AT + l % AT][j * AT + (AT == 32 ? 8q + 4 (l / 32) : 4 (l / 16)) + e]
 #pragma unroll

@@ -411,7 +411,7 @@ void init_ffi_runtime(py::module_&& m) {
      "asynchronous launch, in program order on `stream`, of a kernel made of fill / copy / reduce on its arguments");
 
   m.def("launch", [](py::object kernel, std::vector<uint64_t> args, uint64_t stream, py::object module, const std::string& epilogue,
-                     uint64_t scale_a, uint64_t scale_b) {
+                     uint64_t scale_a, uint64_t scale_b, bool retile) {
     Operation* k = op_of_handle(kernel);
     Operation* mod = module.is_none() ? nullptr : op_of_handle(module);
     const ProgramKind kind = classify(k);
@@ -452,6 +452,9 @@ void init_ffi_runtime(py::module_&& m) {
     size_t need = (size_t)std::max(g.arg_a, std::max(g.arg_b, g.arg_c)) + 1;
     if (args.size() < need) throw std::invalid_argument("launch needs one device pointer per kernel argument");
     frisk_gemm_desc d = desc_of(g, epilogue_of(epilogue));
+    // The tile sizes in the IR describe the program; which kernel variant computes it best is the planner's call for the
+    // whole problem (1024^3 fp32 written with 128 x 128 tiles is 64 work-groups on 256 CUs).  retile = False keeps the IR's tile.
+    if (retile) d.tile_m = d.tile_n = d.tile_k = 0;
     HipLibrary& lib = library();
     int st;
     {
@@ -461,7 +464,7 @@ void init_ffi_runtime(py::module_&& m) {
     }
     if (st) throw std::runtime_error(std::string("frisk_hip_gemm: ") + lib.last_error() + " (status " + std::to_string(st) + ")");
   }, py::arg("kernel"), py::arg("args"), py::arg("stream") = 0, py::arg("module") = py::none(), py::arg("epilogue") = "none",
-     py::arg("scale_a") = 0, py::arg("scale_b") = 0,
+     py::arg("scale_a") = 0, py::arg("scale_b") = 0, py::arg("retile") = true,
      "asynchronous launch on `stream` (a hipStream_t value) of a recognised program (tiled GEMM, online softmax, fused attention); "
      "`args` holds one raw device pointer per kernel argument");
 }

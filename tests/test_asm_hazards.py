@@ -1,0 +1,82 @@
+"""The 16-row MFMA atoms are written as inline assembly (gemm_kernel.hip.inc: Mma<*, 16>), so the compiler places none of the
+wait states an MFMA needs around them.  This test compiles a few of those kernels to gfx950 ISA (no GPU needed) and
+checks the two patterns that would be wrong: a vector instruction writing a register that an MFMA reads within the next
+few instructions (accumulator initialisation right before the first MFMA), and a vector instruction reading an MFMA
+result too soon after it (before the drain the kernel issues ahead of the epilogue)."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "frisk_amd", "csrc")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+SOURCE = """
+#include "gemm_kernel.hip.inc"
+namespace frisk {
+template __global__ void gemm_kernel<GemmCfg<FRISK_F16, 0, 1, 256, 256, 64, 2, 2, 2, false, false, 1, 3, 16>>(GemmParams);
+template __global__ void gemm_kernel<GemmCfg<FRISK_F16, 0, 0, 256, 256, 64, 2, 2, 2, false, true, 1, 3, 16>>(GemmParams);
+template __global__ void gemm_kernel<GemmCfg<FRISK_BF16, 1, 1, 256, 256, 64, 2, 2, 2, false, false, 1, 3, 16>>(GemmParams);
+template __global__ void gemm_kernel<GemmCfg<FRISK_I8, 1, 0, 256, 256, 128, 2, 2, 2, false, false, 1, 3, 16>>(GemmParams);
+}
+"""
+
+
+def _registers(text):
+    out = set()
+    for kind, lo, hi in re.findall(r"\b([av])\[(\d+):(\d+)\]", text):
+        out.update(kind + str(r) for r in range(int(lo), int(hi) + 1))
+    out.update(kind + n for kind, n in re.findall(r"\b([av])(\d+)\b", text))
+    return out
+
+
+def _operands(line):
+    parts = line.split(None, 1)
+    return parts[1].split(",") if len(parts) > 1 else []
+
+
+def hazards(listing, window_before=8, window_after=12):
+    found = []
+    for kernel in re.split(r"\n\t\.globl\t", listing)[1:]:
+        name = kernel.split("\n")[0]
+        lines = [l.strip() for l in kernel.split("\n") if l.startswith("\t") and not l.strip().startswith((".", ";"))]
+        for i, line in enumerate(lines):
+            if not line.startswith("v_mfma"):
+                continue
+            ops = _operands(line)
+            reads, result = _registers(",".join(ops)), _registers(ops[0])
+            for back in range(1, window_before + 1):
+                prev = lines[i - back] if i - back >= 0 else ""
+                if prev.startswith("v_") and not prev.startswith("v_mfma") and _registers((_operands(prev) or [""])[0]) & reads:
+                    found.append((name, prev, line))
+            for fwd in range(1, window_after + 1):
+                nxt = lines[i + fwd] if i + fwd < len(lines) else ""
+                if nxt.startswith("v_") and not nxt.startswith("v_mfma") and _registers(",".join(_operands(nxt)[1:])) & result:
+                    found.append((name, line, nxt))
+    return found
+
+
+def test_scanner_sees_both_patterns():
+    listing = "\n\t.globl\tk\nk:\n\tv_accvgpr_mov_b32 a5, a1\n\ts_nop 0\n\tv_mfma_f32_16x16x32_f16 a[4:7], v[0:3], v[4:7], a[4:7]\n\tv_accvgpr_read_b32 v9, a6\n"
+    got = hazards(listing)
+    assert len(got) == 2 and got[0][1].startswith("v_accvgpr_mov") and got[1][2].startswith("v_accvgpr_read")
+    clean = "\n\t.globl\tk\nk:\n\tv_mfma_f32_16x16x32_f16 a[4:7], v[0:3], v[4:7], a[4:7]\n\tv_mfma_f32_16x16x32_f16 a[8:11], v[0:3], v[4:7], a[8:11]\n"
+    assert hazards(clean) == []
+
+
+@pytest.mark.skipif(not (os.path.exists(HIPCC) or shutil.which("hipcc")), reason="needs hipcc to produce the ISA listing")
+def test_inline_assembly_mfma_kernels_keep_their_wait_states(tmp_path):
+    src = tmp_path / "atoms16.hip"
+    src.write_text(SOURCE)
+    out = tmp_path / "atoms16.s"
+    cmd = [HIPCC if os.path.exists(HIPCC) else "hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-Wno-unused-command-line-argument", "--cuda-device-only", "-S", str(src), "-o", str(out)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    listing = out.read_text()
+    assert listing.count("v_mfma_f32_16x16x32_f16") > 300 and "v_mfma_i32_16x16x64_i8" in listing and "v_mfma_f32_16x16x32_bf16" in listing
+    bad = hazards(listing)
+    assert not bad, "\n".join("%s: %s  ->  %s" % (n[:60], a, b) for n, a, b in bad[:10])

@@ -28,9 +28,11 @@ def test_config1_fp32_1024_built_through_the_builder(hip):
     assert h.module.verify()
     A = make_operand(O.F32, M, K, seed=0, tensor=0, kind="uniform")
     B = make_operand(O.F32, K, N, seed=0, tensor=1, kind="uniform")
-    got = _run(kernel, A, B, M, N, np.float32)
-    r = O.compare(O.F32, got, O.gemm_f64(O.F32, A, B))
-    assert r["nonfinite"] == 0 and r["max_rel"] <= 1e-4 and r["fro_rel"] <= 1e-4, r
+    ref = O.gemm_f64(O.F32, A, B)
+    for retile in (True, False):     # the planner's kernel for the whole problem, and the 128 x 128 x 32 tile the program is written with
+        got = _run(kernel, A, B, M, N, np.float32, retile=retile)
+        r = O.compare(O.F32, got, ref)
+        assert r["nonfinite"] == 0 and r["max_rel"] <= 1e-4 and r["fro_rel"] <= 1e-4, (retile, r)
     # the naive definition agrees on a window of rows
     ref_naive = O.gemm_naive(O.F32, np.ascontiguousarray(A[:16]), B)
     assert O.compare(O.F32, np.ascontiguousarray(got[:16]), ref_naive)["max_rel"] <= 1e-4
