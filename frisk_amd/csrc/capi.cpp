@@ -275,6 +275,10 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
       if (want_split && !k->splitk) continue;
       // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
       if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
+      // ... and address a tile's chunks by 32-bit lane offsets from its first row: the stored rows of one tile must span
+      // less than 4 GiB
+      const double span_a = (double)d->lda * es * (d->transA ? k->bk : k->bm), span_b = (double)d->ldb * es * (d->transB ? k->bn : k->bk);
+      if (!k->guard && (span_a >= 4294967296.0 || span_b >= 4294967296.0)) continue;
       if (k->guard && best >= 0 && !ks[best]->guard) continue;  // never a guarded kernel when a fast one fits
       const double cost = estimated_cost(k, d);
       // ties: the first listed variant is the tuned default
