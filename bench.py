@@ -158,8 +158,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs an MI355X"
     dev = torch.device("cuda:0")
     prop = torch.cuda.get_device_properties(0)
-    cus = prop.multi_processor_count
-    clock_khz = getattr(prop, "clock_rate", 0) or 0
+    info = HW.device_info()  # hipDeviceGetAttribute: torch's properties carry no clock on this build
+    cus, clock_khz = info["compute_units"], info["clock_khz"]
     stream = torch.cuda.current_stream()
     cs = stream.cuda_stream
     if a.copy_mib:
@@ -214,7 +214,9 @@ def main():
                      "kernel_ms_min": round(t16["min_ms"], 5)},
         "device": {"name": prop.name, "compute_units": cus, "clock_mhz_reported": round(clock_khz / 1e3, 1),
                    "peak_from_device_properties": {k: round(cus * clock_khz * 1e3 * v / 1e12, 1) for k, v in FLOPS_PER_CU_CLK.items()},
-                   "peak_nominal": PEAK_TFLOPS, "note": "CUs x reported clock x flops per CU and clock (4096 16-bit, 8192 8-bit, 256 fp32)"},
+                   "peak_nominal": PEAK_TFLOPS, "note": "CUs x reported clock x flops per CU and clock (4096 16-bit, 8192 8-bit, 256 fp32)",
+                   "memory_clock_mhz_reported": round(info["memory_clock_khz"] / 1e3, 1), "memory_bus_bits": info["memory_bus_bits"],
+                   "hbm_peak_from_device_properties_GBps": round(2.0 * info["memory_clock_khz"] * 1e3 * info["memory_bus_bits"] / 8 / 1e9, 1)},
     }
 
     if not a.only_headline:
@@ -314,6 +316,32 @@ def main():
                                            "kernel_ms_min": round(tsk["min_ms"], 5), "kernel": R.kernel_names()[pf.kernel_id], "split_k": pf.split_k,
                                            "workload": "fp8 e4m3 M=32 N=K=8192 NT, per-tensor scales, bf16 out (configs[4], decode part); algorithmic bytes "
                                                        "|A|+|B|+|C|+scales per launch, B rotating over 6 buffers"}
+        # what bounds this shape: the same kernel and grid with K shrunk to one K tile (the fixed cost of a launch: dispatch,
+        # the first tile's trip from HBM, the epilogue) and with K doubled; the slope between K and 2K is the rate at which the
+        # kernel streams B once it runs
+        kernel_bk = pf.tile_k
+
+        def skinny_at(k):
+            a_ = torch.randn(Ms, k, device=dev, generator=g).to(torch.float8_e4m3fn)
+            bs = [torch.randn(Ns, k, device=dev, generator=g).to(torch.float8_e4m3fn) for _ in range(max(2, (384 << 20) // (Ns * k)) if k >= Ks else 2)]
+            dk = R.make_desc(R.E4M3, Ms, Ns, k, dtype_out=R.BF16, transB=True, epilogue=R.EPI_TENSOR_SCALE, tile=(pf.tile_m, pf.tile_n, kernel_bk),
+                             stages=pf.stages_b, split_k=1)
+            wk = R.workspace_bytes(dk)
+            wsk = torch.empty(max(wk, 16), dtype=torch.uint8, device=dev)
+            turn_k = [0]
+
+            def fn():
+                b_ = bs[turn_k[0] % len(bs)]
+                turn_k[0] += 1
+                R.gemm(dk, a_.data_ptr(), b_.data_ptr(), Cf.data_ptr(), one.data_ptr(), one.data_ptr(), wsk.data_ptr() if wk else None, wk, cs)
+            return time_launches(torch, fn, a.steps, a.warmup, stream)["mean_ms"]
+        floor_ms, double_ms = skinny_at(kernel_bk), skinny_at(2 * Ks)
+        stream_gbs = (Ms + Ns) * Ks / ((double_ms - tsk["mean_ms"]) * 1e-3) / 1e9
+        legs["fp8_skinny_32x8192x8192"].update({
+            "launch_floor_ms": round(floor_ms, 5), "kernel_ms_at_2K": round(double_ms, 5), "streaming_GBps": round(stream_gbs, 1),
+            "frac_at_2K": round((Ms * 2 * Ks + Ns * 2 * Ks + 2 * Ms * Ns + 8) / (double_ms * 1e-3) / 8e12, 4),
+            "bound_note": "launch_floor_ms is this kernel and grid with K of one K tile; streaming_GBps the slope between K=8192 and K=16384; "
+                          "kernel_ms is close to launch_floor_ms + bytes / streaming rate"})
         del Bf
 
         # the dialect's data-movement ops on a 32768 x 8192 f16 view (512 MiB per array: twice the last-level cache)

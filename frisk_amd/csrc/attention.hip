@@ -80,12 +80,7 @@ template <> struct Pack16<FRISK_BF16> {
 // The final division by the denominator makes the result independent of the reference.
 constexpr float kAttnRescaleSlack = 8.f;
 
-#ifndef FRISK_ATTN_PRIO
-#define FRISK_ATTN_PRIO 0
-#endif
-#ifndef FRISK_ATTN_PREFETCH
-#define FRISK_ATTN_PREFETCH 4  // MFMA units between a fragment's LDS read and its use
-#endif
+constexpr int kAttnPrefetch = 4;  // MFMA units between a fragment's LDS read and its use
 
 template <class C>
 __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p) {
@@ -101,7 +96,6 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
   constexpr int N1 = DSTEPS * KA;   // MFMAs of the first product per tile
   constexpr int N2 = KSTEPS * DA;   // MFMAs of the second product per tile
   constexpr int NE = KA * 16;       // scores per lane per tile
-  static_assert(SK::NVOFF == 1 && SV::NVOFF == 1, "one lane offset per operand");
   static_assert(N1 == 16 && N2 == 16 && NE == 32, "the interleaving below is written for 64 keys x 128 head_dim");
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -133,16 +127,19 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
   const int64_t k_step = C::KT ? (int64_t)KB * 2 : (int64_t)KB * D * 2;
   const char* srcK = (const char*)p.K + (int64_t)bh * p.seq_k * D * 2 + SK::wave_src_offset(wave, k_ld);
   const char* srcV = (const char*)p.V + (int64_t)bh * p.seq_k * D * 2 + SV::wave_src_offset(wave, D * 2);
-  const unsigned voffK[1] = {SK::lane_src_offset(lane, wave, k_ld)};
-  const unsigned voffV[1] = {SV::lane_src_offset(lane, wave, D * 2)};
+  unsigned voffK[SK::PER_WAVE], voffV[SV::PER_WAVE];
+#pragma unroll
+  for (int i = 0; i < SK::PER_WAVE; ++i) voffK[i] = SK::transfer_src_offset(i, lane, wave, k_ld);
+#pragma unroll
+  for (int i = 0; i < SV::PER_WAVE; ++i) voffV[i] = SV::transfer_src_offset(i, lane, wave, D * 2);
   constexpr int PER_TILE = SK::PER_WAVE + SV::PER_WAVE;
   int k_slot_issue = 0, v_slot_issue = 0;
   auto stage_tile = [&]() {
-    const unsigned kdst = k_ring + k_slot_issue * LK::BYTES, vdst = v_ring + v_slot_issue * LV::BYTES;
+    const unsigned kdst = k_ring + k_slot_issue * LK::BYTES + (unsigned)wave * 1024u, vdst = v_ring + v_slot_issue * LV::BYTES + (unsigned)wave * 1024u;
 #pragma unroll
-    for (int i = 0; i < SK::PER_WAVE; ++i) SK::issue_one(i, srcK, voffK, k_ld, kdst, wave);
+    for (int i = 0; i < SK::PER_WAVE; ++i) SK::issue_one(i, srcK, voffK, kdst);
 #pragma unroll
-    for (int i = 0; i < SV::PER_WAVE; ++i) SV::issue_one(i, srcV, voffV, D * 2, vdst, wave);
+    for (int i = 0; i < SV::PER_WAVE; ++i) SV::issue_one(i, srcV, voffV, vdst);
     srcK += k_step;
     srcV += (int64_t)KB * D * 2;
     k_slot_issue = k_slot_issue == C::NSK - 1 ? 0 : k_slot_issue + 1;
@@ -179,17 +176,10 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
 #pragma unroll
     for (int r = 0; r < RK::NREG; ++r) ck[r] = rk[r] + kbase;
     // fragment of unit x (0 .. N2-1: V, N2 .. N2+N1-1: K) goes to f[x % NB], read PF units ahead of its MFMA
-    constexpr int PF = FRISK_ATTN_PREFETCH, NB = PF + 1;
-#ifdef FRISK_ATTN_ABLATE_LDS
-    int f[NB][4] = {};
-#else
+    constexpr int PF = kAttnPrefetch, NB = PF + 1;
     int f[NB][4];
-#endif
     const int last = scores ? N2 + N1 : N2;
     auto fetch = [&](int x) {
-#ifdef FRISK_ATTN_ABLATE_LDS
-      if (nkt > 0) return;  // development aid: fragments are never read
-#endif
       if (x < N2) v_read(vbase, x, f[x % NB]);
       else if (x < last) k_read(ck, x - N2, f[x % NB]);
     };
@@ -198,9 +188,6 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
 #pragma unroll
     for (int u = 0; u < N2; ++u) {
       const v4i vfrag = {f[u % NB][0], f[u % NB][1], f[u % NB][2], f[u % NB][3]};
-#ifdef FRISK_ATTN_ABLATE_MFMA
-      if (nkt < 0)
-#endif
       M::run(vfrag, pf[u / DA], o[u % DA]);
       fetch(u + PF);
       __builtin_amdgcn_sched_barrier(0);
@@ -211,9 +198,6 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
         const int x = u + N2;
         const v4i kfrag = {f[x % NB][0], f[x % NB][1], f[x % NB][2], f[x % NB][3]};
         if (u < KA) s[u % KA] = v16f{};  // folds into the MFMA's C operand: no registers are cleared
-#ifdef FRISK_ATTN_ABLATE_MFMA
-        if (nkt < 0)
-#endif
         M::run(kfrag, qf[u / KA], s[u % KA]);
         fetch(x + PF);
         __builtin_amdgcn_sched_barrier(0);
@@ -223,15 +207,6 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
   // V phase: probabilities of the tile whose scores are in s.  Score e of the lane, e = 16 ka + r, belongs to
   // 16-key step e / 8.
   auto v_phase = [&]() {
-#ifdef FRISK_ATTN_ABLATE_VALU
-    if (nkt > 0) {  // development aid: no softmax work at all
-#pragma unroll
-      for (int t = 0; t < KSTEPS; ++t)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(pf[t][j]));
-      return;
-    }
-#endif
     float mx = s[0][0];
 #pragma unroll
     for (int ka = 0; ka < KA; ++ka)
@@ -258,12 +233,8 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
     float l_part[4] = {l_run, 0.f, 0.f, 0.f};  // four chains instead of one of 16 dependent additions
 #pragma unroll
     for (int e = 0; e < NE; e += 2) {
-#ifdef FRISK_ATTN_ABLATE_EXP
-      const float x0 = __builtin_fmaf(s[e / 16][e % 16], c, -m_run), x1 = __builtin_fmaf(s[e / 16][e % 16 + 1], c, -m_run);
-#else
       const float x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e / 16][e % 16], c, -m_run));
       const float x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e / 16][e % 16 + 1], c, -m_run));
-#endif
       const int pair = PK::two(x0, x1);
       pf[e / 8][(e % 8) / 2] = pair;
       l_part[(e / 2) % 4] = PK::add_pair(pair, l_part[(e / 2) % 4]);
@@ -307,64 +278,25 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
   // the end).  Before either barrier of iteration kt a wave's share of tile kt+1 has landed (at most tile kt+2 is
   // outstanding), so tile kt+1 is complete in LDS before any wave's M(kt); when a wave stages tile kt+3, every wave
   // has passed the barrier that follows its M(kt-1), the last reader of K tile kt and V tile kt-1.
-#ifdef FRISK_ATTN_GROUP_ODD
-  const bool trails = (wave & 1) != 0;
-#elif defined(FRISK_ATTN_GROUP_NONE)
-  const bool trails = false;
-#else
   const bool trails = wave >= C::NW / 2;
-#endif
   if (trails) __builtin_amdgcn_s_barrier();
   int k_slot = 1, v_slot = 0;  // ring slots M(kt) reads: K tile kt+1 and V tile kt
-#ifdef FRISK_ATTN_PROBE
-  unsigned long long pt[5] = {0, 0, 0, 0, 0};
-  const unsigned long long pt_start = __builtin_amdgcn_s_memtime(), pr_start = __builtin_amdgcn_s_memrealtime();
-#define PROBE(i) { const unsigned long long now = __builtin_amdgcn_s_memtime(); pt[i] += now - pt_last; pt_last = now; }
-  unsigned long long pt_last = pt_start;
-#else
-#define PROBE(i)
-#endif
   for (int kt = 0; kt < nkt; ++kt) {
     if (kt + 2 < nkt) wait_vmcnt<PER_TILE>(); else wait_vmcnt<0>();
-    PROBE(0)
     __builtin_amdgcn_s_barrier();
-    PROBE(1)
     __builtin_amdgcn_sched_barrier(0);  // the phases are register-only work: without these the compiler moves it across the barriers
-#if FRISK_ATTN_PRIO == 1
-    __builtin_amdgcn_s_setprio(3);
-#endif
     v_phase();
-#if FRISK_ATTN_PRIO == 1
-    __builtin_amdgcn_s_setprio(0);
-#endif
     __builtin_amdgcn_sched_barrier(0);
-    PROBE(2)
     if (kt + 2 < nkt) wait_vmcnt<PER_TILE>(); else wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    PROBE(3)
     if (kt + 3 < nkt) stage_tile();
-#if FRISK_ATTN_PRIO == 2
-    __builtin_amdgcn_s_setprio(3);
-#endif
     m_phase(v_ring + v_slot * LV::BYTES, k_ring + k_slot * LK::BYTES, kt + 1 < nkt);
-#if FRISK_ATTN_PRIO == 2
-    __builtin_amdgcn_s_setprio(0);
-#endif
     __builtin_amdgcn_sched_barrier(0);
-    PROBE(4)
     k_slot = k_slot == C::NSK - 1 ? 0 : k_slot + 1;
     v_slot = v_slot == C::NSV - 1 ? 0 : v_slot + 1;
   }
   if (!trails) __builtin_amdgcn_s_barrier();
-#ifdef FRISK_ATTN_PROBE
-  if (p.lse && lane == 0 && blockIdx.x == 8) {  // development aid: shader clocks per phase, summed over the tiles
-    unsigned long long* dbg = (unsigned long long*)p.lse + 8 * wave;
-    for (int i = 0; i < 5; ++i) dbg[i] = pt[i];
-    dbg[5] = __builtin_amdgcn_s_memtime() - pt_start;
-    dbg[6] = __builtin_amdgcn_s_memrealtime() - pr_start;
-  }
-#endif
 
   // O = O^T / l.  Lane (q, h) holds head_dim columns 32 da + 8 (r/4) + 4 h + r%4 of its query: 8-byte pieces.  They
   // go through a wave-private LDS region (64 columns at a time, rows padded by 16 B) and come back as 16-byte
@@ -396,9 +328,7 @@ __global__ void __launch_bounds__(C::NW * 64) attention_kernel(AttentionParams p
         FRISK_STORE_C((v4i*)(obase + (int64_t)orow * D * 2 + (64 * half + 8 * chunk) * 2), w);
       }
     }
-#ifndef FRISK_ATTN_PROBE
     if (p.lse && lh == 0) p.lse[row] = (m_run + __builtin_amdgcn_logf(l)) * 0.6931471805599453f;
-#endif
   }
 }
 

@@ -391,4 +391,23 @@ double frisk_hwcheck_mfma_loop_cycles(int kind, int iters) {
   }
 }
 
+// What the driver reports for the current device: compute units, shader clock and memory clock in kHz, memory bus width in
+// bits.  The nominal peaks are priced at 256 CUs x 2.4 GHz and 8 TB/s; this is the figure to hold against them.  Returns a
+// hipError_t.
+int frisk_hwcheck_device_info(int* compute_units, int* clock_khz, int* memory_clock_khz, int* memory_bus_bits) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  struct { hipDeviceAttribute_t attr; int* out; } want[] = {{hipDeviceAttributeMultiprocessorCount, compute_units},
+                                                            {hipDeviceAttributeClockRate, clock_khz},
+                                                            {hipDeviceAttributeMemoryClockRate, memory_clock_khz},
+                                                            {hipDeviceAttributeMemoryBusWidth, memory_bus_bits}};
+  for (auto& w : want) {
+    if (!w.out) continue;
+    e = hipDeviceGetAttribute(w.out, w.attr, dev);
+    if (e != hipSuccess) return (int)e;
+  }
+  return 0;
+}
+
 }  // extern "C"

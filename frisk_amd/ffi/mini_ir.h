@@ -12,6 +12,7 @@
 // (:901-920 kernel, :1264-1283 gemm, :1436-1481 alloc_buffer, :1666-1683 copy,
 // :1688-1701 fill, :1725-1767 reduce) are restated here over plain structs.
 #pragma once
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -1114,12 +1115,17 @@ inline GemmProgram match_tiled_gemm(Operation* kernel, Operation* module = nullp
 }
 
 // ------------------------------------------------------------------ data-movement programs
-// What the runtime extracts from a kernel whose entry block is a straight line of
-//   frisk.fill %arg            frisk.copy %arg[const map], %arg[const map] {src_extents, dst_extents}
+// What the runtime extracts from a kernel made of
+//   frisk.fill %arg            frisk.copy %a[map(indices)], %b[map(indices)] {src_extents, dst_extents}
 //   frisk.reduce %arg, %arg {kind, dim, clear}
-// on kernel arguments of rank 1 or 2 (global memrefs): one entry per op, in program order.  Window origins come from
-// index maps without inputs (constant results); extents follow the op (default: the destination shape left-padded
-// with 1s, FriskOps.cpp:1564-1591).
+// on kernel arguments of rank 1 or 2 (global memrefs): one entry per op, in program order.  A copy's window origin is its
+// index map applied to its index operands; extents follow the op (default: the destination shape left-padded with 1s,
+// FriskOps.cpp:1564-1591).  Copies may sit under frisk.parallel and frisk.for and be indexed by their grid indices and
+// induction variables: the windows of all iterations must then tile one rectangle of each side without gaps or overlap
+// (every index moves the window by whole tiles along one dimension, the same one on both sides), and the copy is lowered
+// as one copy of that rectangle.  A tile may also pass through one frisk.alloc_buffer (global -> buffer -> global in
+// the same block, the buffer used by nothing else): the pair is lowered as the direct copy.  Fill and reduce take whole
+// arguments and must not be repeated by an enclosing grid or loop.
 struct TileOpDesc {
   enum Kind { Fill, Copy, Reduce } kind = Fill;
   int arg_src = -1, arg_dst = -1;          // kernel argument positions (fill: arg_dst only)
@@ -1132,77 +1138,233 @@ struct TileOpDesc {
   bool clear = true;
 };
 
+// an index a copy may use: value lower + step * i for i in [0, count)
+struct IndexRange {
+  Value value;
+  int64_t lower = 0, step = 1, count = 1;
+};
+
+// Window origin of one side of a frisk.copy as a linear function of the iteration numbers i_v of `vars`:
+// origin[r] = c0[r] + sum_v stride[r][v] * i_v.  Every index operand must be one of `vars`.
+struct TiledOrigin {
+  std::vector<int64_t> c0;
+  std::vector<std::vector<int64_t>> stride;  // [result][var]
+};
+
+inline TiledOrigin tiled_origin(const Operation* cp, bool dst_side, const std::vector<IndexRange>& vars, const std::function<void(const std::string&)>& bad) {
+  const AffineMap& map = cp->attr(dst_side ? "dstMap" : "srcMap")->map;
+  const int ns = cp->src_index_count, first = dst_side ? 2 + ns : 2;
+  const int count = dst_side ? (int)cp->operands.size() - 2 - ns : ns;
+  if (count != map.num_inputs()) bad("a copy's index operands do not match its index map");
+  std::vector<int> which((size_t)count, -1);
+  for (int i = 0; i < count; ++i) {
+    for (size_t v = 0; v < vars.size(); ++v) if (cp->operands[(size_t)(first + i)] == vars[v].value) which[(size_t)i] = (int)v;
+    if (which[(size_t)i] < 0) bad("a copy is indexed by a value that is neither a grid index nor an enclosing loop's induction variable");
+  }
+  auto at = [&](const std::vector<int64_t>& iter) {  // origin at iteration numbers `iter`
+    std::vector<int64_t> dims, syms;
+    for (int i = 0; i < count; ++i) {
+      const IndexRange& r = vars[(size_t)which[(size_t)i]];
+      (i < map.num_dims() ? dims : syms).push_back(r.lower + r.step * iter[(size_t)which[(size_t)i]]);
+    }
+    std::vector<int64_t> out;
+    for (int r = 0; r < map.num_results(); ++r) out.push_back(map.impl->results[(size_t)r].eval(dims, syms));
+    return out;
+  };
+  TiledOrigin o;
+  std::vector<int64_t> zero(vars.size(), 0), probe(vars.size());
+  o.c0 = at(zero);
+  o.stride.assign(o.c0.size(), std::vector<int64_t>(vars.size(), 0));
+  for (size_t v = 0; v < vars.size(); ++v) {
+    std::vector<int64_t> unit = zero;
+    unit[v] = 1;
+    const std::vector<int64_t> r = at(unit);
+    for (size_t k = 0; k < r.size(); ++k) o.stride[k][v] = r[k] - o.c0[k];
+    probe[v] = (int64_t)(2 * v + 3);
+  }
+  const std::vector<int64_t> r = at(probe);
+  for (size_t k = 0; k < r.size(); ++k) {
+    int64_t want = o.c0[k];
+    for (size_t v = 0; v < vars.size(); ++v) want += o.stride[k][v] * probe[v];
+    if (r[k] != want) bad("a copy's index map is not linear in its indices");
+  }
+  return o;
+}
+
 inline std::vector<TileOpDesc> match_data_movement(Operation* kernel) {
   auto bad = [](const std::string& m) -> std::vector<TileOpDesc> { throw std::invalid_argument("not a data-movement kernel: " + m); };
+  const std::function<void(const std::string&)> fail = [](const std::string& m) { throw std::invalid_argument("not a data-movement kernel: " + m); };
   if (!kernel || kernel->name != "frisk.kernel") return bad("expected a frisk.kernel");
   if (kernel->regions.empty() || kernel->regions[0]->blocks.empty()) return bad("kernel has no entry block");
   Block* entry = kernel->regions[0]->blocks[0];
-  struct View { int arg; Type elem; int64_t rows, cols; };
+  struct View { int arg; Type elem; int64_t rows, cols; size_t rank; };
   auto view_of = [&](Value v, const char* what) -> View {
     int a = kernel_arg_index(kernel, v);
-    if (a < 0 || !v.type().is_memref()) throw std::invalid_argument(std::string("not a data-movement kernel: ") + what + " is not a kernel argument memref");
+    if (a < 0 || !v.type().is_memref()) fail(std::string(what) + " is not a kernel argument memref");
     const auto& sh = v.type().impl->shape;
-    if (sh.empty() || sh.size() > 2) throw std::invalid_argument(std::string("not a data-movement kernel: ") + what + " must have rank 1 or 2");
-    for (int64_t d : sh) if (d < 0) throw std::invalid_argument(std::string("not a data-movement kernel: ") + what + " has a dynamic extent");
-    return View{a, v.type().element(), sh.size() == 2 ? sh[0] : 1, sh.back()};
+    if (sh.empty() || sh.size() > 2) fail(std::string(what) + " must have rank 1 or 2");
+    for (int64_t d : sh) if (d < 0) fail(std::string(what) + " has a dynamic extent");
+    return View{a, v.type().element(), sh.size() == 2 ? sh[0] : 1, sh.back(), sh.size()};
   };
-  // window (origin, extents) of a copy operand -> (element offset, rows, cols) inside its view
-  auto window_of = [&](const View& v, size_t rank, const AffineMap& map, const std::vector<int64_t>& ext, const char* what, int64_t& off, int64_t& r, int64_t& c) {
-    if (map.num_inputs() != 0) throw std::invalid_argument(std::string("not a data-movement kernel: the ") + what + " map of a copy must have constant results (no index operands)");
-    if ((size_t)map.num_results() != rank) throw std::invalid_argument(std::string("not a data-movement kernel: the ") + what + " map must give one origin per dimension");
-    std::vector<int64_t> org;
-    for (int i = 0; i < map.num_results(); ++i) {
-      const AffineExpr& e = map.impl->results[(size_t)i];
-      if (!e.is_constant()) throw std::invalid_argument(std::string("not a data-movement kernel: the ") + what + " origin is not constant");
-      org.push_back(e.constant_value());
-    }
+  // One side of a copy: the rectangle (r0, c0, rows, cols) that the windows of all iterations cover, in the side's last two
+  // dimensions, the tile (tr, tc) one iteration moves, and per index the (dimension from the end, stride) it moves the tile by.
+  struct Side { int64_t r0 = 0, c0 = 0, rows = 1, cols = 1, tr = 1, tc = 1; std::vector<std::pair<int, int64_t>> moves; };
+  auto side_of = [&](const Operation* cp, bool dst_side, size_t rank, const std::vector<IndexRange>& vars, const char* what) -> Side {
+    const TiledOrigin o = tiled_origin(cp, dst_side, vars, fail);
+    const auto& ext = cp->attr(dst_side ? "dstExtents" : "srcExtents")->ints;
+    if (o.c0.size() != rank) fail(std::string("the ") + what + " map must give one origin per dimension");
     // extents may carry leading 1s (source rank > destination rank): the window is their last `rank` entries
-    if (ext.size() < rank) throw std::invalid_argument(std::string("not a data-movement kernel: too few ") + what + " extents");
-    for (size_t i = 0; i + rank < ext.size(); ++i) if (ext[i] != 1) throw std::invalid_argument(std::string("not a data-movement kernel: leading ") + what + " extents must be 1");
-    std::vector<int64_t> e(ext.end() - (long)rank, ext.end());
-    int64_t r0 = rank == 2 ? org[0] : 0, c0 = org.back();
-    r = rank == 2 ? e[0] : 1;
-    c = e.back();
-    if (r0 < 0 || c0 < 0 || r < 0 || c < 0 || r0 + r > v.rows || c0 + c > v.cols) throw std::invalid_argument(std::string("not a data-movement kernel: the ") + what + " window leaves the memref");
-    off = r0 * v.cols + c0;
-  };
-  std::vector<TileOpDesc> out;
-  for (Operation* op : entry->ops) {
-    TileOpDesc d;
-    if (op->name == "frisk.end") continue;
-    if (op->name == "frisk.fill") {
-      View v = view_of(op->operands[0], "the fill target");
-      d.kind = TileOpDesc::Fill;
-      d.arg_dst = v.arg; d.elem_dst = v.elem; d.rows = v.rows; d.cols = v.cols; d.dst_ld = v.cols;
-      d.value = op->attr("value")->f;
-    } else if (op->name == "frisk.copy") {
-      View s = view_of(op->operands[0], "the copy source"), t = view_of(op->operands[1], "the copy destination");
-      d.kind = TileOpDesc::Copy;
-      d.arg_src = s.arg; d.arg_dst = t.arg; d.elem_src = s.elem; d.elem_dst = t.elem; d.src_ld = s.cols; d.dst_ld = t.cols;
-      int64_t sr, sc, tr, tc;
-      window_of(s, op->operands[0].type().impl->shape.size(), op->attr("srcMap")->map, op->attr("srcExtents")->ints, "source", d.src_offset, sr, sc);
-      window_of(t, op->operands[1].type().impl->shape.size(), op->attr("dstMap")->map, op->attr("dstExtents")->ints, "destination", d.dst_offset, tr, tc);
-      if (sr * sc != tr * tc) return bad("source and destination windows of a copy hold different numbers of elements");
-      if (sr == tr && sc == tc) { d.rows = sr; d.cols = sc; }
-      else if (sr == 1 && tr == 1) { d.rows = 1; d.cols = sc; }
-      else if ((sr == 1 || tr == 1) && (sc == s.cols || sr == 1) && (tc == t.cols || tr == 1)) { d.rows = 1; d.cols = sr * sc; d.src_ld = d.dst_ld = d.cols; }  // a dense window against a row
-      else return bad("source and destination windows of a copy have different shapes");
-    } else if (op->name == "frisk.reduce") {
-      View s = view_of(op->operands[0], "the reduce source"), t = view_of(op->operands[1], "the reduce destination");
-      if (op->operands[0].type().impl->shape.size() != 2) return bad("the reduce source must have rank 2");
-      d.kind = TileOpDesc::Reduce;
-      d.arg_src = s.arg; d.arg_dst = t.arg; d.elem_src = s.elem; d.elem_dst = t.elem; d.rows = s.rows; d.cols = s.cols; d.src_ld = s.cols;
-      d.dim = op->int_attr("dim");
-      d.reduce_kind = op->attr("kind")->s == "sum" ? "add" : op->attr("kind")->s;
-      d.clear = op->attr("clear")->b;
-      if (d.dim != 0 && d.dim != 1) return bad("reduce dimension out of range");
-      if (t.rows * t.cols != (d.dim == 1 ? s.rows : s.cols)) return bad("the reduce destination does not hold one element per kept index");
-      if (!s.elem.equals(t.elem)) return bad("reduce source and destination element types differ");
-    } else {
-      return bad("operation " + op->name + " is not fill, copy or reduce");
+    if (ext.size() < rank) fail(std::string("too few ") + what + " extents");
+    for (size_t i = 0; i + rank < ext.size(); ++i) if (ext[i] != 1) fail(std::string("leading ") + what + " extents must be 1");
+    Side sd;
+    sd.moves.assign(vars.size(), {-1, 0});
+    for (size_t r = 0; r < rank; ++r) {
+      const int from_end = (int)(rank - 1 - r);
+      int64_t tile = ext[ext.size() - rank + r], cover = tile;
+      if (tile <= 0) fail(std::string("a ") + what + " extent is not positive");
+      std::vector<std::pair<int64_t, size_t>> movers;  // (stride, var)
+      for (size_t v = 0; v < vars.size(); ++v) {
+        if (vars[v].count <= 1 || o.stride[r][v] == 0) continue;
+        if (sd.moves[v].first >= 0) fail(std::string("an index moves the ") + what + " window along two dimensions");
+        if (o.stride[r][v] < 0) fail(std::string("an index moves the ") + what + " window backwards");
+        sd.moves[v] = {from_end, o.stride[r][v]};
+        movers.push_back({o.stride[r][v], v});
+      }
+      std::sort(movers.begin(), movers.end());
+      for (const auto& mv : movers) {
+        if (mv.first != cover) fail(std::string("the ") + what + " windows of the iterations do not tile a rectangle (stride " + std::to_string(mv.first) + " where " + std::to_string(cover) + " would continue it)");
+        cover *= vars[mv.second].count;
+      }
+      if (from_end == 0) { sd.c0 = o.c0[r]; sd.cols = cover; sd.tc = tile; } else { sd.r0 = o.c0[r]; sd.rows = cover; sd.tr = tile; }
     }
-    out.push_back(d);
-  }
+    return sd;
+  };
+  auto check_inside = [&](const Side& sd, const View& v, const char* what) {
+    if (sd.r0 < 0 || sd.c0 < 0 || sd.r0 + sd.rows > v.rows || sd.c0 + sd.cols > v.cols) fail(std::string("the ") + what + " window leaves the memref");
+  };
+  auto uses_of = [&](Value buf) {
+    int n = 0;
+    std::function<void(Block*)> walk = [&](Block* b) {
+      for (Operation* op : b->ops) {
+        for (const Value& v : op->operands) if (v == buf) ++n;
+        for (Region* r : op->regions) for (Block* inner : r->blocks) walk(inner);
+      }
+    };
+    walk(entry);
+    return n;
+  };
+
+  std::vector<TileOpDesc> out;
+  std::vector<IndexRange> vars;
+  struct Staged { Value buffer; Operation* load; Block* block; };
+  std::function<void(Block*)> walk = [&](Block* block) {
+    std::vector<Staged> staged;  // tiles loaded into a buffer in this block and not yet stored
+    for (Operation* op : block->ops) {
+      TileOpDesc d;
+      if (op->name == "frisk.end" || op->name == "frisk.alloc_buffer") continue;
+      if (op->name == "frisk.parallel" || op->name == "frisk.for") {
+        if (!staged.empty()) fail("a tile staged in a buffer must be stored in the block that loaded it");
+        if (op->regions.empty() || op->regions[0]->blocks.empty()) fail(op->name + " has no body");
+        Block* body = op->regions[0]->blocks[0];
+        const size_t depth = vars.size();
+        if (op->name == "frisk.parallel") {
+          const auto& ranges = op->attr("ranges")->ints;
+          for (size_t i = 0; i < ranges.size(); ++i) vars.push_back(IndexRange{Value{body->args[i]}, 0, 1, ranges[i]});
+        } else {
+          const int64_t lo = op->int_attr("lower"), hi = op->int_attr("upper"), step = op->int_attr("step");
+          if (hi <= lo) fail("a frisk.for runs no iteration");
+          vars.push_back(IndexRange{Value{body->args[0]}, lo, step, (hi - lo + step - 1) / step});
+        }
+        walk(body);
+        vars.resize(depth);
+        continue;
+      }
+      bool repeated = false;
+      for (const IndexRange& r : vars) repeated = repeated || r.count > 1;
+      if (op->name == "frisk.fill") {
+        if (repeated) fail("a fill under a grid or a loop would run once per iteration");
+        View v = view_of(op->operands[0], "the fill target");
+        d.kind = TileOpDesc::Fill;
+        d.arg_dst = v.arg; d.elem_dst = v.elem; d.rows = v.rows; d.cols = v.cols; d.dst_ld = v.cols;
+        d.value = op->attr("value")->f;
+      } else if (op->name == "frisk.copy") {
+        Operation* load = op;  // the op whose source side is the global source
+        const Value src_v = op->operands[0], dst_v = op->operands[1];
+        const bool src_is_arg = kernel_arg_index(kernel, src_v) >= 0, dst_is_arg = kernel_arg_index(kernel, dst_v) >= 0;
+        auto whole_buffer = [&](const Operation* cp, bool dst_side, Value buf) {
+          const TiledOrigin o = tiled_origin(cp, dst_side, vars, fail);
+          for (size_t r = 0; r < o.c0.size(); ++r) {
+            if (o.c0[r] != 0) fail("the buffer side of a staged copy must start at 0");
+            for (size_t v = 0; v < vars.size(); ++v) if (o.stride[r][v] != 0 && vars[v].count > 1) fail("the buffer side of a staged copy must not move");
+          }
+          const auto& sh = buf.type().impl->shape;
+          const auto& ext = cp->attr(dst_side ? "dstExtents" : "srcExtents")->ints;
+          if (ext.size() < sh.size()) fail("too few extents on the buffer side of a staged copy");
+          for (size_t i = 0; i + sh.size() < ext.size(); ++i) if (ext[i] != 1) fail("leading extents on the buffer side of a staged copy must be 1");
+          for (size_t i = 0; i < sh.size(); ++i) if (ext[ext.size() - sh.size() + i] != sh[i]) fail("a staged copy must move the whole buffer");
+        };
+        if (src_is_arg && !dst_is_arg) {  // global -> buffer: remember it, the store completes it
+          if (!dst_v.impl || !dst_v.impl->def || dst_v.impl->def->name != "frisk.alloc_buffer") fail("a copy's destination is neither a kernel argument nor a frisk.alloc_buffer");
+          if (uses_of(dst_v) != 2) fail("a staging buffer must be used by exactly one load and one store");
+          whole_buffer(op, true, dst_v);
+          staged.push_back(Staged{dst_v, op, block});
+          continue;
+        }
+        if (!src_is_arg) {  // buffer -> global: complete the staged copy
+          if (!dst_is_arg) fail("a copy moves between two buffers");
+          size_t at = staged.size();
+          for (size_t i = 0; i < staged.size(); ++i) if (staged[i].buffer == src_v) at = i;
+          if (at == staged.size()) fail("a copy stores a buffer that no copy in the same block has loaded");
+          whole_buffer(op, false, src_v);
+          load = staged[at].load;
+          staged.erase(staged.begin() + (long)at);
+          const Type via = src_v.type().element();
+          if (!via.equals(load->operands[0].type().element()) && !via.equals(dst_v.type().element())) fail("a staging buffer's element type is neither the source's nor the destination's");
+        }
+        View s = view_of(load->operands[0], "the copy source"), t = view_of(dst_v, "the copy destination");
+        d.kind = TileOpDesc::Copy;
+        d.arg_src = s.arg; d.arg_dst = t.arg; d.elem_src = s.elem; d.elem_dst = t.elem; d.src_ld = s.cols; d.dst_ld = t.cols;
+        const Side ss = side_of(load, false, s.rank, vars, "source"), ts = side_of(op, true, t.rank, vars, "destination");
+        check_inside(ss, s, "source");
+        check_inside(ts, t, "destination");
+        d.src_offset = ss.r0 * s.cols + ss.c0;
+        d.dst_offset = ts.r0 * t.cols + ts.c0;
+        if (!repeated) {
+          // one window on each side: equal shapes, or a dense window against a row
+          if (ss.rows * ss.cols != ts.rows * ts.cols) fail("source and destination windows of a copy hold different numbers of elements");
+          if (ss.rows == ts.rows && ss.cols == ts.cols) { d.rows = ss.rows; d.cols = ss.cols; }
+          else if (ss.rows == 1 && ts.rows == 1) { d.rows = 1; d.cols = ss.cols; }
+          else if ((ss.rows == 1 || ts.rows == 1) && (ss.cols == s.cols || ss.rows == 1) && (ts.cols == t.cols || ts.rows == 1)) { d.rows = 1; d.cols = ss.rows * ss.cols; d.src_ld = d.dst_ld = d.cols; }
+          else fail("source and destination windows of a copy have different shapes");
+        } else {
+          if (ss.tr != ts.tr || ss.tc != ts.tc) fail("source and destination tiles of a tiled copy have different shapes");
+          for (size_t v = 0; v < vars.size(); ++v) {
+            if (vars[v].count <= 1) continue;
+            if (ss.moves[v].first < 0 || ts.moves[v].first < 0) fail("an enclosing grid index or induction variable does not move both windows of a copy: its iterations would repeat or overwrite one another");
+            if (ss.moves[v] != ts.moves[v]) fail("an index moves the source and destination windows of a tiled copy differently");
+          }
+          d.rows = ss.rows; d.cols = ss.cols;  // equal on both sides by the checks above
+        }
+      } else if (op->name == "frisk.reduce") {
+        if (repeated) fail("a reduce under a grid or a loop would run once per iteration");
+        View s = view_of(op->operands[0], "the reduce source"), t = view_of(op->operands[1], "the reduce destination");
+        if (op->operands[0].type().impl->shape.size() != 2) fail("the reduce source must have rank 2");
+        d.kind = TileOpDesc::Reduce;
+        d.arg_src = s.arg; d.arg_dst = t.arg; d.elem_src = s.elem; d.elem_dst = t.elem; d.rows = s.rows; d.cols = s.cols; d.src_ld = s.cols;
+        d.dim = op->int_attr("dim");
+        d.reduce_kind = op->attr("kind")->s == "sum" ? "add" : op->attr("kind")->s;
+        d.clear = op->attr("clear")->b;
+        if (d.dim != 0 && d.dim != 1) fail("reduce dimension out of range");
+        if (t.rows * t.cols != (d.dim == 1 ? s.rows : s.cols)) fail("the reduce destination does not hold one element per kept index");
+        if (!s.elem.equals(t.elem)) fail("reduce source and destination element types differ");
+      } else {
+        fail("operation " + op->name + " is not fill, copy or reduce");
+      }
+      out.push_back(d);
+    }
+    if (!staged.empty()) fail("a tile is loaded into a buffer and never stored");
+  };
+  walk(entry);
   if (out.empty()) return bad("the kernel holds no fill, copy or reduce");
   return out;
 }

@@ -18,7 +18,7 @@ LOOP_KINDS = {0: ("f16 32x32x16", "f16"), 1: ("f16 16x16x32", "f16"), 2: ("bf16 
 
 _lib = None
 EXPORTS = ["frisk_hwcheck_mfma_atom", "frisk_hwcheck_fragment_path", "frisk_hwcheck_tr_read", "frisk_hwcheck_mfma_loop",
-           "frisk_hwcheck_mfma_loop_flops", "frisk_hwcheck_mfma_loop_cycles"]
+           "frisk_hwcheck_mfma_loop_flops", "frisk_hwcheck_mfma_loop_cycles", "frisk_hwcheck_device_info"]
 
 
 def lib():
@@ -36,6 +36,7 @@ def lib():
         L.frisk_hwcheck_mfma_loop_flops.restype = ctypes.c_double
         L.frisk_hwcheck_mfma_loop_cycles.argtypes = [i, i]
         L.frisk_hwcheck_mfma_loop_cycles.restype = ctypes.c_double
+        L.frisk_hwcheck_device_info.argtypes = [ctypes.POINTER(i)] * 4
         _lib = L
     return _lib
 
@@ -68,3 +69,10 @@ def mfma_loop_flops(kind, iters, workgroups):
 def mfma_loop_cycles(kind, iters):
     """matrix-pipe cycles one wave of the loop needs at full issue rate"""
     return float(lib().frisk_hwcheck_mfma_loop_cycles(kind, iters))
+
+
+def device_info():
+    """what the driver reports for the current device: {"compute_units", "clock_khz", "memory_clock_khz", "memory_bus_bits"}"""
+    vals = [ctypes.c_int(0) for _ in range(4)]
+    _check(lib().frisk_hwcheck_device_info(*[ctypes.byref(v) for v in vals]), "device_info")
+    return dict(zip(("compute_units", "clock_khz", "memory_clock_khz", "memory_bus_bits"), (v.value for v in vals)))

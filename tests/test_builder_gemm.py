@@ -318,3 +318,95 @@ def test_data_movement_kernel_is_recognised_op_by_op():
     with pytest.raises(ValueError) as e:
         F.runtime.match_ops(k2)
     assert "window leaves the memref" in str(e.value)
+
+
+def _tiled_copy_kernel(h, *, staged=True, dst_origin=(16, 64), src_tile_step=None, dst_scale=(32, 64), rows=128, cols=256, loop=True):
+    """kernel(x: rows x cols f32, y: (rows+32) x (cols+64) f16): y[16 + i, 64 + j] := f16(x[i, j]), written tile by tile: a grid over
+    32-row bands, a loop over 64-column tiles, every 32 x 64 tile through a shared buffer (or directly)"""
+    b = h.builder
+    x_t, y_t = h.memref_type((rows, cols), "fp32"), h.memref_type((rows + 32, cols + 64), "fp16")
+    kernel, entry = h.new_kernel("tiled_copy", [x_t, y_t])
+    x, y = entry.get_argument(0), entry.get_argument(1)
+    body = b.create_parallel_op([rows // 32], 256).add_entry_block()
+    b.set_insertion_point_to_start(body)
+    by = body.get_argument(0)
+    tile = h.alloc_buffer((32, 64), "fp32", space=F.MemorySpace.SHARED) if staged else None
+    d0, d1 = b.get_affine_dim_expr(0), b.get_affine_dim_expr(1)
+    c = b.get_affine_constant_expr
+    src_map = F.AffineMap.get(2, 0, [d0 * 32, d1 * (src_tile_step or 1)])
+    dst_map = F.AffineMap.get(2, 0, [d0 * dst_scale[0] + dst_origin[0], d1 * (dst_scale[1] // 64) + dst_origin[1]])
+    zero = F.AffineMap.get(0, 0, [c(0), c(0)])
+
+    def tile_body(bb, j):  # j walks columns in elements (step 64)
+        if staged:
+            bb.create_copy_op(x, tile, [by, j], [], src_map, zero, [32, 64], [32, 64])
+            bb.create_copy_op(tile, y, [], [by, j], zero, dst_map, [32, 64], [32, 64])
+        else:
+            bb.create_copy_op(x, y, [by, j], [by, j], src_map, dst_map, [32, 64], [32, 64])
+
+    if loop:
+        b.create_for_op(0, cols, 64, tile_body)
+    else:
+        tile_body(b, by)
+    return kernel
+
+
+def test_tiled_copy_is_lowered_as_one_window_copy():
+    """frisk.copy with index operands (FriskOps.cpp:1551-1683): the tiles of a grid and a loop, through a shared buffer or not,
+    are recognised as one copy of the rectangle they cover"""
+    for staged in (True, False):
+        h = F.create_session()
+        kernel = _tiled_copy_kernel(h, staged=staged)
+        assert h.module.verify()
+        ops = F.runtime.match_ops(kernel)
+        assert len(ops) == 1 and ops[0]["op"] == "copy"
+        o = ops[0]
+        assert (o["src"], o["dst"], o["rows"], o["cols"]) == (0, 1, 128, 256)
+        assert (o["src_offset"], o["dst_offset"], o["src_ld"], o["dst_ld"]) == (0, 16 * 320 + 64, 256, 320)
+        assert (o["src_dtype"], o["dst_dtype"]) == ("f32", "f16")
+        # the printed form parses back to the same program
+        again = F.parse_module(h.context, str(h.module))
+        assert F.runtime.match_ops(again.get_kernel("tiled_copy")) == ops
+
+
+@pytest.mark.parametrize("kw, message", [
+    (dict(src_tile_step=2), "do not tile a rectangle"),            # source tiles 128 columns apart: gaps
+    (dict(dst_scale=(16, 64)), "do not tile a rectangle"),         # destination bands overlap
+    (dict(dst_scale=(64, 64), rows=64), "do not tile a rectangle"),  # destination bands 64 rows apart: gaps
+    (dict(loop=False), "along two dimensions"),                     # one index drives rows and columns
+])
+def test_tiled_copy_that_is_not_one_rectangle_is_refused(kw, message):
+    h = F.create_session()
+    kernel = _tiled_copy_kernel(h, **kw)
+    with pytest.raises(ValueError) as e:
+        F.runtime.match_ops(kernel)
+    assert message in str(e.value), str(e.value)
+
+
+def test_fill_under_a_grid_is_refused():
+    h = F.create_session()
+    t = h.memref_type((64, 64), "fp16")
+    kernel, entry = h.new_kernel("k", [t])
+    body = h.builder.create_parallel_op([4], 64).add_entry_block()
+    h.builder.set_insertion_point_to_start(body)
+    h.builder.create_fill_op(entry.get_argument(0), 1.0, "fp16")
+    with pytest.raises(ValueError) as e:
+        F.runtime.match_ops(kernel)
+    assert "once per iteration" in str(e.value)
+
+
+def test_tiled_copy_that_places_tiles_transposed_is_refused():
+    """both sides tile a square, but tile (by, bx) of the source lands at (bx, by) of the destination: not a window copy"""
+    h = F.create_session()
+    b = h.builder
+    t = h.memref_type((64, 64), "fp16")
+    kernel, entry = h.new_kernel("k", [t, t])
+    body = b.create_parallel_op([2, 2], 64).add_entry_block()
+    b.set_insertion_point_to_start(body)
+    by, bx = body.get_argument(0), body.get_argument(1)
+    d0, d1 = b.get_affine_dim_expr(0), b.get_affine_dim_expr(1)
+    b.create_copy_op(entry.get_argument(0), entry.get_argument(1), [by, bx], [by, bx], F.AffineMap.get(2, 0, [d0 * 32, d1 * 32]),
+                     F.AffineMap.get(2, 0, [d1 * 32, d0 * 32]), [32, 32], [32, 32])
+    with pytest.raises(ValueError) as e:
+        F.runtime.match_ops(kernel)
+    assert "moves the source and destination windows of a tiled copy differently" in str(e.value)

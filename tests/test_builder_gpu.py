@@ -83,3 +83,22 @@ def test_data_movement_kernel_through_the_builder(hip):
     want_y[8:40, 16:80] = T.copy(O.F32, np.ascontiguousarray(x[0:32, 32:96]), O.F16)
     assert np.array_equal(from_dev(dy, np.uint16, (64, 96)), want_y)
     assert np.array_equal(from_dev(dv, np.uint16, (64,)), T.reduce(O.F16, want_y, 1, "max"))
+
+
+def test_tiled_copy_through_the_builder(hip):
+    """a converting copy written tile by tile (grid over row bands, loop over column tiles, every tile through a shared buffer) runs
+    as one window copy on the device; elements outside the destination window keep their bytes"""
+    import torch
+    from oracle import tile_ops as T
+    from test_builder_gemm import _tiled_copy_kernel
+    for staged in (True, False):
+        h = F.create_session()
+        kernel = _tiled_copy_kernel(h, staged=staged)
+        x = O.encode(O.F32, O.normal(128 * 256, 77, 0, 3.0)).reshape(128, 256)
+        dx = to_dev(x)
+        dy = torch.full((160 * 320 * 2,), 0xEE, dtype=torch.uint8, device="cuda")
+        F.runtime.launch_ops(kernel, [dx.data_ptr(), dy.data_ptr()], torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        want = np.full((160, 320), 0xEEEE, dtype=np.uint16)
+        want[16:144, 64:320] = T.copy(O.F32, x, O.F16)
+        assert np.array_equal(from_dev(dy, np.uint16, (160, 320)), want)
