@@ -22,9 +22,9 @@ sys.path.insert(0, ROOT)
 PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "i8": 5033.2, "e4m3": 5033.2, "f32": 157.3}
 FLOPS_PER_CU_CLK = {"f16": 4096, "bf16": 4096, "i8": 8192, "e4m3": 8192, "f32": 256}
 # L2-miss bytes of one fp16 4096^3 launch, a constant taken from rocprofv3 counters (not measured by this run):
-# FETCH_SIZE 98 458.0 KiB x 2.00 (the factor a 1 GiB copy shows for this counter) + WRITE_SIZE 36 371.4 KiB x 1.00
-TRAFFIC_BYTES_F16_4096 = int((98458.0 * 2.0 + 36371.4) * 1024)
-TRAFFIC_SOURCE = "constant from profiles/bench_kernels_f16_4096_i8_4096_fp8_skinny.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE), not measured by this run"
+# FETCH_SIZE 98 426.0 KiB x 2.00 (the factor a 1 GiB copy shows for this counter) + WRITE_SIZE 32 774.8 KiB x 1.00
+TRAFFIC_BYTES_F16_4096 = int((98426.0 * 2.0 + 32774.8) * 1024)
+TRAFFIC_SOURCE = "constant from profiles/bench_gemm_legs_f16_i8_bf16_fp8_f32.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE), not measured by this run"
 
 SETTLE_MS = 100.0
 
@@ -216,7 +216,8 @@ def main():
                    "peak_from_device_properties": {k: round(cus * clock_khz * 1e3 * v / 1e12, 1) for k, v in FLOPS_PER_CU_CLK.items()},
                    "peak_nominal": PEAK_TFLOPS, "note": "CUs x reported clock x flops per CU and clock (4096 16-bit, 8192 8-bit, 256 fp32)",
                    "memory_clock_mhz_reported": round(info["memory_clock_khz"] / 1e3, 1), "memory_bus_bits": info["memory_bus_bits"],
-                   "hbm_peak_from_device_properties_GBps": round(2.0 * info["memory_clock_khz"] * 1e3 * info["memory_bus_bits"] / 8 / 1e9, 1)},
+                   "hbm_peak_from_device_properties_GBps": round(4.0 * info["memory_clock_khz"] * 1e3 * info["memory_bus_bits"] / 8 / 1e9, 1),
+                   "hbm_note": "bus bits x reported memory clock x 4 transfers per clock (HBM3E at 8 Gb/s per pin on a 2 GHz reported clock) / 8"},
     }
 
     if not a.only_headline:
