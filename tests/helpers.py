@@ -32,7 +32,7 @@ def from_dev(t, np_dtype, shape):
 
 
 def run_gemm(R, dtype, A, B, transA, transB, dtype_out, M, N, K, epilogue=0, sA=None, sB=None, C_init=None,
-             clear_accum=True, tile=(0, 0, 0), waves=(0, 0), pad=0, shift=0, split_k=0, workspace=True, stages=0):
+             clear_accum=True, tile=(0, 0, 0), waves=(0, 0), pad=0, shift=0, split_k=0, workspace=True, stages=0, atom=0):
     """launch through the C ABI; returns the output as a numpy array in storage type.
     pad: extra elements at the end of every stored row of A, B and C (odd leading dimensions);
     shift: the operands start `shift` elements into their allocations (pointers only element-aligned);
@@ -56,7 +56,7 @@ def run_gemm(R, dtype, A, B, transA, transB, dtype_out, M, N, K, epilogue=0, sA=
     dsA = to_dev(np.asarray(sA, dtype=np.float32)) if sA is not None else None
     dsB = to_dev(np.asarray(sB, dtype=np.float32)) if sB is not None else None
     desc = R.make_desc(dtype, M, N, K, dtype_out=dtype_out, transA=transA, transB=transB, clear_accum=clear_accum,
-                       epilogue=epilogue, tile=tile, waves=waves, lda=lda, ldb=ldb, ldc=ldc, split_k=split_k, stages=stages)
+                       epilogue=epilogue, tile=tile, waves=waves, lda=lda, ldb=ldb, ldc=ldc, split_k=split_k, stages=stages, atom=atom)
     stream = torch.cuda.current_stream().cuda_stream
     ws_bytes = R.workspace_bytes(desc) if workspace else 0
     ws = torch.full((ws_bytes,), 0xFF, dtype=torch.uint8, device="cuda") if ws_bytes else None

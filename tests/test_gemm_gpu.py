@@ -182,6 +182,25 @@ def _sampled_rows(M, tile, count=64):
     return sorted(rows)
 
 
+def check_marginal_sums(dtype, dtype_out, got, A, B, scale=1.0):
+    """Every element of C = A B^T (A [M][K], B [N][K]) through two linear properties that cost O(MK + NK + MN): the column sums
+    1^T C = (1^T A) B^T and the row sums C 1 = A (B^T 1), in float64.  The rounding of the M (or N) summed outputs is independent
+    from element to element, so a sum is off by about sqrt(count) * eps/3 * rms(C), at most 6e-3 * sqrt(count) * rms(C) over 8192
+    sums of bf16 outputs; one 256 x 256 tile of an 8192^2 result that is wrong by 2 % moves its sums by 4.5e-2 of that unit.
+    Bar: 2e-2 of sqrt(count) * rms(C)."""
+    C = O.decode(dtype_out, got).astype(np.float64)
+    Af, Bf = O.decode(dtype, A).astype(np.float64), O.decode(dtype, B).astype(np.float64)
+    M, N = C.shape
+    rms = float(np.sqrt(np.mean(C * C)))
+    col_ref = (Af.sum(axis=0) @ Bf.T) * scale
+    row_ref = (Af @ Bf.sum(axis=0)) * scale
+    col_err = float(np.abs(C.sum(axis=0) - col_ref).max() / (np.sqrt(M) * rms))
+    row_err = float(np.abs(C.sum(axis=1) - row_ref).max() / (np.sqrt(N) * rms))
+    assert np.isfinite(C).all()
+    assert col_err <= 2e-2 and row_err <= 2e-2, (col_err, row_err)
+    return {"col_sum_err": col_err, "row_sum_err": row_err}
+
+
 def test_config_bf16_8192_nt(hip):
     """8192^3: the oracle checks 64 evenly spaced rows plus the first and last row of every tile band"""
     M = N = K = 8192
@@ -192,6 +211,7 @@ def test_config_bf16_8192_nt(hip):
     ref = O.gemm_f64(O.BF16, np.ascontiguousarray(A[rows]), B, False, True)
     r = check(O.BF16, O.BF16, np.ascontiguousarray(got[rows]), ref)
     note(f"bf16 8192^3 NT ({len(rows)} rows): {r}")
+    note(f"bf16 8192^3 NT, all elements through row and column sums: {check_marginal_sums(O.BF16, O.BF16, got, A, B)}")
 
 
 def test_config_fp8_8192(hip):
@@ -206,6 +226,8 @@ def test_config_fp8_8192(hip):
     ref = O.gemm_f64(O.E4M3, np.ascontiguousarray(A[rows]), B, False, True)
     r = check(O.E4M3, O.BF16, np.ascontiguousarray(got[rows]), O.epilogue_tensor(ref, sA, sB))
     note(f"fp8 8192^3 NT ({len(rows)} rows): {r}")
+    sums = check_marginal_sums(O.E4M3, O.BF16, got, A, B, scale=float(sA) * float(sB))
+    note(f"fp8 8192^3 NT, all elements through row and column sums: {sums}")
 
 
 # ------------------------------------------------------------------ ragged shapes, odd leading dimensions, K = 0
