@@ -294,3 +294,24 @@ def test_atom_choice_follows_the_fill_of_the_round():
                                         ((4096, 4096, 4096), 0, 0, 16), ((8192, 8192, 8192), 0, 1, 16)):
             p = R.plan(R.make_desc(dt, M, N, K, transA=tA, transB=tB))
             assert (p.tile_m, p.tile_n, p.mfma_m) == (256, 256, atom), (dt, M, N, K, tA, tB, p.mfma_m)
+
+
+def test_tiles_whose_rows_span_4_gib_are_not_given_to_the_fast_kernels():
+    """the fast kernels address a tile's chunks by 32-bit lane offsets from its first row: the planner must not pick one whose
+    stored tile rows span 4 GiB or more (views with enormous leading dimensions); it falls to smaller tiles, then to the guarded kernel"""
+    seen_smaller = seen_guarded = False
+    for dt, es, bk in ((R.F16, 2, 64), (R.I8, 1, 128)):
+        for tA, tB in ((0, 0), (0, 1), (1, 0)):
+            for shift in range(20, 33):
+                for operand in "AB":
+                    ld = 1 << shift
+                    kw = dict(lda=ld) if operand == "A" else dict(ldb=ld)
+                    p = R.plan(R.make_desc(dt, 4096, 4096, 4096, dtype_out=R.F16 if dt == R.F16 else R.I32, transA=bool(tA), transB=bool(tB), **kw))
+                    if p.guarded:
+                        seen_guarded = True
+                        continue
+                    rows = (p.tile_k if tA else p.tile_m) if operand == "A" else (p.tile_n if tB else p.tile_k)
+                    assert rows * ld * es < 1 << 32, (dt, tA, tB, operand, ld, R.kernel_names()[p.kernel_id])
+                    seen_smaller = seen_smaller or (operand == "A" and not tA and p.tile_m < 256)
+    assert seen_smaller and seen_guarded
+    assert not R.plan(R.make_desc(R.F16, 4096, 4096, 4096, dtype_out=R.F16, lda=1 << 22)).guarded   # 256 rows x 8 MiB = 2 GiB: the default tile
