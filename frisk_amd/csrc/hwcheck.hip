@@ -74,13 +74,13 @@ template <int ID> __global__ void __launch_bounds__(64) atom_kernel(const float*
     v8i a, b; unsigned char* pa = (unsigned char*)&a; unsigned char* pb = (unsigned char*)&b;
     for (int e = 0; e < 32; ++e) { const int k = 32 * (l / 32) + e; pa[e] = e4m3_of_small_int(A[(l % 32) * 64 + k]); pb[e] = e4m3_of_small_int(B[k * 32 + (l % 32)]); }
     v16f c = {0};
-    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);  // zero scale operands: the instruction without block scales, as in the GEMM kernels
     for (int r = 0; r < 16; ++r) D[d_row<32>(l, r) * 32 + (l % 32)] = c[r];
   } else if constexpr (ID == 7) {  // f8f6f4 (e4m3) 16x16x128
     v8i a, b; unsigned char* pa = (unsigned char*)&a; unsigned char* pb = (unsigned char*)&b;
     for (int e = 0; e < 32; ++e) { const int k = 32 * (l / 16) + e; pa[e] = e4m3_of_small_int(A[(l % 16) * 128 + k]); pb[e] = e4m3_of_small_int(B[k * 16 + (l % 16)]); }
     f4v c = {0};
-    c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+    c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
     for (int r = 0; r < 4; ++r) D[d_row<16>(l, r) * 16 + (l % 16)] = c[r];
   } else if constexpr (ID == 8) {  // fp8 16x16x32 (64-bit operands)
     long a, b; unsigned char* pa = (unsigned char*)&a; unsigned char* pb = (unsigned char*)&b;
