@@ -112,6 +112,52 @@ def test_accumulate_into_c(hip):
     assert np.array_equal(goti, O.gemm_i32(A8, B8) + Ci)
 
 
+OUT_TYPES = {O.F16: [O.F16, O.F32], O.BF16: [O.BF16, O.F32], O.I8: [O.I32, O.F16, O.F32], O.E4M3: [O.BF16, O.F16, O.F32], O.F32: [O.F32]}
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.I8, O.E4M3, O.F32])
+def test_every_output_type_epilogue_and_accumulation(hip, dtype):
+    """all valid (output type, epilogue kind, clear_accum) combinations of a type on the unguarded kernels (the large tile with
+    both atom sizes where compiled, and a small one): out = convert(old C + (acc * sA) * sB), against the oracle's float64
+    accumulators with the same fp32 scale products; int32 outputs exact"""
+    M, N, K = 512, 512, 3 * BK[dtype]
+    tB = 1 if dtype == O.E4M3 else 0
+    A = make_operand(dtype, M, K, seed=21, tensor=0, scale=0.5)
+    B = make_operand(dtype, *((N, K) if tB else (K, N)), seed=21, tensor=1, scale=0.5)
+    acc = O.gemm_i32(A, B, 0, tB).astype(np.float64) if dtype == O.I8 else O.gemm_f64(dtype, A, B, 0, tB)
+    rowA, colB = O.uniform(M, 21, 2, 0.25, 2.0), O.uniform(N, 21, 3, 0.25, 2.0)
+    if dtype == O.I8:
+        rowA, colB = rowA * np.float32(2.0 ** -9), colB * np.float32(2.0 ** -9)
+    tiles = [((0, 0, 0), 0)] if dtype == O.F32 else [((BIG[dtype], BIG[dtype], BK[dtype]), 32), ((SMALL[dtype], SMALL[dtype], BK[dtype]), 0)]
+    if dtype in (O.F16, O.BF16, O.I8):
+        tiles.insert(0, ((256, 256, BK[dtype]), 16))
+    for out_dt in OUT_TYPES[dtype]:
+        for epi in (hip.EPI_NONE, hip.EPI_ROW_COL_SCALE, hip.EPI_TENSOR_SCALE):
+            if out_dt == O.I32 and epi != hip.EPI_NONE:
+                continue
+            if dtype == O.I8 and out_dt == O.F16 and epi == hip.EPI_NONE:
+                continue  # raw int8 accumulators of this size overflow fp16
+            sA = None if epi == hip.EPI_NONE else (rowA if epi == hip.EPI_ROW_COL_SCALE else rowA[:1])
+            sB = None if epi == hip.EPI_NONE else (colB if epi == hip.EPI_ROW_COL_SCALE else colB[:1])
+            scaled = acc if epi == hip.EPI_NONE else ((acc * (sA.astype(np.float64)[:, None] if len(sA) > 1 else float(sA[0]))) * (sB.astype(np.float64)[None, :] if len(sB) > 1 else float(sB[0])))
+            for accumulate in (False, True):
+                if out_dt == O.I32:
+                    C0 = (np.arange(M * N, dtype=np.int64).reshape(M, N) % 2001 - 1000).astype(np.int32)
+                    old = C0.astype(np.float64)
+                else:
+                    old = O.decode(out_dt, O.encode(out_dt, O.uniform(M * N, 22, 4, -2.0, 2.0))).reshape(M, N).astype(np.float64)
+                    C0 = O.encode(out_dt, old.astype(np.float32)).reshape(M, N)
+                ref = scaled + (old if accumulate else 0.0)
+                for tile, atom in tiles:
+                    note(f"case epilogue {NAMES[dtype]}->{out_dt} epi={epi} accumulate={accumulate} tile={tile} atom={atom}")
+                    got = run_gemm(hip, dtype, A, B, 0, tB, out_dt, M, N, K, epilogue=epi, sA=sA, sB=sB, C_init=C0 if accumulate else None,
+                                   clear_accum=not accumulate, tile=tile, atom=atom)
+                    if out_dt == O.I32:
+                        assert np.array_equal(got, ref.astype(np.int64).astype(np.int32))
+                    else:
+                        check(dtype, out_dt, got, ref)
+
+
 def test_int8_dequant_epilogue_bit_exact(hip):
     """out = f16((float(acc) * sA[m]) * sB[n]) with the multiplication order fixed: bit-exact against the oracle"""
     M, N, K = 512, 512, 1024
