@@ -337,12 +337,17 @@ def main():
                 R.gemm(dk, a_.data_ptr(), b_.data_ptr(), Cf.data_ptr(), one.data_ptr(), one.data_ptr(), wsk.data_ptr() if wk else None, wk, cs)
             return time_launches(torch, fn, a.steps, a.warmup, stream)["mean_ms"]
         floor_ms, double_ms = skinny_at(kernel_bk), skinny_at(2 * Ks)
+        # what the platform charges for any launch: a kernel of the same grid (256 work-groups of 256 lanes) that issues 64 MFMAs on
+        # registers and touches no memory
+        empty_ms = time_launches(torch, lambda: HW.mfma_loop(0, 1, False, cus, cs), a.steps, a.warmup, stream)["mean_ms"]
         stream_gbs = (Ms + Ns) * Ks / ((double_ms - tsk["mean_ms"]) * 1e-3) / 1e9
         legs["fp8_skinny_32x8192x8192"].update({
-            "launch_floor_ms": round(floor_ms, 5), "kernel_ms_at_2K": round(double_ms, 5), "streaming_GBps": round(stream_gbs, 1),
+            "launch_floor_ms": round(floor_ms, 5), "register_only_kernel_ms": round(empty_ms, 5), "kernel_ms_at_2K": round(double_ms, 5),
+            "streaming_GBps": round(stream_gbs, 1),
             "frac_at_2K": round((Ms * 2 * Ks + Ns * 2 * Ks + 2 * Ms * Ns + 8) / (double_ms * 1e-3) / 8e12, 4),
-            "bound_note": "launch_floor_ms is this kernel and grid with K of one K tile; streaming_GBps the slope between K=8192 and K=16384; "
-                          "kernel_ms is close to launch_floor_ms + bytes / streaming rate"})
+            "bound_note": "launch_floor_ms is this kernel and grid with K of one K tile; register_only_kernel_ms a launch of the same grid that "
+                          "touches no memory; streaming_GBps the slope between K=8192 and K=16384; kernel_ms is close to "
+                          "launch_floor_ms + bytes / streaming rate"})
         del Bf
 
         # the dialect's data-movement ops on a 32768 x 8192 f16 view (512 MiB per array: twice the last-level cache)
