@@ -26,6 +26,10 @@ FLOPS_PER_CU_CLK = {"f16": 4096, "bf16": 4096, "i8": 8192, "e4m3": 8192, "f32": 
 TRAFFIC_BYTES_F16_4096 = int((98426.0 * 2.0 + 32774.8) * 1024)
 TRAFFIC_SOURCE = "constant from profiles/bench_gemm_legs_f16_i8_bf16_fp8_f32.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE), not measured by this run"
 
+# duration of the register-only kernel (256 work-groups, 64 MFMAs, no memory) in a rocprofv3 kernel trace; event-timed back to
+# back the same launch takes longer by the gap between two launches
+REGISTER_ONLY_KERNEL_TRACE_MS = 0.00355
+
 SETTLE_MS = 100.0
 
 
@@ -115,9 +119,48 @@ def mfma_ceiling(torch, HW, stream, cus):
     return out
 
 
+def data_fed_ceiling(torch, HW, stream, cus, kind, dtype_key, A, B):
+    """the same MFMA-only loop with its operand registers loaded once from the benchmark's own A and B (row-major device
+    tensors): the matrix pipe then switches on the bits of the workload, not on a synthetic pattern"""
+    iters = 4000
+    lda, ldb = A.stride(0) * A.element_size(), B.stride(0) * B.element_size()
+    run = lambda: HW.mfma_loop_data(kind, iters, cus, A.data_ptr(), lda, A.shape[0], B.data_ptr(), ldb, B.shape[0], stream.cuda_stream)
+    settle(torch, run, stream, 60.0)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    times = []
+    for _ in range(5):
+        e0.record(stream)
+        run()
+        e1.record(stream)
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1))
+    ms = statistics.median(times)
+    rate = HW.mfma_loop_flops(kind, iters, cus) / (ms * 1e-3) / 1e12
+    return {"dtype": dtype_key, "rate": round(rate, 1), "frac_of_nominal": round(rate / PEAK_TFLOPS[dtype_key], 4),
+            "implied_clock_mhz": round(HW.mfma_loop_cycles(kind, iters) / (ms * 1e3), 1), "ms": round(ms, 4)}
+
+
+def vendor_leg(torch, name, call, flops_or_bytes, steps, warmup, stream, ours_ms, note=""):
+    """One launch of the vendor library (torch -> hipBLASLt / rocBLAS) on the same device tensors, timed with the same
+    settle and event protocol as the product's legs.  An external comparator: never the product path.  A call that this
+    torch build does not offer is recorded with its error text."""
+    try:
+        call()
+        torch.cuda.synchronize()
+        t = time_launches(torch, call, steps, warmup, stream)
+    except Exception as exc:  # noqa: BLE001  (whatever the library raises is the record)
+        return {"error": "%s: %s" % (type(exc).__name__, str(exc).split("\n")[0][:300]), "call": name}
+    out = {"call": name, "kernel_ms": round(t["mean_ms"], 5), "kernel_ms_median": round(t["median_ms"], 5), "kernel_ms_min": round(t["min_ms"], 5),
+           "rate": round(flops_or_bytes / (t["mean_ms"] * 1e-3) / 1e12, 2), "ours_ms": round(ours_ms, 5),
+           "vs_vendor": round(t["mean_ms"] / ours_ms, 4)}
+    if note:
+        out["note"] = note
+    return out
+
+
 def sustained_peak(ceiling, dtype_key):
     """best MFMA-only rate any atom of this element type sustained in this run"""
-    return max(v["rate"] for k, v in ceiling.items() if v["dtype"] == dtype_key and "constant" not in k)
+    return max(v["rate"] for k, v in ceiling.items() if v["dtype"] == dtype_key and "constant" not in k and "operands of" not in k)
 
 
 def cpu_baseline(M, N, K):
@@ -135,6 +178,22 @@ def cpu_baseline(M, N, K):
     best = min(runs)
     return {"value": round(2.0 * M * N * K / best / 1e12, 4), "unit": "TFLOP/s", "cores": O.num_threads(), "kind": "port",
             "sample": "full fp16 4096^3 NN GEMM, fp32 arithmetic, best of 3 runs (%.2f s each)" % best}
+
+
+def cpu_baseline_int8(M, N, K):
+    """the CPU oracle's exact int8 x int8 -> int32 GEMM (OpenMP over all host cores) on the second headline shape"""
+    import oracle as O
+    A = O.int8_uniform(M * K, 3, 0).reshape(M, K)
+    B = O.int8_uniform(K * N, 3, 1).reshape(K, N)
+    O.gemm_i32(A, B, nrows=256)
+    runs = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        O.gemm_i32(A, B)
+        runs.append(time.perf_counter() - t0)
+    best = min(runs)
+    return {"value": round(2.0 * M * N * K / best / 1e12, 4), "unit": "TOP/s", "cores": O.num_threads(), "kind": "port",
+            "sample": "full int8 4096^3 NN GEMM, int32 accumulate, best of 3 runs (%.2f s each)" % best}
 
 
 def main():
@@ -197,7 +256,7 @@ def main():
     t8 = time_launches(torch, gemm_launcher(d8, (A8.data_ptr(), B8.data_ptr(), C8.data_ptr(), sA.data_ptr(), sB.data_ptr())), a.steps, a.warmup, stream)
     legs = {"int8_4096": mfma_leg("W8A8 int8 4096^3 NN, int32 accumulate, per-row/per-column fp32 scales, fp16 out (configs[3])", "i8", flops, t8,
                                   {"kernel": R.kernel_names()[R.plan(d8).kernel_id]})}
-    del A8, B8, C8
+    vendor = {}
 
     line = {
         "metric": "GEMM TFLOP/s at 4096^3 fp16 (fp32 accumulate), 1 GPU",
@@ -233,16 +292,29 @@ def main():
             R.gemm(desc, a_.data_ptr(), b_.data_ptr(), c_.data_ptr(), None, None, None, 0, cs)
         line["roofline"]["kernel_ms_rotating_4_buffer_sets"] = round(time_launches(torch, cold, a.steps, a.warmup, stream)["mean_ms"], 5)
         del sets
+        Cv = torch.empty(M, N, device=dev, dtype=torch.float16)
+        vendor["fp16_4096_nn"] = vendor_leg(torch, "torch.matmul(A, B, out=C), fp16 4096^3 NN", lambda: torch.matmul(A, B, out=Cv), flops, a.steps, a.warmup,
+                                            stream, t16["mean_ms"])
+        C32 = torch.empty(M, N, device=dev, dtype=torch.int32)
+        vendor["int8_4096"] = vendor_leg(torch, "torch._int_mm(A, B, out=C), int8 4096^3 NN", lambda: torch._int_mm(A8, B8, out=C32), flops, a.steps, a.warmup,
+                                         stream, t8["mean_ms"], "the vendor call writes raw int32 accumulators (64 MiB), the product leg dequantises to fp16 (32 MiB)")
+        del C32
 
         # the same problem with B stored [N][K]: both operands K-contiguous in LDS, no transpose reads
         Bt = B.t().contiguous()
         dnt = R.make_desc(R.F16, M, N, K, dtype_out=R.F16, transB=True)
         tnt = time_launches(torch, gemm_launcher(dnt, (A.data_ptr(), Bt.data_ptr(), C.data_ptr(), None, None)), a.steps, a.warmup, stream)
         legs["fp16_4096_nt"] = mfma_leg("fp16 4096^3 NT (B stored [N][K])", "f16", flops, tnt, {"kernel": R.kernel_names()[R.plan(dnt).kernel_id]})
-        del Bt
+        vendor["fp16_4096_nt"] = vendor_leg(torch, "torch.matmul(A, Bt.t(), out=C), fp16 4096^3 NT", lambda: torch.matmul(A, Bt.t(), out=Cv), flops, a.steps, a.warmup,
+                                            stream, tnt["mean_ms"])
+        del Cv
 
         # what the matrix pipe sustains on this box when nothing else runs
         ceiling = mfma_ceiling(torch, HW, stream, cus)
+        # the atoms the headline kernels run on, fed from the workloads' own operands
+        ceiling["f16 16x16x32, operands of the fp16 4096^3 workload"] = data_fed_ceiling(torch, HW, stream, cus, 1, "f16", A, Bt)
+        ceiling["i8 16x16x64, operands of the int8 4096^3 workload"] = data_fed_ceiling(torch, HW, stream, cus, 5, "i8", A8, B8)
+        del Bt, A8, B8, C8
         line["mfma_ceiling"] = ceiling
         sp = sustained_peak(ceiling, "f16")
         line["roofline"]["sustained_peak"] = sp
@@ -269,6 +341,9 @@ def main():
         t1c = time_launches(torch, gemm_launcher(d1, (A1.data_ptr(), B1.data_ptr(), C1.data_ptr(), None, None)), a.steps, a.warmup, stream)
         legs["fp32_1024"] = mfma_leg("fp32 1024^3 NN through the C ABI, planner's choice of tile", "f32", 2.0 * M1 ** 3, t1c,
                                      {"kernel": R.kernel_names()[R.plan(d1).kernel_id]})
+        C1v = torch.empty(M1, M1, device=dev)
+        vendor["fp32_1024"] = vendor_leg(torch, "torch.matmul(A, B, out=C), fp32 1024^3 NN (allow_tf32 = %s)" % torch.backends.cuda.matmul.allow_tf32,
+                                         lambda: torch.matmul(A1, B1, out=C1v), 2.0 * M1 ** 3, a.steps, a.warmup, stream, t1c["mean_ms"])
 
         # configs[2]: bf16 8192^3 NT; configs[4], square part: fp8 e4m3 8192^3 NT with per-tensor scales, bf16 out
         Mb = 8192
@@ -282,6 +357,10 @@ def main():
                                         {"kernel": R.kernel_names()[R.plan(db).kernel_id], "steps": big_steps,
                                          "sustained_peak": sustained_peak(ceiling, "bf16")})
         legs["bf16_8192_nt"]["frac_of_sustained"] = round(legs["bf16_8192_nt"]["achieved"] / legs["bf16_8192_nt"]["sustained_peak"], 4)
+        Cbv = torch.empty(Mb, Mb, device=dev, dtype=torch.bfloat16)
+        vendor["bf16_8192_nt"] = vendor_leg(torch, "torch.matmul(A, Bt.t(), out=C), bf16 8192^3 NT", lambda: torch.matmul(Ab, Bb.t(), out=Cbv), 2.0 * Mb ** 3, big_steps, 3,
+                                            stream, tb["mean_ms"])
+        ceiling["bf16 16x16x32, operands of the bf16 8192^3 workload"] = data_fed_ceiling(torch, HW, stream, cus, 3, "bf16", Ab, Bb)
         A8f = (torch.randn(Mb, Mb, device=dev, generator=g) * 100).clamp(-448, 448).to(torch.float8_e4m3fn)
         B8f = (torch.randn(Mb, Mb, device=dev, generator=g) * 100).clamp(-448, 448).to(torch.float8_e4m3fn)
         one = torch.full((1,), 0.01, device=dev)
@@ -291,7 +370,12 @@ def main():
                                        "e4m3", 2.0 * Mb ** 3, t8f, {"kernel": R.kernel_names()[R.plan(d8f).kernel_id], "steps": big_steps,
                                                                     "sustained_peak": sustained_peak(ceiling, "e4m3")})
         legs["fp8_8192_nt"]["frac_of_sustained"] = round(legs["fp8_8192_nt"]["achieved"] / legs["fp8_8192_nt"]["sustained_peak"], 4)
-        del Ab, Bb, Cb, A8f, B8f
+        vendor["fp8_8192_nt"] = vendor_leg(torch, "torch._scaled_mm(A, Bt.t(), scale_a, scale_b, out_dtype=bfloat16), e4m3 8192^3 NT",
+                                           lambda: torch._scaled_mm(A8f, B8f.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16), 2.0 * Mb ** 3, big_steps, 3,
+                                           stream, t8f["mean_ms"], "the vendor call allocates its output in every call (torch's caching allocator)")
+        ceiling["f8f6f4 32x32x64, operands of the fp8 8192^3 workload"] = data_fed_ceiling(torch, HW, stream, cus, 6, "e4m3", A8f, B8f)
+        ceiling["f8f6f4 16x16x128, operands of the fp8 8192^3 workload"] = data_fed_ceiling(torch, HW, stream, cus, 7, "e4m3", A8f, B8f)
+        del Ab, Bb, Cb, Cbv, A8f, B8f
 
         # HBM-bound shape of the configuration list: fp8 e4m3 M=32, N=K=8192 (B stored [N][K]), per-tensor scales, bf16 out.
         # B rotates over 6 buffers (384 MiB > the 256 MiB last-level cache) so every launch streams it from HBM.
@@ -317,6 +401,14 @@ def main():
                                            "kernel_ms_min": round(tsk["min_ms"], 5), "kernel": R.kernel_names()[pf.kernel_id], "split_k": pf.split_k,
                                            "workload": "fp8 e4m3 M=32 N=K=8192 NT, per-tensor scales, bf16 out (configs[4], decode part); algorithmic bytes "
                                                        "|A|+|B|+|C|+scales per launch, B rotating over 6 buffers"}
+        vk_turn = [0]
+
+        def vendor_skinny():
+            b_ = Bf[vk_turn[0] % len(Bf)]
+            vk_turn[0] += 1
+            return torch._scaled_mm(Af, b_.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+        vendor["fp8_skinny_32x8192x8192"] = vendor_leg(torch, "torch._scaled_mm(A, Bt.t(), ...), e4m3 32x8192x8192 NT, B rotating over the same 6 buffers", vendor_skinny,
+                                                       float(sk_bytes) , a.steps, a.warmup, stream, tsk["mean_ms"], "rate in TB/s of algorithmic bytes")
         # what bounds this shape: the same kernel and grid with K shrunk to one K tile (the fixed cost of a launch: dispatch,
         # the first tile's trip from HBM, the epilogue) and with K doubled; the slope between K and 2K is the rate at which the
         # kernel streams B once it runs
@@ -345,6 +437,11 @@ def main():
             "launch_floor_ms": round(floor_ms, 5), "register_only_kernel_ms": round(empty_ms, 5), "kernel_ms_at_2K": round(double_ms, 5),
             "streaming_GBps": round(stream_gbs, 1),
             "frac_at_2K": round((Ms * 2 * Ks + Ns * 2 * Ks + 2 * Ms * Ns + 8) / (double_ms * 1e-3) / 8e12, 4),
+            "kernel_ms_without_launch_gap": round(tsk["mean_ms"] - max(0.0, empty_ms - REGISTER_ONLY_KERNEL_TRACE_MS), 5),
+            "frac_without_launch_gap": round(sk_bytes / ((tsk["mean_ms"] - max(0.0, empty_ms - REGISTER_ONLY_KERNEL_TRACE_MS)) * 1e-3) / 8e12, 4),
+            "launch_gap_note": "kernel_ms is an event pair around back-to-back launches and so holds the gap between two launches; the gap is taken as "
+                               "register_only_kernel_ms minus that kernel's own duration in a kernel trace (%.5f ms, a constant of the committed profile): "
+                               "kernel_ms_without_launch_gap is the figure to hold against a rocprofv3 kernel duration" % REGISTER_ONLY_KERNEL_TRACE_MS,
             "bound_note": "launch_floor_ms is this kernel and grid with K of one K tile; register_only_kernel_ms a launch of the same grid that "
                           "touches no memory; streaming_GBps the slope between K=8192 and K=16384; kernel_ms is close to "
                           "launch_floor_ms + bytes / streaming rate"})
@@ -398,9 +495,19 @@ def main():
                                                "workload": "softmax(Q K^T / sqrt(128)) V, 32 heads, 4096 queries x 4096 keys, head_dim 128, "
                                                            "fp16 in / out, fp32 accumulate; 4 * heads * seq^2 * head_dim flops per launch"}
 
+    for key, v in vendor.items():
+        leg = line["roofline"] if key == "fp16_4096_nn" else legs.get(key)
+        if leg is not None and "vs_vendor" in v:
+            leg["vs_vendor"] = v["vs_vendor"]
+            leg["vendor_kernel_ms"] = v["kernel_ms"]
+    if vendor:
+        line["vendor_same_run"] = {"what": "torch %s -> hipBLASLt / rocBLAS on the same device tensors, same settle and HIP-event protocol; vs_vendor = vendor "
+                                           "time / this build's time (above 1: this build is faster); an external comparator, never the product path" % torch.__version__,
+                                   **vendor}
     line.update(legs)
     if not a.no_cpu and not a.only_headline:
         line["cpu_baseline"] = cpu_baseline(M, N, K)
+        line["cpu_baseline_int8"] = cpu_baseline_int8(M, N, K)
     print(json.dumps(line))
 
 

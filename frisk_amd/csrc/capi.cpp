@@ -474,9 +474,15 @@ int frisk_hip_gemm_static_ws(const frisk_gemm_desc* desc, const void* A, const v
   frisk_gemm_plan plan;
   int st = make_plan(desc, &plan, false);
   if (st != FRISK_OK) return st;
-  if (plan.workspace_bytes > (size_t)FRISK_HIP_STATIC_WS_BYTES)
-    return fail(FRISK_ERR_WORKSPACE, "this problem's partial sums need %zu bytes, the static workspace holds %zu: pass split_k = 1 or use frisk_hip_gemm with a workspace",
-                plan.workspace_bytes, (size_t)FRISK_HIP_STATIC_WS_BYTES);
+  // What does not fit the array: an explicit split_k is refused (the caller asked for exactly that split); a split the
+  // planner chose by itself (tail splits of large grids reach 64 MiB) is dropped, and the launch runs as one pass, which
+  // is what frisk_hip_gemm does for the same descriptor without a workspace.
+  if (plan.workspace_bytes > (size_t)FRISK_HIP_STATIC_WS_BYTES) {
+    if (desc->split_k > 1)
+      return fail(FRISK_ERR_WORKSPACE, "split_k=%d needs %zu bytes of partial sums, the static workspace holds %zu: pass a smaller split_k, or use frisk_hip_gemm with a workspace",
+                  desc->split_k, plan.workspace_bytes, (size_t)FRISK_HIP_STATIC_WS_BYTES);
+    return frisk_hip_gemm(desc, A, B, C, scaleA, scaleB, nullptr, 0, stream);
+  }
   void* ws = nullptr;
   if (plan.workspace_bytes > 0) {
     if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");

@@ -239,7 +239,16 @@ template <int KIND> struct LoopShape {
   static constexpr int CYCLES_PER_MFMA = AT == 32 ? (KIND >= 6 ? 64 : 32) : (KIND >= 6 ? 32 : 16);
 };
 
-template <int KIND, bool RANDOM> __global__ void __launch_bounds__(256) mfma_loop_kernel(int iters) {
+// The operands of a data-fed loop: two row-major device arrays (the benchmark's own A and B); `rows` rows of at least 256 bytes; every lane takes its fragments from them exactly as a K-contiguous operand tile would deliver them
+// (lane l of an atom: row l % AT, the l / AT-th group of consecutive bytes along the row).
+struct LoopData {
+  const char* a;
+  const char* b;
+  long long lda_bytes, ldb_bytes;
+  int rows_a, rows_b;
+};
+
+template <int KIND, bool RANDOM> __global__ void __launch_bounds__(256) mfma_loop_kernel(int iters, LoopData data) {
 #ifdef __HIP_DEVICE_COMPILE__  // the host pass only needs the launch stub; it cannot parse the 256-bit register operands
   typedef LoopShape<KIND> S;
   constexpr int NAT = S::NAT, KS = S::KS, FI = S::FRAG_INTS;
@@ -274,6 +283,22 @@ template <int KIND, bool RANDOM> __global__ void __launch_bounds__(256) mfma_loo
           else bits = 0x38383838u | (x & 0x87878787u);
           if (side == 0) a[s][i][e] = (int)bits; else b[s][i][e] = (int)bits;
         }
+  if (data.a) {
+    // fragments of real operands: wave w of work-group g owns rows (4 g + w) * 128 ... + 127 of both arrays (modulo
+    // their row counts); K step s, lane group l / AT reads FI * 4 consecutive bytes of its row
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row0 = (blockIdx.x * 4 + wave) * 128;
+    const int kbyte = (lane / S::AT) * FI * 4;
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int i = 0; i < NAT; ++i) {
+        const long long ko = (long long)s * (64 / S::AT) * FI * 4 + kbyte;
+        const int ra = (row0 + i * S::AT + lane % S::AT) % data.rows_a, rb = (row0 + i * S::AT + lane % S::AT) % data.rows_b;
+        a[s][i] = *(const frag_t*)(data.a + ra * data.lda_bytes + ko);
+        b[s][i] = *(const frag_t*)(data.b + rb * data.ldb_bytes + ko);
+      }
+  }
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
     for (int s = 0; s < KS; ++s)
@@ -299,9 +324,9 @@ template <int KIND, bool RANDOM> __global__ void __launch_bounds__(256) mfma_loo
 #endif
 }
 
-template <int KIND> hipError_t launch_loop(int iters, int random_operands, int workgroups, hipStream_t s) {
-  if (random_operands) hipLaunchKernelGGL((mfma_loop_kernel<KIND, true>), dim3(workgroups), dim3(256), 0, s, iters);
-  else hipLaunchKernelGGL((mfma_loop_kernel<KIND, false>), dim3(workgroups), dim3(256), 0, s, iters);
+template <int KIND> hipError_t launch_loop(int iters, int random_operands, int workgroups, hipStream_t s, const LoopData& data = LoopData{}) {
+  if (random_operands) hipLaunchKernelGGL((mfma_loop_kernel<KIND, true>), dim3(workgroups), dim3(256), 0, s, iters, data);
+  else hipLaunchKernelGGL((mfma_loop_kernel<KIND, false>), dim3(workgroups), dim3(256), 0, s, iters, data);
   return hipGetLastError();
 }
 
@@ -367,6 +392,29 @@ int frisk_hwcheck_mfma_loop(int kind, int iters, int random_operands, int workgr
     case 5: return (int)launch_loop<5>(iters, random_operands, workgroups, s);
     case 6: return (int)launch_loop<6>(iters, random_operands, workgroups, s);
     case 7: return (int)launch_loop<7>(iters, random_operands, workgroups, s);
+    default: return -1;
+  }
+}
+
+// The same loop with its operand registers loaded once from two row-major device arrays (16-byte aligned rows of at least
+// 256 bytes, leading dimensions in bytes): the bits the matrix pipe switches on are then those of the workload itself.
+// Returns a hipError_t, -1 for an unknown kind, -2 for arrays that do not fit.
+int frisk_hwcheck_mfma_loop_data(int kind, int iters, int workgroups, const void* A, long long lda_bytes, int rows_a, const void* B, long long ldb_bytes,
+                                 int rows_b, void* stream) {
+  hipStream_t s = (hipStream_t)stream;
+  if (iters < 0 || workgroups <= 0) return -1;
+  if (!A || !B || rows_a <= 0 || rows_b <= 0 || lda_bytes < 256 || ldb_bytes < 256 || ((uintptr_t)A | (uintptr_t)B | (uintptr_t)lda_bytes | (uintptr_t)ldb_bytes) & 31)
+    return -2;
+  const LoopData data{(const char*)A, (const char*)B, lda_bytes, ldb_bytes, rows_a, rows_b};
+  switch (kind) {
+    case 0: return (int)launch_loop<0>(iters, 1, workgroups, s, data);
+    case 1: return (int)launch_loop<1>(iters, 1, workgroups, s, data);
+    case 2: return (int)launch_loop<2>(iters, 1, workgroups, s, data);
+    case 3: return (int)launch_loop<3>(iters, 1, workgroups, s, data);
+    case 4: return (int)launch_loop<4>(iters, 1, workgroups, s, data);
+    case 5: return (int)launch_loop<5>(iters, 1, workgroups, s, data);
+    case 6: return (int)launch_loop<6>(iters, 1, workgroups, s, data);
+    case 7: return (int)launch_loop<7>(iters, 1, workgroups, s, data);
     default: return -1;
   }
 }

@@ -107,6 +107,15 @@ frisk_gemm_desc desc_of(const GemmProgram& g, int epilogue) {
   return d;
 }
 
+// The descriptor `launch` hands to the C ABI, shared with `plan` so that the plan describes the kernel that runs.  The tile
+// sizes in the IR describe the program; which kernel variant computes it best is the planner's call for the whole problem
+// (1024^3 fp32 written with 128 x 128 tiles is 64 work-groups on 256 CUs).  retile = false keeps the IR's tile.
+frisk_gemm_desc launch_desc_of(const GemmProgram& g, int epilogue, bool retile) {
+  frisk_gemm_desc d = desc_of(g, epilogue);
+  if (retile) d.tile_m = d.tile_n = d.tile_k = 0;
+  return d;
+}
+
 GemmProgram program_of(py::object kernel, py::object module) {
   Operation* k = op_of_handle(kernel);
   Operation* m = module.is_none() ? nullptr : op_of_handle(module);
@@ -272,9 +281,9 @@ void init_ffi_runtime(py::module_&& m) {
         "recognise one of the programs of the reference's design sketches and return what it computes: the tiled GEMM "
         "kernel{parallel{alloc x3, fill, for{copy, copy, gemm}, copy}}, the row softmax with a running log-sum, or the fused attention; pure host");
 
-  m.def("plan", [](py::object kernel, py::object module, const std::string& epilogue) {
+  m.def("plan", [](py::object kernel, py::object module, const std::string& epilogue, bool retile) {
     GemmProgram g = program_of(kernel, module);
-    frisk_gemm_desc d = desc_of(g, epilogue_of(epilogue));
+    frisk_gemm_desc d = launch_desc_of(g, epilogue_of(epilogue), retile);
     HipLibrary& lib = library();
     frisk_gemm_plan p{};
     if (int st = lib.plan(&d, &p)) throw std::invalid_argument(std::string("frisk_hip_plan: ") + lib.last_error() + " (status " + std::to_string(st) + ")");
@@ -295,7 +304,9 @@ void init_ffi_runtime(py::module_&& m) {
     out["flops"] = p.flops;
     out["bytes"] = p.bytes;
     return out;
-  }, py::arg("kernel"), py::arg("module") = py::none(), py::arg("epilogue") = "none");
+  }, py::arg("kernel"), py::arg("module") = py::none(), py::arg("epilogue") = "none", py::arg("retile") = true,
+     "the plan of the kernel that `launch` runs for the same `retile`: by default the planner's own tile for the whole problem, with "
+     "retile = False the tile the program is written with; pure host");
 
   m.def("lds_layout_string", [](int rows, int row_bytes, int elem_bytes, int row_shift, int row_mask, int chunk_shift,
                                 int row_shift2, int row_mask2, int chunk_shift2) {
@@ -451,10 +462,7 @@ void init_ffi_runtime(py::module_&& m) {
     GemmProgram g = match_tiled_gemm(k, mod);
     size_t need = (size_t)std::max(g.arg_a, std::max(g.arg_b, g.arg_c)) + 1;
     if (args.size() < need) throw std::invalid_argument("launch needs one device pointer per kernel argument");
-    frisk_gemm_desc d = desc_of(g, epilogue_of(epilogue));
-    // The tile sizes in the IR describe the program; which kernel variant computes it best is the planner's call for the
-    // whole problem (1024^3 fp32 written with 128 x 128 tiles is 64 work-groups on 256 CUs).  retile = False keeps the IR's tile.
-    if (retile) d.tile_m = d.tile_n = d.tile_k = 0;
+    frisk_gemm_desc d = launch_desc_of(g, epilogue_of(epilogue), retile);
     HipLibrary& lib = library();
     int st;
     {

@@ -17,7 +17,7 @@ LOOP_KINDS = {0: ("f16 32x32x16", "f16"), 1: ("f16 16x16x32", "f16"), 2: ("bf16 
               4: ("i8 32x32x32", "i8"), 5: ("i8 16x16x64", "i8"), 6: ("f8f6f4 32x32x64", "e4m3"), 7: ("f8f6f4 16x16x128", "e4m3")}
 
 _lib = None
-EXPORTS = ["frisk_hwcheck_mfma_atom", "frisk_hwcheck_fragment_path", "frisk_hwcheck_tr_read", "frisk_hwcheck_mfma_loop",
+EXPORTS = ["frisk_hwcheck_mfma_atom", "frisk_hwcheck_fragment_path", "frisk_hwcheck_tr_read", "frisk_hwcheck_mfma_loop", "frisk_hwcheck_mfma_loop_data",
            "frisk_hwcheck_mfma_loop_flops", "frisk_hwcheck_mfma_loop_cycles", "frisk_hwcheck_device_info"]
 
 
@@ -32,6 +32,7 @@ def lib():
         L.frisk_hwcheck_fragment_path.argtypes = [i, i, i, i, vp, vp, vp, vp]
         L.frisk_hwcheck_tr_read.argtypes = [i, vp, vp, i, vp]
         L.frisk_hwcheck_mfma_loop.argtypes = [i, i, i, i, vp]
+        L.frisk_hwcheck_mfma_loop_data.argtypes = [i, i, i, vp, ctypes.c_longlong, i, vp, ctypes.c_longlong, i, vp]
         L.frisk_hwcheck_mfma_loop_flops.argtypes = [i, i, i]
         L.frisk_hwcheck_mfma_loop_flops.restype = ctypes.c_double
         L.frisk_hwcheck_mfma_loop_cycles.argtypes = [i, i]
@@ -60,6 +61,11 @@ def tr_read(bits, lane_addr_ptr, out_ptr, shift=0, stream=None):
 
 def mfma_loop(kind, iters, random_operands, workgroups, stream=None):
     _check(lib().frisk_hwcheck_mfma_loop(kind, iters, int(bool(random_operands)), workgroups, stream), "frisk_hwcheck_mfma_loop")
+
+
+def mfma_loop_data(kind, iters, workgroups, A_ptr, lda_bytes, rows_a, B_ptr, ldb_bytes, rows_b, stream=None):
+    """the MFMA-only loop with its operand registers loaded once from two row-major device arrays"""
+    _check(lib().frisk_hwcheck_mfma_loop_data(kind, iters, workgroups, A_ptr, lda_bytes, rows_a, B_ptr, ldb_bytes, rows_b, stream), "frisk_hwcheck_mfma_loop_data")
 
 
 def mfma_loop_flops(kind, iters, workgroups):

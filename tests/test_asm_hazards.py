@@ -59,10 +59,26 @@ def hazards(listing, window_before=8, window_after=12):
     return found
 
 
+def foreign_m0_uses(listing):
+    """lines that name M0 outside the three-instruction transfer the kernels write themselves (s_add_u32 m0 / s_nop /
+    global_load_lds_dwordx4): the transfer writes M0 without telling the compiler, which is only sound while the
+    compiler has no use of M0 of its own in the kernel"""
+    lines = [l.strip() for l in listing.split("\n") if l.startswith("\t") and not l.strip().startswith((".", ";"))]
+    found = []
+    for i, line in enumerate(lines):
+        if not re.search(r"\bm0\b", line):
+            continue
+        own = line.startswith("s_add_u32 m0, ") and lines[i + 1].startswith("s_nop") and lines[i + 2].startswith("global_load_lds_dwordx4")
+        if not own:
+            found.append(line)
+    return found
+
+
 def test_scanner_sees_both_patterns():
     listing = "\n\t.globl\tk\nk:\n\tv_accvgpr_mov_b32 a5, a1\n\ts_nop 0\n\tv_mfma_f32_16x16x32_f16 a[4:7], v[0:3], v[4:7], a[4:7]\n\tv_accvgpr_read_b32 v9, a6\n"
     got = hazards(listing)
     assert len(got) == 2 and got[0][1].startswith("v_accvgpr_mov") and got[1][2].startswith("v_accvgpr_read")
+    assert foreign_m0_uses("\ts_add_u32 m0, s4, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 v1, s[2:3]\n\ts_mov_b32 m0, s7\n\tds_read_b32 v1, v2\n") == ["s_mov_b32 m0, s7"]
     clean = "\n\t.globl\tk\nk:\n\tv_mfma_f32_16x16x32_f16 a[4:7], v[0:3], v[4:7], a[4:7]\n\tv_mfma_f32_16x16x32_f16 a[8:11], v[0:3], v[4:7], a[8:11]\n"
     assert hazards(clean) == []
 
@@ -80,3 +96,4 @@ def test_inline_assembly_mfma_kernels_keep_their_wait_states(tmp_path):
     assert listing.count("v_mfma_f32_16x16x32_f16") > 300 and "v_mfma_i32_16x16x64_i8" in listing and "v_mfma_f32_16x16x32_bf16" in listing
     bad = hazards(listing)
     assert not bad, "\n".join("%s: %s  ->  %s" % (n[:60], a, b) for n, a, b in bad[:10])
+    assert listing.count("global_load_lds_dwordx4") > 100 and foreign_m0_uses(listing) == []

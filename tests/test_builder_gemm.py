@@ -251,6 +251,21 @@ def test_plan_goes_through_the_hip_library():
     assert p["hip_kernel"].startswith("f16_nt_256x256x64") and p["flops"] == 2.0 * 4096 ** 3
 
 
+def test_plan_names_the_kernel_that_launch_runs_for_either_retile():
+    """`plan` and `launch` build their descriptor in one place: with retile (the default of both) the planner's tile for the
+    whole problem, without it the tile the program is written with"""
+    from frisk_amd import runtime as R
+    h = F.create_session()
+    kernel = h.tiled_gemm("g", 1024, 1024, 1024, "fp32", tile=(128, 128, 32), threads=256)
+    own = R.plan(R.make_desc(R.F32, 1024, 1024, 1024))
+    kept = R.plan(R.make_desc(R.F32, 1024, 1024, 1024, tile=(128, 128, 32)))
+    p = F.runtime.plan(kernel)
+    assert p["hip_kernel"] == R.kernel_names()[own.kernel_id] and p["hip_tile"] == (own.tile_m, own.tile_n, own.tile_k) != (128, 128, 32)
+    assert p["lds_bytes"] == own.lds_bytes and F.runtime.plan(kernel, retile=True) == p
+    q = F.runtime.plan(kernel, retile=False)
+    assert q["hip_kernel"] == R.kernel_names()[kept.kernel_id] and q["hip_tile"] == (128, 128, 32) and q["lds_bytes"] == kept.lds_bytes
+
+
 @pytest.mark.parametrize("dtype,tile,trans_a,trans_b", [("fp16", (256, 256, 64), False, False), ("fp16", (256, 256, 64), False, True),
                                                         ("bf16", (128, 128, 64), True, False),
                                                         ("fp32", (128, 128, 32), False, False)])
@@ -267,7 +282,7 @@ def test_plan_prints_lds_layouts_in_the_reference_debug_form(dtype, tile, trans_
     h = F.create_session()
     n = 4 * max(tile)
     kernel = h.tiled_gemm("g", n, n, n, dtype, tile=tile, trans_a=trans_a, trans_b=trans_b)
-    p = F.runtime.plan(kernel)
+    p = F.runtime.plan(kernel, retile=False)
     for text, (sh, mk, cs) in zip((p["lds_a"], p["lds_b"]), p["lds_swizzle"]):
         m = re.fullmatch(r"Layout\(shape=\[(\d+), (\d+)\], index=(affine_map<.*>)\)", text)
         assert m, text

@@ -315,3 +315,35 @@ def test_tiles_whose_rows_span_4_gib_are_not_given_to_the_fast_kernels():
                     seen_smaller = seen_smaller or (operand == "A" and not tA and p.tile_m < 256)
     assert seen_smaller and seen_guarded
     assert not R.plan(R.make_desc(R.F16, 4096, 4096, 4096, dtype_out=R.F16, lda=1 << 22)).guarded   # 256 rows x 8 MiB = 2 GiB: the default tile
+
+
+def test_planner_choices_for_the_benchmark_shapes_are_pinned():
+    """the kernels bench.py times: a change of the cost table that moves one of them must show here"""
+    want = [
+        ((R.F32, 1024, 1024, 1024, 0, R.F32, R.EPI_NONE), "f32_nn_64x64x128_w2x2x2_s2"),
+        ((R.F16, 4096, 4096, 4096, 0, R.F16, R.EPI_NONE), "f16_nn_256x256x64_w2x2_s2x3_a16"),
+        ((R.F16, 4096, 4096, 4096, 1, R.F16, R.EPI_NONE), "f16_nt_256x256x64_w2x2_s2x3_a16"),
+        ((R.BF16, 8192, 8192, 8192, 1, R.BF16, R.EPI_NONE), "bf16_nt_256x256x64_w2x2_s2x3_a16"),
+        ((R.I8, 4096, 4096, 4096, 0, R.F16, R.EPI_ROW_COL_SCALE), "i8_nn_256x256x128_w2x2_s2x3_a16"),
+        ((R.E4M3, 32, 8192, 8192, 1, R.BF16, R.EPI_TENSOR_SCALE), "e4m3_nt_32x32x512_w1x1x4_s4_splitk"),
+        ((R.E4M3, 8192, 8192, 8192, 1, R.BF16, R.EPI_TENSOR_SCALE), "e4m3_nt_256x256x128_w2x2_s2x3"),
+    ]
+    for (dt, M, N, K, tB, out, epi), name in want:
+        p = R.plan(R.make_desc(dt, M, N, K, dtype_out=out, transB=tB, epilogue=epi))
+        assert R.kernel_names()[p.kernel_id] == name and p.split_k == 1 and p.tail_split == 1, (M, N, K, R.kernel_names()[p.kernel_id])
+
+
+def test_tail_splits_the_planner_chooses_can_exceed_the_static_workspace():
+    """grids whose last round holds 17 ... 128 tiles: the tail split is the planner's own choice (split_k stays 1) and may want more
+    partial sums than frisk_hip_gemm_static_ws holds, which then runs the launch unsplit instead of refusing it"""
+    static = R.static_workspace_bytes()
+    over = 0
+    for dt, M, N, K in [(R.F16, 4608, 4096, 4096), (R.F16, 5120, 4096, 4096), (R.I8, 5120, 4096, 4096), (R.F16, 8192, 4352, 8192), (R.F16, 4096, 4608, 8192),
+                        (R.F16, 4352, 4096, 4096)]:
+        for tB in (0, 1):
+            p = R.plan(R.make_desc(dt, M, N, K, transB=tB, dtype_out=R.I32 if dt == R.I8 else None))
+            tiles = p.grid_x * p.grid_y
+            assert 16 <= tiles % 256 <= 128 and p.split_k == 1 and p.tail_split > 1 and p.tail_tiles == tiles % 256
+            assert p.workspace_bytes == p.tail_split * p.tail_tiles * 256 * 256 * 4
+            over += p.workspace_bytes > static
+    assert over >= 8

@@ -23,9 +23,16 @@ def _static(hip, dtype, A, B, transB, dtype_out, M, N, K, split_k=0, epilogue=0,
     dsA = to_dev(np.asarray(sA, dtype=np.float32)) if sA is not None else None
     dsB = to_dev(np.asarray(sB, dtype=np.float32)) if sB is not None else None
     desc = hip.make_desc(dtype, M, N, K, dtype_out=dtype_out, transB=transB, epilogue=epilogue, split_k=split_k)
+    # the property the entry point exists for: with inputs and outputs on the device, the call leaves the device's free
+    # memory as it found it (hipMemGetInfo through torch; a hipMalloc anywhere below the call would show here)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
     hip.gemm_static_ws(desc, dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), dsA.data_ptr() if dsA is not None else None,
                        dsB.data_ptr() if dsB is not None else None, torch.cuda.current_stream().cuda_stream)
+    free_during = torch.cuda.mem_get_info()[0]
     torch.cuda.synchronize()
+    free_after = torch.cuda.mem_get_info()[0]
+    assert free_before == free_during == free_after, "frisk_hip_gemm_static_ws changed the device's free memory"
     return dC.cpu().numpy().view(out_np).reshape(M, N)
 
 
@@ -67,6 +74,23 @@ def test_static_workspace_tail_split_and_unsplit_plans(hip):
     A = make_operand(O.F16, 256, 128, 51, 0)
     B = make_operand(O.F16, 128, 256, 51, 1)
     assert np.array_equal(_static(hip, O.F16, A, B, 0, O.F16, 256, 256, 128), run_gemm(hip, O.F16, A, B, 0, 0, O.F16, 256, 256, 128))
+
+
+def test_planner_chosen_split_beyond_the_array_runs_as_one_pass(hip):
+    # 4608 x 4096 x 4096 fp16 NT: 288 tiles, the planner splits the last 32 eight ways = 64 MiB of partial sums, twice the
+    # array.  Nobody asked for that split: the call runs the single pass frisk_hip_gemm runs without a workspace.
+    M, N, K = 4608, 4096, 4096
+    d = hip.make_desc(O.F16, M, N, K, transB=True)
+    p = hip.plan(d)
+    note(f"case static workspace, planner split too large {M}x{N}x{K}: tail {p.tail_tiles} x {p.tail_split}, workspace {p.workspace_bytes}")
+    assert p.tail_split > 1 and p.workspace_bytes > hip.static_workspace_bytes()
+    A = make_operand(O.F16, M, K, 52, 0, scale=0.02)
+    B = make_operand(O.F16, N, K, 52, 1, scale=0.02)
+    want = run_gemm(hip, O.F16, A, B, 0, 1, O.F16, M, N, K, workspace=False)
+    got = _static(hip, O.F16, A, B, 1, O.F16, M, N, K)
+    assert np.array_equal(got, want)
+    r = O.compare(O.F16, got[:256].view(np.uint16), O.gemm_f64(O.F16, A[:256], B, transB=1))
+    assert r["nonfinite"] == 0 and r["max_rel"] <= 1e-2 and r["fro_rel"] <= 1e-2, r
 
 
 def test_static_workspace_refuses_what_does_not_fit(hip):
