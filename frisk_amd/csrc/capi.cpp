@@ -448,6 +448,9 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
   p.split_k = plan.split_k;
   p.kt_per_slice = (int)((desc->K + k->bk - 1) / k->bk) / plan.split_k;
   p.partial = plan.split_k > 1 || plan.tail_split > 1 ? workspace : nullptr;
+#ifdef FRISK_WGPROBE
+  p.partial = workspace;
+#endif
   p.tail_split = plan.tail_split;
   p.tail_tiles = plan.tail_tiles;
   p.tail_from = p.tiles_m * p.tiles_n - plan.tail_tiles;
