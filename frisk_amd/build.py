@@ -28,7 +28,7 @@ COMMON = [
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
     "-Wno-unused-command-line-argument",
 ]
-SOURCES = ["kernels_f16.hip", "kernels_bf16.hip", "kernels_i8.hip", "kernels_e4m3.hip", "kernels_f32.hip", "splitk_reduce.hip", "tile_ops.hip", "softmax.hip", "attention.hip", "capi.cpp"]
+SOURCES = ["kernels_f16.hip", "kernels_bf16.hip", "kernels_i8.hip", "kernels_e4m3.hip", "kernels_f32.hip", "splitk_reduce.hip", "tile_ops.hip", "elementwise.hip", "softmax.hip", "attention.hip", "capi.cpp"]
 
 
 def _compile(src):

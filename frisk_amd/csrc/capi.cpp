@@ -448,9 +448,6 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
   p.split_k = plan.split_k;
   p.kt_per_slice = (int)((desc->K + k->bk - 1) / k->bk) / plan.split_k;
   p.partial = plan.split_k > 1 || plan.tail_split > 1 ? workspace : nullptr;
-#ifdef FRISK_WGPROBE
-  p.partial = workspace;
-#endif
   p.tail_split = plan.tail_split;
   p.tail_tiles = plan.tail_tiles;
   p.tail_from = p.tiles_m * p.tiles_n - plan.tail_tiles;
@@ -564,6 +561,70 @@ int frisk_hip_copy(int src_dtype, const void* src, int64_t src_ld, int dst_dtype
   const int vec = rows_on_16_bytes(src_dtype, src, src_ld) && rows_on_16_bytes(dst_dtype, dst, dst_ld);
   hipError_t e = launch_copy(src_dtype, src, src_ld, dst_dtype, dst, dst_ld, rows, cols, vec, (hipStream_t)stream);
   if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "copy launch failed: %s", hipGetErrorString(e));
+  return FRISK_OK;
+}
+
+int frisk_hip_copy_tiles(int src_dtype, const void* src, int64_t src_ld, int dst_dtype, void* dst, int64_t dst_ld, int64_t tile_rows, int64_t tile_cols,
+                         int64_t n0, int64_t src_step0, int64_t dst_step0, int64_t n1, int64_t src_step1, int64_t dst_step1, void* stream) {
+  const int64_t view_rows = (n0 == 0 || n1 == 0) ? 0 : tile_rows;  // no tile: no pointer is looked at
+  if (int st = check_view("tiled copy source", src_dtype, src, view_rows, tile_cols, src_ld)) return st;
+  if (int st = check_view("tiled copy destination", dst_dtype, dst, view_rows, tile_cols, dst_ld)) return st;
+  if (n0 < 0 || n1 < 0 || src_step0 < 0 || src_step1 < 0 || dst_step0 < 0 || dst_step1 < 0) return fail(FRISK_ERR_SHAPE, "tiled copy: negative tile count or step");
+  if (n0 > INT32_MAX || n1 > INT32_MAX || n0 * n1 > INT32_MAX) return fail(FRISK_ERR_SHAPE, "tiled copy: more than 2^31-1 tiles");
+  if (tile_rows == 0 || tile_cols == 0 || n0 == 0 || n1 == 0) return FRISK_OK;
+  if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
+  const int ss = elem_size(src_dtype), ds = elem_size(dst_dtype);
+  const bool steps16 = (src_step0 * ss) % 16 == 0 && (src_step1 * ss) % 16 == 0 && (dst_step0 * ds) % 16 == 0 && (dst_step1 * ds) % 16 == 0;
+  const int vec = steps16 && rows_on_16_bytes(src_dtype, src, src_ld) && rows_on_16_bytes(dst_dtype, dst, dst_ld);
+  TilePlacement t;
+  t.n0 = n0; t.n1 = n1; t.src_step0 = src_step0; t.src_step1 = src_step1; t.dst_step0 = dst_step0; t.dst_step1 = dst_step1;
+  hipError_t e = launch_copy_tiles(src_dtype, src, src_ld, dst_dtype, dst, dst_ld, tile_rows, tile_cols, t, vec, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "tiled copy launch failed: %s", hipGetErrorString(e));
+  return FRISK_OK;
+}
+
+int frisk_hip_elementwise(const frisk_elementwise_desc* d, const void* const* inputs, void* out, void* stream) {
+  if (!d) return fail(FRISK_ERR_NULL, "elementwise descriptor is null");
+  if (d->abi_version != FRISK_HIP_ABI_VERSION) return fail(FRISK_ERR_ABI, "descriptor abi_version %d, library %d", d->abi_version, FRISK_HIP_ABI_VERSION);
+  if (d->n_inputs < 0 || d->n_inputs > FRISK_EW_MAX_INPUTS) return fail(FRISK_ERR_ARGUMENT, "elementwise: %d operands, at most %d", d->n_inputs, FRISK_EW_MAX_INPUTS);
+  if (d->n_ops < 1 || d->n_ops > FRISK_EW_MAX_OPS) return fail(FRISK_ERR_ARGUMENT, "elementwise: a program of %d steps, 1 to %d allowed", d->n_ops, FRISK_EW_MAX_OPS);
+  if (int st = check_view("elementwise output", d->out_dtype, out, d->rows, d->cols, d->out_ld)) return st;
+  if (d->n_inputs > 0 && !inputs) return fail(FRISK_ERR_NULL, "elementwise: the operand pointer array is null");
+  // the program on a counting stack: never empty when it pops, never deeper than the interpreter's registers, one value left
+  int depth = 0;
+  for (int i = 0; i < d->n_ops; ++i) {
+    const int op = d->op[i];
+    if (op < FRISK_EW_INPUT || op > FRISK_EW_LOG2) return fail(FRISK_ERR_ARGUMENT, "elementwise: unknown opcode %d at step %d", op, i);
+    if (op == FRISK_EW_INPUT && (d->arg[i] < 0 || d->arg[i] >= d->n_inputs)) return fail(FRISK_ERR_ARGUMENT, "elementwise: step %d reads operand %d of %d", i, d->arg[i], d->n_inputs);
+    const int pops = op <= FRISK_EW_CONST ? 0 : (op >= FRISK_EW_NEG ? 1 : 2);
+    if (depth < pops) return fail(FRISK_ERR_ARGUMENT, "elementwise: step %d pops an empty stack", i);
+    depth += 1 - pops;
+    if (depth > FRISK_EW_MAX_STACK) return fail(FRISK_ERR_ARGUMENT, "elementwise: the program needs a stack deeper than %d", FRISK_EW_MAX_STACK);
+  }
+  if (depth != 1) return fail(FRISK_ERR_ARGUMENT, "elementwise: the program leaves %d values, not one", depth);
+  if (d->rows == 0 || d->cols == 0) return FRISK_OK;
+  EwParams p{};
+  // a dense problem (every operand walked, every row following the one before) is one long row
+  bool dense = d->out_ld == d->cols;
+  for (int k = 0; k < d->n_inputs; ++k) dense = dense && d->in_col_stride[k] == 1 && d->in_row_stride[k] == d->cols;
+  p.rows = dense ? 1 : d->rows;
+  p.cols = dense ? d->rows * d->cols : d->cols;
+  bool vec = p.cols % 8 == 0 && rows_on_16_bytes(d->out_dtype, out, dense ? 0 : d->out_ld);
+  for (int k = 0; k < d->n_inputs; ++k) {
+    const int dt = d->in_dtype[k];
+    if (dt != FRISK_F32 && dt != FRISK_F16 && dt != FRISK_BF16) return fail(FRISK_ERR_DTYPE, "elementwise operand %d: element type %d is not f32, f16 or bf16", k, dt);
+    if (d->in_col_stride[k] != 0 && d->in_col_stride[k] != 1) return fail(FRISK_ERR_SHAPE, "elementwise operand %d: column stride %d is not 0 or 1", k, d->in_col_stride[k]);
+    if (d->in_row_stride[k] < 0) return fail(FRISK_ERR_SHAPE, "elementwise operand %d: negative row stride", k);
+    if (!inputs[k]) return fail(FRISK_ERR_NULL, "elementwise operand %d: pointer is null", k);
+    if ((uintptr_t)inputs[k] & (uintptr_t)(elem_size(dt) - 1)) return fail(FRISK_ERR_ALIGNMENT, "elementwise operand %d: pointer is not aligned to its element size", k);
+    if (d->in_col_stride[k] == 1) vec = vec && rows_on_16_bytes(dt, inputs[k], dense ? 0 : d->in_row_stride[k]);
+    p.in[k] = inputs[k]; p.in_row_stride[k] = d->in_row_stride[k]; p.in_dtype[k] = dt; p.in_col_stride[k] = d->in_col_stride[k];
+  }
+  if (!device_ok()) return fail(FRISK_ERR_DEVICE, "no gfx950 device is current");
+  p.out = out; p.out_ld = d->out_ld; p.out_dtype = d->out_dtype; p.n_ops = d->n_ops;
+  for (int i = 0; i < d->n_ops; ++i) { p.op[i] = d->op[i]; p.arg[i] = d->arg[i]; p.imm[i] = d->imm[i]; }
+  hipError_t e = launch_elementwise(p, vec ? 1 : 0, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(FRISK_ERR_DEVICE, "elementwise launch failed: %s", hipGetErrorString(e));
   return FRISK_OK;
 }
 

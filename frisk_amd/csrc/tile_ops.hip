@@ -74,8 +74,8 @@ fill_kernel(typename Elem<DT>::T* dst, int64_t rows, int64_t cols, int64_t ld, f
     }
 }
 
-template <int SDT, int DDT, bool ALONG> __global__ void __launch_bounds__(256)
-copy_kernel(const typename Elem<SDT>::T* src, int64_t sld, typename Elem<DDT>::T* dst, int64_t dld, int64_t rows, int64_t cols, int vec_ok, int lanes_log2) {
+template <int SDT, int DDT, bool ALONG> __device__ __forceinline__ void
+copy_window(const typename Elem<SDT>::T* src, int64_t sld, typename Elem<DDT>::T* dst, int64_t dld, int64_t rows, int64_t cols, int vec_ok, int lanes_log2) {
   typedef typename Elem<SDT>::T S;
   typedef typename Elem<DDT>::T D;
   constexpr int G = 16 / (sizeof(S) < sizeof(D) ? sizeof(S) : sizeof(D));  // 16 bytes of the narrower side, 32 of the wider
@@ -120,6 +120,22 @@ copy_kernel(const typename Elem<SDT>::T* src, int64_t sld, typename Elem<DDT>::T
         }
       }
     }
+}
+
+template <int SDT, int DDT, bool ALONG> __global__ void __launch_bounds__(256)
+copy_kernel(const typename Elem<SDT>::T* src, int64_t sld, typename Elem<DDT>::T* dst, int64_t dld, int64_t rows, int64_t cols, int vec_ok, int lanes_log2) {
+  copy_window<SDT, DDT, ALONG>(src, sld, dst, dld, rows, cols, vec_ok, lanes_log2);
+}
+
+// the same window copied once per tile of a placement: z walks the n0 x n1 tiles, each displacing both sides by its steps
+template <int SDT, int DDT, bool ALONG> __global__ void __launch_bounds__(256)
+copy_tiles_kernel(const typename Elem<SDT>::T* src, int64_t sld, typename Elem<DDT>::T* dst, int64_t dld, int64_t rows, int64_t cols, TilePlacement t, int vec_ok,
+                  int lanes_log2) {
+  const int64_t tiles = t.n0 * t.n1;
+  for (int64_t z = blockIdx.z; z < tiles; z += gridDim.z) {
+    const int64_t a = z / t.n1, b = z - a * t.n1;
+    copy_window<SDT, DDT, ALONG>(src + a * t.src_step0 + b * t.src_step1, sld, dst + a * t.dst_step0 + b * t.dst_step1, dld, rows, cols, vec_ok, lanes_log2);
+  }
 }
 
 // ------------------------------------------------------------------ reduce
@@ -341,6 +357,19 @@ template <int SDT, int DDT> hipError_t copy_t(const void* src, int64_t sld, void
   return hipGetLastError();
 }
 
+template <int SDT, int DDT> hipError_t copy_tiles_t(const void* src, int64_t sld, void* dst, int64_t dld, int64_t rows, int64_t cols, const TilePlacement& t, int vec_ok,
+                                                    hipStream_t s) {
+  typedef typename Elem<SDT>::T S;
+  typedef typename Elem<DDT>::T D;
+  constexpr int G = 16 / (sizeof(S) < sizeof(D) ? sizeof(S) : sizeof(D));
+  WalkLaunch w(rows, (cols + G - 1) / G);
+  const int64_t tiles = t.n0 * t.n1;
+  w.grid.z = (unsigned)(tiles > 65535 ? 65535 : tiles);
+  if (w.along) hipLaunchKernelGGL((copy_tiles_kernel<SDT, DDT, true>), w.grid, dim3(256), 0, s, (const S*)src, sld, (D*)dst, dld, rows, cols, t, vec_ok, w.lanes_log2);
+  else hipLaunchKernelGGL((copy_tiles_kernel<SDT, DDT, false>), w.grid, dim3(256), 0, s, (const S*)src, sld, (D*)dst, dld, rows, cols, t, vec_ok, w.lanes_log2);
+  return hipGetLastError();
+}
+
 // a launch may hold fewer than 2^32 lanes: grids are capped and work-groups loop
 constexpr int64_t kMaxGrid = 1 << 22;
 
@@ -410,6 +439,16 @@ hipError_t launch_fill(int dtype, void* dst, int64_t rows, int64_t cols, int64_t
     case FRISK_F16: return fill_t<FRISK_F16>(dst, rows, cols, ld, value, vec_ok, s);
     default: return fill_t<FRISK_BF16>(dst, rows, cols, ld, value, vec_ok, s);
   }
+}
+
+hipError_t launch_copy_tiles(int sdt, const void* src, int64_t sld, int ddt, void* dst, int64_t dld, int64_t rows, int64_t cols, const TilePlacement& t, int vec_ok,
+                             hipStream_t s) {
+#define FRISK_COPY_CASE(S, D) if (sdt == S && ddt == D) return copy_tiles_t<S, D>(src, sld, dst, dld, rows, cols, t, vec_ok, s);
+  FRISK_COPY_CASE(FRISK_F32, FRISK_F32) FRISK_COPY_CASE(FRISK_F32, FRISK_F16) FRISK_COPY_CASE(FRISK_F32, FRISK_BF16)
+  FRISK_COPY_CASE(FRISK_F16, FRISK_F32) FRISK_COPY_CASE(FRISK_F16, FRISK_F16) FRISK_COPY_CASE(FRISK_F16, FRISK_BF16)
+  FRISK_COPY_CASE(FRISK_BF16, FRISK_F32) FRISK_COPY_CASE(FRISK_BF16, FRISK_F16) FRISK_COPY_CASE(FRISK_BF16, FRISK_BF16)
+#undef FRISK_COPY_CASE
+  return hipErrorInvalidValue;
 }
 
 hipError_t launch_copy(int sdt, const void* src, int64_t sld, int ddt, void* dst, int64_t dld, int64_t rows, int64_t cols, int vec_ok, hipStream_t s) {

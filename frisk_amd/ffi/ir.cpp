@@ -797,6 +797,8 @@ void init_ffi_ir(py::module_&& m) {
       .def("create_subf", [](Builder& b, Value l, Value r) { return b.scalar_op("arith.subf", {l, r}); })
       .def("create_divf", [](Builder& b, Value l, Value r) { return b.scalar_op("arith.divf", {l, r}); })
       .def("create_maxnumf", [](Builder& b, Value l, Value r) { return b.scalar_op("arith.maxnumf", {l, r}); })
+      .def("create_minnumf", [](Builder& b, Value l, Value r) { return b.scalar_op("arith.minnumf", {l, r}); })
+      .def("create_negf", [](Builder& b, Value x) { return b.scalar_op("arith.negf", {x}); })
       .def("create_exp2", [](Builder& b, Value x) { return b.scalar_op("math.exp2", {x}); })
       .def("create_log2", [](Builder& b, Value x) { return b.scalar_op("math.log2", {x}); })
       .def("create_extf", [](Builder& b, Value x, Type to) { return b.cast_op("arith.extf", x, to); })

@@ -1122,17 +1122,19 @@ inline GemmProgram match_tiled_gemm(Operation* kernel, Operation* module = nullp
 // index map applied to its index operands; extents follow the op (default: the destination shape left-padded with 1s,
 // FriskOps.cpp:1564-1591).  Copies may sit under frisk.parallel and frisk.for and be indexed by their grid indices and
 // induction variables: the windows of all iterations must then tile one rectangle of each side without gaps or overlap
-// (every index moves the window by whole tiles along one dimension, the same one on both sides), and the copy is lowered
-// as one copy of that rectangle.  A tile may also pass through one frisk.alloc_buffer (global -> buffer -> global in
+// (every index moves the window by whole tiles along one dimension); when every index moves both sides alike the copy is
+// lowered as one copy of that rectangle, otherwise (tiles placed transposed, say) as one tile-by-tile copy.  A tile may also pass through one frisk.alloc_buffer (global -> buffer -> global in
 // the same block, the buffer used by nothing else): the pair is lowered as the direct copy.  Fill and reduce take whole
 // arguments and must not be repeated by an enclosing grid or loop.
 struct TileOpDesc {
-  enum Kind { Fill, Copy, Reduce } kind = Fill;
+  enum Kind { Fill, Copy, Reduce, CopyTiles } kind = Fill;
   int arg_src = -1, arg_dst = -1;          // kernel argument positions (fill: arg_dst only)
   Type elem_src, elem_dst;
   int64_t src_offset = 0, dst_offset = 0;  // elements from the start of the argument
   int64_t rows = 0, cols = 0, src_ld = 0, dst_ld = 0;
   double value = 0.0;                      // fill
+  // CopyTiles: rows x cols is one tile; tile (a, b) of n0 x n1 lies a * step0 + b * step1 elements further on each side
+  int64_t n0 = 1, n1 = 1, src_step0 = 0, src_step1 = 0, dst_step0 = 0, dst_step1 = 0;
   std::string reduce_kind;                 // add | mul | min | max
   int64_t dim = 0;
   bool clear = true;
@@ -1338,12 +1340,31 @@ inline std::vector<TileOpDesc> match_data_movement(Operation* kernel) {
           else fail("source and destination windows of a copy have different shapes");
         } else {
           if (ss.tr != ts.tr || ss.tc != ts.tc) fail("source and destination tiles of a tiled copy have different shapes");
+          bool same_placement = true;
+          std::vector<size_t> movers;
           for (size_t v = 0; v < vars.size(); ++v) {
             if (vars[v].count <= 1) continue;
             if (ss.moves[v].first < 0 || ts.moves[v].first < 0) fail("an enclosing grid index or induction variable does not move both windows of a copy: its iterations would repeat or overwrite one another");
-            if (ss.moves[v] != ts.moves[v]) fail("an index moves the source and destination windows of a tiled copy differently");
+            same_placement = same_placement && ss.moves[v] == ts.moves[v];
+            movers.push_back(v);
           }
-          d.rows = ss.rows; d.cols = ss.cols;  // equal on both sides by the checks above
+          if (same_placement) {
+            d.rows = ss.rows; d.cols = ss.cols;  // equal on both sides by the checks above
+          } else {
+            // The tiles land elsewhere than they came from (placed transposed, or at another pitch): each side still tiles
+            // its own rectangle without gap or overlap (side_of), so every destination element is written once.  One
+            // launch copies tile by tile, each index displacing the two sides by its own steps.
+            if (movers.size() > 2) fail("a tiled copy that rearranges its tiles may be indexed by at most two grid indices or induction variables");
+            d.kind = TileOpDesc::CopyTiles;
+            d.rows = ss.tr; d.cols = ss.tc;
+            auto step = [](const std::pair<int, int64_t>& mv, int64_t ld) { return mv.first == 0 ? mv.second : mv.second * ld; };
+            d.n0 = vars[movers[0]].count;
+            d.src_step0 = step(ss.moves[movers[0]], s.cols); d.dst_step0 = step(ts.moves[movers[0]], t.cols);
+            if (movers.size() == 2) {
+              d.n1 = vars[movers[1]].count;
+              d.src_step1 = step(ss.moves[movers[1]], s.cols); d.dst_step1 = step(ts.moves[movers[1]], t.cols);
+            }
+          }
         }
       } else if (op->name == "frisk.reduce") {
         if (repeated) fail("a reduce under a grid or a loop would run once per iteration");

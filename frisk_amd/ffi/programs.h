@@ -18,6 +18,7 @@
 // indices; mul and add match in either operand order.
 #pragma once
 #include <cmath>
+#include <functional>
 #include <map>
 #include <string>
 #include <vector>
@@ -653,6 +654,137 @@ inline AttentionProgram match_attention(Operation* kernel, Operation* module = n
   for (Value t : {gk, gv, go}) if (!g.elem.equals(t.type().element())) m.bad("Q, K, V and O must have one element type");
   check_4d(top[7], true, go, 2, bx, 1, 0, g.tile_q, g.head_dim, "storing the output tile");
   if (!is_zero_origin(linear_origin(m, top[7], false, {}))) m.bad("storing the output tile: the shared side must start at 0");
+  return g;
+}
+
+// ------------------------------------------------------------------ free-standing frisk.block bodies
+// A kernel whose entry block holds nothing but frisk.block ops (and the constants they use): every block runs its body
+// for each point of a rank-1 or rank-2 iteration space, the body loads from kernel arguments, computes with arith / math
+// ops and stores one value per point (FriskOps.td:143-190).  Each block becomes one postfix program for
+// frisk_hip_elementwise; blocks run in program order.
+// A load or store index must be linear in the block's induction variables.  With (row, col) = (0, i) for a rank-1 block
+// and (i, j) for a rank-2 one, an access is  offset + row * row_stride + col * col_stride  elements into its argument;
+// loads may broadcast (col stride 0, row stride 0), the store must walk its row (col stride 1) and give every point an
+// element of its own.
+struct EwOperand {
+  int arg = -1;
+  Type elem;
+  int64_t offset = 0, row_stride = 0, col_stride = 0;
+  bool operator==(const EwOperand& o) const { return arg == o.arg && offset == o.offset && row_stride == o.row_stride && col_stride == o.col_stride; }
+};
+struct EwStep { std::string op; int operand = -1; double value = 0.0; };  // op: input | const | add sub mul div max min neg exp2 log2
+struct EwBlock {
+  int64_t rows = 1, cols = 1;
+  EwOperand out;
+  std::vector<EwOperand> inputs;
+  std::vector<EwStep> steps;
+  int max_stack = 0;
+};
+struct EwProgram {
+  std::string kernel_name, target;
+  std::vector<EwBlock> blocks;
+};
+
+inline bool is_elementwise_kernel(Operation* kernel) {
+  if (!kernel || kernel->name != "frisk.kernel" || kernel->regions.empty() || kernel->regions[0]->blocks.empty()) return false;
+  bool any = false;
+  for (Operation* op : kernel->regions[0]->blocks[0]->ops) {
+    if (op->name == "frisk.block") any = true;
+    else if (op->name != "arith.constant" && op->name != "frisk.end") return false;
+  }
+  return any;
+}
+
+inline EwProgram match_elementwise(Operation* kernel, Operation* module = nullptr) {
+  const BodyMatcher m("an elementwise kernel");
+  if (!kernel || kernel->name != "frisk.kernel") m.bad("expected a frisk.kernel");
+  if (kernel->regions.empty() || kernel->regions[0]->blocks.empty()) m.bad("kernel has no entry block");
+  EwProgram g;
+  g.kernel_name = kernel->attr("sym_name") ? kernel->attr("sym_name")->s : std::string();
+  g.target = "gfx950";
+  for (const Operation* scope : {(const Operation*)kernel, (const Operation*)module})
+    if (scope) if (auto t = scope->attr("frisk.target")) { g.target = t->s; break; }
+  if (g.target.rfind("gfx950", 0) != 0) m.bad("frisk.target '" + g.target + "' is not gfx950");
+  for (Operation* op : kernel->regions[0]->blocks[0]->ops) {
+    if (op->name == "arith.constant" || op->name == "frisk.end") continue;
+    if (op->name != "frisk.block") m.bad("operation " + op->name + " beside the blocks");
+    const auto& ranges = op->attr("ranges")->ints;
+    if (ranges.empty() || ranges.size() > 2) m.bad("a block of rank " + std::to_string(ranges.size()) + " (1 or 2 supported)");
+    EwBlock b;
+    b.rows = ranges.size() == 2 ? ranges[0] : 1;
+    b.cols = ranges.back();
+    const BodyMatcher::Store st = m.single_store(op);
+    // an access as offset + row * rs + col * cs, from the index expressions over the induction variables
+    auto operand_of = [&](Value buffer, const std::vector<AffineExpr>& index, const char* what) {
+      EwOperand o;
+      o.arg = kernel_arg_index(kernel, buffer);
+      if (o.arg < 0 || !buffer.type().is_memref()) m.bad(std::string(what) + " is not a kernel argument memref");
+      const auto& sh = buffer.type().impl->shape;
+      if (sh.empty() || sh.size() > 2) m.bad(std::string(what) + " must have rank 1 or 2");
+      for (int64_t d : sh) if (d < 0) m.bad(std::string(what) + " has a dynamic extent");
+      if (index.size() != sh.size()) m.bad(std::string(what) + " is indexed with " + std::to_string(index.size()) + " expressions for rank " + std::to_string(sh.size()));
+      o.elem = buffer.type().element();
+      const size_t nv = ranges.size();
+      auto at = [&](int64_t i, int64_t j) {  // element offset at induction values (i, j)
+        std::vector<int64_t> dims = nv == 2 ? std::vector<int64_t>{i, j} : std::vector<int64_t>{i};
+        int64_t off = 0;
+        for (size_t d = 0; d < sh.size(); ++d) {
+          const int64_t v = index[d].eval(dims, {});
+          off = off * sh[d] + v;
+        }
+        return off;
+      };
+      const int64_t c0 = at(0, 0), ci = at(1, 0) - c0, cj = nv == 2 ? at(0, 1) - c0 : 0;
+      if (at(3, nv == 2 ? 5 : 0) != c0 + 3 * ci + (nv == 2 ? 5 * cj : 0)) m.bad(std::string(what) + " is not indexed linearly by the block's induction variables");
+      o.offset = c0;
+      o.row_stride = nv == 2 ? ci : 0;
+      o.col_stride = nv == 2 ? cj : ci;
+      // every point inside the memref: the corners of the iteration space bound a linear access
+      int64_t total = 1;
+      for (int64_t d : sh) total *= d;
+      for (size_t d = 0; d < sh.size(); ++d)
+        for (int64_t i : {int64_t(0), ranges[0] - 1})
+          for (int64_t j : {int64_t(0), nv == 2 ? ranges[1] - 1 : int64_t(0)}) {
+            std::vector<int64_t> dims = nv == 2 ? std::vector<int64_t>{i, j} : std::vector<int64_t>{i};
+            const int64_t v = index[d].eval(dims, {});
+            if (v < 0 || v >= sh[d]) m.bad(std::string(what) + " is indexed outside its extents");
+          }
+      (void)total;
+      if (o.row_stride < 0 || o.col_stride < 0) m.bad(std::string(what) + " is walked backwards");
+      return o;
+    };
+    b.out = operand_of(st.buffer, st.index, "the stored buffer");
+    if (b.out.col_stride != 1) m.bad("the store must walk a row of its buffer (column stride " + std::to_string(b.out.col_stride) + ")");
+    if (b.rows > 1 && b.out.row_stride < b.cols) m.bad("the stores of different rows overlap");
+    // postfix program of the stored expression; the operand pushed first is the left one
+    int depth = 0;
+    std::function<void(const Expr&)> emit = [&](const Expr& e) {
+      if (e.op == "load") {
+        const EwOperand o = operand_of(e.buffer, e.index, "a loaded buffer");
+        if (o.col_stride > 1) m.bad("a load with column stride " + std::to_string(o.col_stride) + " (0 or 1 supported)");
+        size_t k = 0;
+        while (k < b.inputs.size() && !(b.inputs[k] == o)) ++k;
+        if (k == b.inputs.size()) b.inputs.push_back(o);
+        b.steps.push_back(EwStep{"input", (int)k, 0.0});
+        b.max_stack = std::max(b.max_stack, ++depth);
+        return;
+      }
+      if (e.op == "const") {
+        b.steps.push_back(EwStep{"const", -1, e.value});
+        b.max_stack = std::max(b.max_stack, ++depth);
+        return;
+      }
+      for (const Expr& k : e.kids) emit(k);
+      b.steps.push_back(EwStep{e.op, -1, 0.0});
+      depth -= (int)e.kids.size() - 1;
+    };
+    emit(st.value);
+    // an in-place block may only read the element it writes
+    for (const EwOperand& o : b.inputs)
+      if (o.arg == b.out.arg && !(o == b.out)) m.bad("a block reads its own output buffer at other elements than the one it writes");
+    g.blocks.push_back(b);
+  }
+  if (g.blocks.empty()) m.bad("the kernel holds no frisk.block");
   return g;
 }
 

@@ -8,6 +8,7 @@
 #include <dlfcn.h>
 
 #include <mutex>
+#include <sstream>
 
 #include "ffi.h"
 #include "frisk_hip.h"
@@ -37,6 +38,8 @@ struct HipLibrary {
   decltype(&frisk_hip_softmax) softmax = nullptr;
   decltype(&frisk_hip_softmax_workspace_bytes) softmax_workspace_bytes = nullptr;
   decltype(&frisk_hip_attention) attention = nullptr;
+  decltype(&frisk_hip_elementwise) elementwise = nullptr;
+  decltype(&frisk_hip_copy_tiles) copy_tiles = nullptr;
 };
 
 HipLibrary g_lib;
@@ -64,7 +67,9 @@ HipLibrary& library() {
   lib.softmax = (decltype(lib.softmax))dlsym(h, "frisk_hip_softmax");
   lib.softmax_workspace_bytes = (decltype(lib.softmax_workspace_bytes))dlsym(h, "frisk_hip_softmax_workspace_bytes");
   lib.attention = (decltype(lib.attention))dlsym(h, "frisk_hip_attention");
-  if (!lib.softmax || !lib.softmax_workspace_bytes || !lib.attention || !lib.plan || !lib.gemm || !lib.last_error || !lib.abi_version || !lib.kernel_name || !lib.fill || !lib.copy || !lib.reduce || !lib.reduce_workspace_bytes)
+  lib.elementwise = (decltype(lib.elementwise))dlsym(h, "frisk_hip_elementwise");
+  lib.copy_tiles = (decltype(lib.copy_tiles))dlsym(h, "frisk_hip_copy_tiles");
+  if (!lib.elementwise || !lib.copy_tiles || !lib.softmax || !lib.softmax_workspace_bytes || !lib.attention || !lib.plan || !lib.gemm || !lib.last_error || !lib.abi_version || !lib.kernel_name || !lib.fill || !lib.copy || !lib.reduce || !lib.reduce_workspace_bytes)
     throw std::runtime_error("frisk runtime: " + g_lib_path + " does not export the frisk_hip entry points");
   if (lib.abi_version() != FRISK_HIP_ABI_VERSION) throw std::runtime_error("frisk runtime: libfrisk_hip.so ABI version mismatch");
   g_lib = lib;
@@ -202,7 +207,12 @@ int reduce_kind_of(const std::string& k) {
 
 py::dict tile_op_dict(const TileOpDesc& d) {
   py::dict o;
-  o["op"] = d.kind == TileOpDesc::Fill ? "fill" : d.kind == TileOpDesc::Copy ? "copy" : "reduce";
+  o["op"] = d.kind == TileOpDesc::Fill ? "fill" : d.kind == TileOpDesc::Copy ? "copy" : d.kind == TileOpDesc::CopyTiles ? "copy_tiles" : "reduce";
+  if (d.kind == TileOpDesc::CopyTiles) {
+    o["tiles"] = py::make_tuple(d.n0, d.n1);
+    o["src_steps"] = py::make_tuple(d.src_step0, d.src_step1);
+    o["dst_steps"] = py::make_tuple(d.dst_step0, d.dst_step1);
+  }
   o["rows"] = d.rows; o["cols"] = d.cols;
   if (d.kind != TileOpDesc::Fill) { o["src"] = d.arg_src; o["src_offset"] = d.src_offset; o["src_ld"] = d.src_ld; o["src_dtype"] = d.elem_src.str(); }
   o["dst"] = d.arg_dst; o["dst_offset"] = d.dst_offset; o["dst_dtype"] = d.elem_dst.str();
@@ -214,8 +224,9 @@ py::dict tile_op_dict(const TileOpDesc& d) {
 
 // Which of the recognised programs a kernel is, by the ops it holds: frisk.block bodies only occur in the softmax and
 // attention programs; two products make the attention program.
-enum class ProgramKind { TiledGemm, OnlineSoftmax, Attention };
+enum class ProgramKind { TiledGemm, OnlineSoftmax, Attention, Elementwise };
 ProgramKind classify(Operation* kernel) {
+  if (is_elementwise_kernel(kernel)) return ProgramKind::Elementwise;  // nothing but free-standing frisk.block ops
   int gemms = 0, blocks = 0;
   std::function<void(Operation*)> walk = [&](Operation* op) {
     if (op->name == "frisk.gemm") ++gemms;
@@ -240,6 +251,73 @@ py::dict softmax_dict(const SoftmaxProgram& g) {
   o["args"] = py::make_tuple(g.arg_src, g.arg_dst);
   o["target"] = g.target;
   return o;
+}
+
+int ew_opcode(const std::string& op) {
+  static const std::map<std::string, int> codes = {{"input", FRISK_EW_INPUT}, {"const", FRISK_EW_CONST}, {"add", FRISK_EW_ADD}, {"sub", FRISK_EW_SUB},
+                                                    {"mul", FRISK_EW_MUL}, {"div", FRISK_EW_DIV}, {"max", FRISK_EW_MAX}, {"min", FRISK_EW_MIN},
+                                                    {"neg", FRISK_EW_NEG}, {"exp2", FRISK_EW_EXP2}, {"log2", FRISK_EW_LOG2}};
+  auto it = codes.find(op);
+  if (it == codes.end()) throw std::invalid_argument("operation '" + op + "' has no elementwise opcode");
+  return it->second;
+}
+
+// the postfix program of a block as text: x<k> operand k, c<value> constant, else the operation
+std::string ew_text(const EwBlock& b) {
+  std::ostringstream os;
+  for (size_t i = 0; i < b.steps.size(); ++i) {
+    if (i) os << ' ';
+    if (b.steps[i].op == "input") os << 'x' << b.steps[i].operand;
+    else if (b.steps[i].op == "const") os << 'c' << b.steps[i].value;
+    else os << b.steps[i].op;
+  }
+  return os.str();
+}
+
+py::dict elementwise_dict(const EwProgram& g) {
+  py::dict o;
+  o["program"] = "elementwise";
+  o["kernel"] = g.kernel_name;
+  o["target"] = g.target;
+  py::list blocks;
+  for (const EwBlock& b : g.blocks) {
+    py::dict d;
+    d["rows"] = b.rows; d["cols"] = b.cols;
+    d["out"] = py::make_tuple(b.out.arg, b.out.offset, b.out.row_stride, b.out.elem.str());
+    py::list ins;
+    for (const EwOperand& x : b.inputs) ins.append(py::make_tuple(x.arg, x.offset, x.row_stride, x.col_stride, x.elem.str()));
+    d["inputs"] = ins;
+    d["postfix"] = ew_text(b);
+    d["stack"] = b.max_stack;
+    blocks.append(d);
+  }
+  o["blocks"] = blocks;
+  return o;
+}
+
+// descriptor of one block for frisk_hip_elementwise; throws what the library would refuse, with the block's own words
+frisk_elementwise_desc ew_desc_of(const EwBlock& b) {
+  if (b.inputs.size() > FRISK_EW_MAX_INPUTS) throw std::invalid_argument("a block body reads " + std::to_string(b.inputs.size()) + " different operands, at most " + std::to_string(FRISK_EW_MAX_INPUTS) + " are supported");
+  if (b.steps.size() > FRISK_EW_MAX_OPS) throw std::invalid_argument("a block body of " + std::to_string(b.steps.size()) + " steps, at most " + std::to_string(FRISK_EW_MAX_OPS) + " are supported");
+  if (b.max_stack > FRISK_EW_MAX_STACK) throw std::invalid_argument("a block body needs an evaluation stack of " + std::to_string(b.max_stack) + ", at most " + std::to_string(FRISK_EW_MAX_STACK) + " is supported");
+  frisk_elementwise_desc d{};
+  d.abi_version = FRISK_HIP_ABI_VERSION;
+  d.n_inputs = (int)b.inputs.size();
+  d.n_ops = (int)b.steps.size();
+  d.out_dtype = dtype_of(b.out.elem);
+  d.rows = b.rows; d.cols = b.cols;
+  d.out_ld = b.rows > 1 ? b.out.row_stride : b.cols;
+  for (size_t k = 0; k < b.inputs.size(); ++k) {
+    d.in_dtype[k] = dtype_of(b.inputs[k].elem);
+    d.in_row_stride[k] = b.inputs[k].row_stride;
+    d.in_col_stride[k] = (int)b.inputs[k].col_stride;
+  }
+  for (size_t i = 0; i < b.steps.size(); ++i) {
+    d.op[i] = ew_opcode(b.steps[i].op);
+    d.arg[i] = b.steps[i].operand < 0 ? 0 : b.steps[i].operand;
+    d.imm[i] = (float)b.steps[i].value;
+  }
+  return d;
 }
 
 py::dict attention_dict(const AttentionProgram& g) {
@@ -270,6 +348,11 @@ void init_ffi_runtime(py::module_&& m) {
     Operation* k = op_of_handle(kernel);
     Operation* mod = module.is_none() ? nullptr : op_of_handle(module);
     switch (classify(k)) {
+      case ProgramKind::Elementwise: {
+        const EwProgram g = match_elementwise(k, mod);
+        for (const EwBlock& b : g.blocks) (void)ew_desc_of(b);  // what the library could not run is refused here already
+        return elementwise_dict(g);
+      }
       case ProgramKind::OnlineSoftmax: return softmax_dict(match_online_softmax(k, mod));
       case ProgramKind::Attention: return attention_dict(match_attention(k, mod));
       default: break;
@@ -279,7 +362,8 @@ void init_ffi_runtime(py::module_&& m) {
     return d;
   }, py::arg("kernel"), py::arg("module") = py::none(),
         "recognise one of the programs of the reference's design sketches and return what it computes: the tiled GEMM "
-        "kernel{parallel{alloc x3, fill, for{copy, copy, gemm}, copy}}, the row softmax with a running log-sum, or the fused attention; pure host");
+        "kernel{parallel{alloc x3, fill, for{copy, copy, gemm}, copy}}, the row softmax with a running log-sum, the fused attention, or a kernel of "
+        "free-standing frisk.block bodies (one postfix program per block); pure host");
 
   m.def("plan", [](py::object kernel, py::object module, const std::string& epilogue, bool retile) {
     GemmProgram g = program_of(kernel, module);
@@ -407,6 +491,9 @@ void init_ffi_runtime(py::module_&& m) {
       int st = 0;
       if (d.kind == TileOpDesc::Fill)
         st = lib.fill(dtype_of(d.elem_dst), ptr(d.arg_dst, d.dst_offset, d.elem_dst), d.rows, d.cols, d.dst_ld, d.value, (void*)stream);
+      else if (d.kind == TileOpDesc::CopyTiles)
+        st = lib.copy_tiles(dtype_of(d.elem_src), ptr(d.arg_src, d.src_offset, d.elem_src), d.src_ld, dtype_of(d.elem_dst), ptr(d.arg_dst, d.dst_offset, d.elem_dst),
+                            d.dst_ld, d.rows, d.cols, d.n0, d.src_step0, d.dst_step0, d.n1, d.src_step1, d.dst_step1, (void*)stream);
       else if (d.kind == TileOpDesc::Copy)
         st = lib.copy(dtype_of(d.elem_src), ptr(d.arg_src, d.src_offset, d.elem_src), d.src_ld, dtype_of(d.elem_dst), ptr(d.arg_dst, d.dst_offset, d.elem_dst),
                       d.dst_ld, d.rows, d.cols, (void*)stream);
@@ -426,6 +513,27 @@ void init_ffi_runtime(py::module_&& m) {
     Operation* k = op_of_handle(kernel);
     Operation* mod = module.is_none() ? nullptr : op_of_handle(module);
     const ProgramKind kind = classify(k);
+    if (kind == ProgramKind::Elementwise) {
+      const EwProgram g = match_elementwise(k, mod);
+      HipLibrary& lib = library();
+      for (const EwBlock& b : g.blocks) {  // program order on one stream: a block sees what the blocks before it stored
+        const frisk_elementwise_desc d = ew_desc_of(b);
+        auto ptr = [&](const EwOperand& o) -> uint64_t {
+          if ((size_t)o.arg >= args.size()) throw std::invalid_argument("launch needs one device pointer per kernel argument");
+          return args[(size_t)o.arg] + (uint64_t)o.offset * (uint64_t)(o.elem.bit_width() / 8);
+        };
+        const void* inputs[FRISK_EW_MAX_INPUTS] = {};
+        for (size_t i = 0; i < b.inputs.size(); ++i) inputs[i] = (const void*)ptr(b.inputs[i]);
+        void* out = (void*)ptr(b.out);
+        int st;
+        {
+          py::gil_scoped_release release;
+          st = lib.elementwise(&d, inputs, out, (void*)stream);
+        }
+        if (st) throw std::runtime_error(std::string("frisk_hip_elementwise: ") + lib.last_error() + " (status " + std::to_string(st) + ")");
+      }
+      return;
+    }
     if (kind == ProgramKind::OnlineSoftmax) {
       const SoftmaxProgram g = match_online_softmax(k, mod);
       if (args.size() < (size_t)std::max(g.arg_src, g.arg_dst) + 1) throw std::invalid_argument("launch needs one device pointer per kernel argument");
@@ -473,7 +581,8 @@ void init_ffi_runtime(py::module_&& m) {
     if (st) throw std::runtime_error(std::string("frisk_hip_gemm: ") + lib.last_error() + " (status " + std::to_string(st) + ")");
   }, py::arg("kernel"), py::arg("args"), py::arg("stream") = 0, py::arg("module") = py::none(), py::arg("epilogue") = "none",
      py::arg("scale_a") = 0, py::arg("scale_b") = 0, py::arg("retile") = true,
-     "asynchronous launch on `stream` (a hipStream_t value) of a recognised program (tiled GEMM, online softmax, fused attention); "
+     "asynchronous launch on `stream` (a hipStream_t value) of a recognised program (tiled GEMM, online softmax, fused attention, "
+     "free-standing frisk.block bodies); "
      "`args` holds one raw device pointer per kernel argument");
 }
 

@@ -57,6 +57,18 @@ class AttentionDesc(ctypes.Structure):
                 ("k_transposed", ctypes.c_uint8), ("reserved", ctypes.c_uint8 * 3)]
 
 
+EW_MAX_INPUTS, EW_MAX_OPS, EW_MAX_STACK = 8, 48, 6
+EW_OPS = {"input": 0, "const": 1, "add": 2, "sub": 3, "mul": 4, "div": 5, "max": 6, "min": 7, "neg": 8, "exp2": 9, "log2": 10}
+
+
+class ElementwiseDesc(ctypes.Structure):
+    _fields_ = [("abi_version", ctypes.c_int32), ("n_inputs", ctypes.c_int32), ("n_ops", ctypes.c_int32), ("out_dtype", ctypes.c_int32),
+                ("rows", ctypes.c_int64), ("cols", ctypes.c_int64), ("out_ld", ctypes.c_int64),
+                ("in_dtype", ctypes.c_int32 * EW_MAX_INPUTS), ("in_col_stride", ctypes.c_int32 * EW_MAX_INPUTS),
+                ("in_row_stride", ctypes.c_int64 * EW_MAX_INPUTS), ("op", ctypes.c_int32 * EW_MAX_OPS), ("arg", ctypes.c_int32 * EW_MAX_OPS),
+                ("imm", ctypes.c_float * EW_MAX_OPS)]
+
+
 globals().update({name: code for code, name in STATUS_NAMES.items()})  # OK, ERR_NULL, ... as module constants
 
 
@@ -72,7 +84,7 @@ EXPORTS = ["frisk_hip_init", "frisk_hip_abi_version", "frisk_hip_last_error", "f
            "frisk_hip_gemm", "frisk_hip_lds_access_cycles", "frisk_hip_lds_search", "frisk_hip_lds_search_atom", "frisk_hip_lds_offset", "frisk_hip_wave_partition",
            "frisk_hip_kernel_count", "frisk_hip_kernel_name", "frisk_hip_fill", "frisk_hip_copy", "frisk_hip_reduce",
            "frisk_hip_reduce_workspace_bytes", "frisk_hip_attention", "frisk_hip_softmax", "frisk_hip_softmax_workspace_bytes",
-           "frisk_hip_gemm_static_ws", "frisk_hip_static_workspace_bytes"]
+           "frisk_hip_gemm_static_ws", "frisk_hip_static_workspace_bytes", "frisk_hip_copy_tiles", "frisk_hip_elementwise"]
 
 
 def lib():
@@ -109,6 +121,8 @@ def lib():
     i64, vp = ctypes.c_int64, ctypes.c_void_p
     L.frisk_hip_fill.argtypes = [ctypes.c_int, vp, i64, i64, i64, ctypes.c_double, vp]
     L.frisk_hip_copy.argtypes = [ctypes.c_int, vp, i64, ctypes.c_int, vp, i64, i64, i64, vp]
+    L.frisk_hip_copy_tiles.argtypes = [ctypes.c_int, vp, i64, ctypes.c_int, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64, vp]
+    L.frisk_hip_elementwise.argtypes = [ctypes.POINTER(ElementwiseDesc), ctypes.POINTER(ctypes.c_void_p), vp, vp]
     L.frisk_hip_reduce_workspace_bytes.restype = ctypes.c_size_t
     L.frisk_hip_reduce_workspace_bytes.argtypes = [ctypes.c_int, i64, i64, ctypes.c_int]
     L.frisk_hip_softmax.argtypes = [ctypes.c_int, vp, i64, vp, i64, i64, i64, ctypes.c_float, vp, vp, ctypes.c_size_t, vp]
@@ -192,6 +206,39 @@ def fill(dtype, dst_ptr, rows, cols, ld, value, stream=None):
 def copy(src_dtype, src_ptr, src_ld, dst_dtype, dst_ptr, dst_ld, rows, cols, stream=None):
     """frisk.copy of a rows x cols window, converting between f32 / f16 / bf16 when the types differ"""
     _check(lib().frisk_hip_copy(src_dtype, src_ptr, src_ld, dst_dtype, dst_ptr, dst_ld, rows, cols, stream))
+
+
+def copy_tiles(src_dtype, src_ptr, src_ld, dst_dtype, dst_ptr, dst_ld, tile_rows, tile_cols, n0, src_step0, dst_step0, n1=1, src_step1=0, dst_step1=0, stream=None):
+    """n0 x n1 tiles of tile_rows x tile_cols, tile (a, b) displaced by a * step0 + b * step1 elements on either side"""
+    _check(lib().frisk_hip_copy_tiles(src_dtype, src_ptr, src_ld, dst_dtype, dst_ptr, dst_ld, tile_rows, tile_cols, n0, src_step0, dst_step0, n1, src_step1, dst_step1,
+                                      stream))
+
+
+def make_elementwise_desc(program, inputs, out_dtype, rows, cols, out_ld=None):
+    """program: postfix steps, each ("input", k) | ("const", value) | "add" | "sub" | "mul" | "div" | "max" | "min" | "neg" | "exp2" | "log2";
+    inputs: one (dtype, row_stride, col_stride) per operand"""
+    d = ElementwiseDesc()
+    d.abi_version = ABI_VERSION
+    d.n_inputs, d.n_ops, d.out_dtype = len(inputs), len(program), out_dtype
+    d.rows, d.cols, d.out_ld = rows, cols, cols if out_ld is None else out_ld
+    if len(inputs) > EW_MAX_INPUTS or len(program) > EW_MAX_OPS:
+        raise ValueError("an elementwise program holds at most %d operands and %d steps" % (EW_MAX_INPUTS, EW_MAX_OPS))
+    for k, (dt, rs, cs) in enumerate(inputs):
+        d.in_dtype[k], d.in_row_stride[k], d.in_col_stride[k] = dt, rs, cs
+    for i, step in enumerate(program):
+        name, val = (step, None) if isinstance(step, str) else step
+        d.op[i] = EW_OPS[name]
+        if name == "input":
+            d.arg[i] = int(val)
+        elif name == "const":
+            d.imm[i] = float(val)
+    return d
+
+
+def elementwise(desc, input_ptrs, out_ptr, stream=None):
+    """frisk.block body as one interpreted kernel: out = program(inputs) for every point (asynchronous on `stream`)"""
+    arr = (ctypes.c_void_p * max(1, len(input_ptrs)))(*input_ptrs)
+    _check(lib().frisk_hip_elementwise(ctypes.byref(desc), arr, out_ptr, stream))
 
 
 def reduce_workspace_bytes(dtype, rows, cols, dim):

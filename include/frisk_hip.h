@@ -227,6 +227,17 @@ int frisk_hip_fill(int dtype, void* dst, int64_t rows, int64_t cols, int64_t ld,
 int frisk_hip_copy(int src_dtype, const void* src, int64_t src_ld, int dst_dtype, void* dst, int64_t dst_ld, int64_t rows,
                    int64_t cols, void* stream);
 
+/* frisk.copy under frisk.parallel / frisk.for whose windows are placed by index maps (FriskOps.td:348-389; maps, index
+ * operands and extents FriskOps.cpp:1551-1683): n0 x n1 tiles of tile_rows x tile_cols elements.  Tile (a, b) is read
+ * at element offset a * src_step0 + b * src_step1 from `src` and written at a * dst_step0 + b * dst_step1 from `dst`;
+ * inside a tile consecutive rows lie src_ld / dst_ld elements apart.  One launch for placements that a single window
+ * copy cannot express, e.g. tiles placed transposed (the tile at block (a, b) of the source going to block (b, a) of the
+ * destination; the elements of a tile keep their order, as frisk.copy copies a window).  Destination tiles must not
+ * overlap one another or the source.  Steps are non-negative; n0 * n1 <= 2^31 - 1. */
+int frisk_hip_copy_tiles(int src_dtype, const void* src, int64_t src_ld, int dst_dtype, void* dst, int64_t dst_ld, int64_t tile_rows,
+                         int64_t tile_cols, int64_t n0, int64_t src_step0, int64_t dst_step0, int64_t n1, int64_t src_step1,
+                         int64_t dst_step1, void* stream);
+
 /* frisk.reduce (FriskOps.td:412-441, verifier FriskOps.cpp:1733-1767): reduces the rows x cols view along
  * `dim` (0: over rows, dst has cols entries; 1: over columns, dst has rows entries) with `kind`.  Arithmetic
  * in fp32, result rounded to dtype.  clear = 1: dst := reduction; clear = 0: dst := kind(dst, reduction).
@@ -248,6 +259,54 @@ int frisk_hip_reduce(int dtype, const void* src, int64_t rows, int64_t cols, int
 size_t frisk_hip_softmax_workspace_bytes(int dtype, int64_t rows, int64_t cols);
 int frisk_hip_softmax(int dtype, const void* src, int64_t src_ld, void* dst, int64_t dst_ld, int64_t rows, int64_t cols,
                       float scale_log2, float* lse, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * frisk.block (include/Dialect/Frisk/IR/FriskOps.td:143-190; built by create_block_op, ffi/ir.cpp:383-394): a body of
+ * affine.load / arith / math / affine.store ops run for every point of an iteration space.  The reference defines the
+ * op and lowers it nowhere.  Here a body that stores one value per point is run as ONE kernel that interprets the
+ * stored expression, given as a postfix program: no code is generated at run time.
+ *   out[r][c] = program(in_0[r][c], in_1[r][c], ...)   for r < rows, c < cols   (a rank-1 block is rows = 1)
+ * Operand k is read at element  r * in_row_stride[k] + c * in_col_stride[k]  from inputs[k]: col stride 1 walks a row,
+ * col stride 0 broadcasts one element along the row, row stride 0 the same row to every row (so a per-row scalar x[r]
+ * is (1, 0), a per-column vector (0, 1), a scalar (0, 0)).  Element types F32, F16, BF16, per operand.  The program
+ * is evaluated on a stack in fp32 (width casts inside a body are transparent) and the result rounded once to out_dtype:
+ *   FRISK_EW_INPUT  push operand arg[i]          FRISK_EW_CONST  push imm[i]
+ *   ADD SUB MUL DIV MAX MIN   pop b, pop a, push a op b   (MAX / MIN ignore a NaN operand: arith.maxnumf / minnumf)
+ *   NEG EXP2 LOG2             replace the top            (math.exp2 / math.log2: base 2)
+ * A program must leave exactly one value and never hold more than FRISK_EW_MAX_STACK.  out must not overlap an input
+ * other than element for element (in place is allowed).  Asynchronous on `stream`; nothing is allocated.
+ * ------------------------------------------------------------------------------------------------ */
+#define FRISK_EW_MAX_INPUTS 8
+#define FRISK_EW_MAX_OPS 48
+#define FRISK_EW_MAX_STACK 6
+typedef enum frisk_ew_op {
+  FRISK_EW_INPUT = 0,
+  FRISK_EW_CONST = 1,
+  FRISK_EW_ADD = 2,
+  FRISK_EW_SUB = 3,
+  FRISK_EW_MUL = 4,
+  FRISK_EW_DIV = 5,
+  FRISK_EW_MAX = 6,
+  FRISK_EW_MIN = 7,
+  FRISK_EW_NEG = 8,
+  FRISK_EW_EXP2 = 9,
+  FRISK_EW_LOG2 = 10
+} frisk_ew_op;
+
+typedef struct frisk_elementwise_desc {
+  int32_t abi_version;   /* FRISK_HIP_ABI_VERSION */
+  int32_t n_inputs, n_ops;
+  int32_t out_dtype;
+  int64_t rows, cols, out_ld;
+  int32_t in_dtype[FRISK_EW_MAX_INPUTS];
+  int32_t in_col_stride[FRISK_EW_MAX_INPUTS];   /* 0 or 1 */
+  int64_t in_row_stride[FRISK_EW_MAX_INPUTS];   /* >= 0, elements */
+  int32_t op[FRISK_EW_MAX_OPS];                 /* frisk_ew_op */
+  int32_t arg[FRISK_EW_MAX_OPS];                /* operand index of FRISK_EW_INPUT */
+  float imm[FRISK_EW_MAX_OPS];                  /* value of FRISK_EW_CONST */
+} frisk_elementwise_desc;
+
+int frisk_hip_elementwise(const frisk_elementwise_desc* desc, const void* const* inputs, void* out, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Fused attention forward: O = softmax(scale * Q K^T) V per (batch, head), the kernel sketched in the

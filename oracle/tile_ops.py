@@ -74,3 +74,26 @@ def online_softmax_sketch(dtype, src, cst, chunk=1024):
         with np.errstate(invalid="ignore"):
             lse = max_x * cst + np.log2(np.where(np.isneginf(lse), 0.0, np.exp2(lse - max_x * cst)) + sum_exp_x)
     return np.exp2(x * cst - lse[:, None]), lse
+
+
+def elementwise(program, inputs, rows, cols):
+    """frisk.block body (FriskOps.td:143-190) as the postfix program frisk_hip_elementwise takes, in float64.
+    program: steps ("input", k) | ("const", v) | "add" | "sub" | "mul" | "div" | "max" | "min" | "neg" | "exp2" | "log2";
+    inputs: arrays that broadcast against (rows, cols).  max / min ignore a NaN operand (arith.maxnumf / minnumf)."""
+    stack = []
+    for step in program:
+        name, val = (step, None) if isinstance(step, str) else step
+        if name == "input":
+            stack.append(np.broadcast_to(np.asarray(inputs[val], dtype=np.float64), (rows, cols)))
+        elif name == "const":
+            stack.append(np.full((rows, cols), float(val)))
+        elif name in ("neg", "exp2", "log2"):
+            x = stack.pop()
+            with np.errstate(all="ignore"):
+                stack.append(-x if name == "neg" else np.exp2(x) if name == "exp2" else np.log2(x))
+        else:
+            b, a = stack.pop(), stack.pop()
+            with np.errstate(all="ignore"):
+                stack.append({"add": np.add, "sub": np.subtract, "mul": np.multiply, "div": np.divide, "max": np.fmax, "min": np.fmin}[name](a, b))
+    assert len(stack) == 1, "the program must leave one value"
+    return stack[0]

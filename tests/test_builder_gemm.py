@@ -410,18 +410,39 @@ def test_fill_under_a_grid_is_refused():
     assert "once per iteration" in str(e.value)
 
 
-def test_tiled_copy_that_places_tiles_transposed_is_refused():
-    """both sides tile a square, but tile (by, bx) of the source lands at (bx, by) of the destination: not a window copy"""
-    h = F.create_session()
+def _transposed_tiles_kernel(h, n=64, tile=32, dtype="fp16", out_dtype=None):
+    """tile (by, bx) of the n x n source lands at (bx, by) of the destination; the elements of a tile keep their order"""
     b = h.builder
-    t = h.memref_type((64, 64), "fp16")
-    kernel, entry = h.new_kernel("k", [t, t])
-    body = b.create_parallel_op([2, 2], 64).add_entry_block()
+    kernel, entry = h.new_kernel("k", [h.memref_type((n, n), dtype), h.memref_type((n, n), out_dtype or dtype)])
+    body = b.create_parallel_op([n // tile, n // tile], 64).add_entry_block()
     b.set_insertion_point_to_start(body)
     by, bx = body.get_argument(0), body.get_argument(1)
     d0, d1 = b.get_affine_dim_expr(0), b.get_affine_dim_expr(1)
-    b.create_copy_op(entry.get_argument(0), entry.get_argument(1), [by, bx], [by, bx], F.AffineMap.get(2, 0, [d0 * 32, d1 * 32]),
-                     F.AffineMap.get(2, 0, [d1 * 32, d0 * 32]), [32, 32], [32, 32])
-    with pytest.raises(ValueError) as e:
+    b.create_copy_op(entry.get_argument(0), entry.get_argument(1), [by, bx], [by, bx], F.AffineMap.get(2, 0, [d0 * tile, d1 * tile]),
+                     F.AffineMap.get(2, 0, [d1 * tile, d0 * tile]), [tile, tile], [tile, tile])
+    return kernel
+
+
+def test_tiled_copy_that_places_tiles_transposed_is_one_tile_by_tile_copy():
+    """both sides tile a square, but tile (by, bx) of the source lands at (bx, by) of the destination: not a window copy; it is
+    lowered as one launch that copies tile by tile, each grid index displacing the two sides by its own step"""
+    h = F.create_session()
+    (op,) = F.runtime.match_ops(_transposed_tiles_kernel(h))
+    assert op["op"] == "copy_tiles" and (op["rows"], op["cols"]) == (32, 32) and op["tiles"] == (2, 2)
+    assert op["src_steps"] == (32 * 64, 32) and op["dst_steps"] == (32, 32 * 64) and (op["src_ld"], op["dst_ld"]) == (64, 64)
+    # a third index that rearranges is more than one launch places
+    h = F.create_session()
+    b = h.builder
+    t = h.memref_type((64, 128), "fp16")
+    kernel, entry = h.new_kernel("k", [t, h.memref_type((128, 64), "fp16")])
+    body = b.create_parallel_op([2, 2], 64).add_entry_block()
+    b.set_insertion_point_to_start(body)
+    by, bx = body.get_argument(0), body.get_argument(1)
+
+    def loop(bb, iv):
+        d0, d1, d2 = (bb.get_affine_dim_expr(i) for i in range(3))
+        bb.create_copy_op(entry.get_argument(0), entry.get_argument(1), [by, bx, iv], [by, bx, iv], F.AffineMap.get(3, 0, [d0 * 32, d1 * 64 + d2 * 32]),
+                          F.AffineMap.get(3, 0, [d1 * 64 + d2 * 32, d0 * 32]), [32, 32], [32, 32])
+    b.create_for_op(0, 2, 1, loop)
+    with pytest.raises(ValueError, match="at most two"):
         F.runtime.match_ops(kernel)
-    assert "moves the source and destination windows of a tiled copy differently" in str(e.value)

@@ -102,3 +102,24 @@ def test_tiled_copy_through_the_builder(hip):
         want = np.full((160, 320), 0xEEEE, dtype=np.uint16)
         want[16:144, 64:320] = T.copy(O.F32, x, O.F16)
         assert np.array_equal(from_dev(dy, np.uint16, (160, 320)), want)
+
+
+def test_tiles_placed_transposed_through_the_builder(hip):
+    """frisk.copy under a grid whose destination map swaps the grid indices: block (by, bx) of the source becomes block (bx, by)
+    of the destination, every tile keeping the order of its elements; one tile-by-tile launch, converting f32 -> f16 on the way"""
+    import torch
+    from oracle import tile_ops as T
+    from test_builder_gemm import _transposed_tiles_kernel
+    for n, tile, dt, out_dt in ((64, 32, "fp16", None), (256, 64, "fp32", "fp16"), (96, 24, "bf16", None)):
+        h = F.create_session()
+        kernel = _transposed_tiles_kernel(h, n, tile, dt, out_dt)
+        code, out_code = {"fp16": O.F16, "fp32": O.F32, "bf16": O.BF16}[dt], {"fp16": O.F16, "fp32": O.F32, "bf16": O.BF16}[out_dt or dt]
+        x = O.encode(code, O.normal(n * n, 78, 0, 2.0)).reshape(n, n)
+        dx = to_dev(x)
+        dy = torch.full((n * n * O.NP_STORAGE[out_code]().itemsize,), 0xEE, dtype=torch.uint8, device="cuda")
+        F.runtime.launch_ops(kernel, [dx.data_ptr(), dy.data_ptr()], torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        conv = T.copy(code, x, out_code)
+        nb = n // tile
+        want = conv.reshape(nb, tile, nb, tile).transpose(2, 1, 0, 3).reshape(n, n)   # block indices swapped, tiles as they were
+        assert np.array_equal(from_dev(dy, O.NP_STORAGE[out_code], (n, n)), want), (n, tile, dt)

@@ -294,3 +294,118 @@ def test_softmax_gpu(hip, dt):
         assert np.all(np.isfinite(g)) and np.all(g[:, masked] == 0.0), (rows, cols)
         assert np.all(np.abs(g - ref) <= tol * scale + floor), (rows, cols, float(np.max(np.abs(g - ref) / scale)))
         assert np.abs(dL.cpu().numpy() - lse).max() <= 1e-4 * max(1.0, np.abs(lse).max()), (rows, cols)
+
+
+# ------------------------------------------------------------------ frisk.block bodies as postfix programs, tiled copies
+def test_oracle_elementwise_closed_forms():
+    x = np.array([[0.25, 1.0, 4.0, 1024.0]])
+    assert np.array_equal(T.elementwise([("input", 0), "log2", "exp2"], [x], 1, 4), x)                       # powers of two: exact both ways
+    assert np.array_equal(T.elementwise([("input", 0), ("input", 0), "sub"], [x], 1, 4), np.zeros((1, 4)))
+    # the operand pushed first is the left one
+    assert np.array_equal(T.elementwise([("input", 0), ("const", 2.0), "div"], [x], 1, 4), x / 2) and np.array_equal(T.elementwise([("const", 2.0), ("input", 0), "sub"], [x], 1, 4), 2 - x)
+    # max / min ignore a NaN operand
+    n = np.array([[np.nan, 3.0]])
+    assert np.array_equal(T.elementwise([("input", 0), ("const", 1.0), "max"], [n], 1, 2), [[1.0, 3.0]]) and np.array_equal(T.elementwise([("input", 0), ("const", 1.0), "min"], [n], 1, 2), [[1.0, 1.0]])
+    # operands broadcast: a value per row, a value per column
+    r, c = np.arange(3.0).reshape(3, 1), np.arange(4.0).reshape(1, 4)
+    assert np.array_equal(T.elementwise([("input", 0), ("input", 1), "mul", "neg"], [r, c], 3, 4), -(r * c))
+
+
+def test_elementwise_and_tiled_copy_status_codes_before_any_launch():
+    from frisk_amd import runtime as R
+
+    def status(program, inputs=((R.F32, 8, 1),), ptrs=(0x1000,), out=0x2000, rows=4, cols=8, out_dtype=R.F32):
+        with pytest.raises(R.FriskHipError) as e:
+            R.elementwise(R.make_elementwise_desc(program, list(inputs), out_dtype, rows, cols), list(ptrs), out)
+        return e.value.status
+    x = ("input", 0)
+    assert status(["add"]) == R.ERR_ARGUMENT                                              # pops an empty stack
+    assert status([x, x]) == R.ERR_ARGUMENT                                               # leaves two values
+    assert status([x] * 7 + ["add"] * 6) == R.ERR_ARGUMENT                                # needs a stack of 7
+    assert status([("input", 1)]) == R.ERR_ARGUMENT                                       # no such operand
+    assert status([x], inputs=((R.F32, 8, 2),)) == R.ERR_SHAPE                            # column stride
+    assert status([x], inputs=((R.I8, 8, 1),)) == R.ERR_DTYPE
+    assert status([x], ptrs=(None,)) == R.ERR_NULL
+    assert status([x], out=None) == R.ERR_NULL
+    assert status([x], ptrs=(0x1002,)) == R.ERR_ALIGNMENT
+    d = R.make_elementwise_desc([x], [(R.F32, 8, 1)], R.F32, 4, 8)
+    d.n_ops = 0
+    with pytest.raises(R.FriskHipError) as e:
+        R.elementwise(d, [0x1000], 0x2000)
+    assert e.value.status == R.ERR_ARGUMENT
+    R.elementwise(R.make_elementwise_desc([x], [(R.F32, 8, 1)], R.F32, 0, 8), [0x1000], None)   # an empty space touches nothing
+    with pytest.raises(R.FriskHipError) as e:
+        R.copy_tiles(R.F16, 0x1000, 64, R.F16, 0x2000, 64, 8, 8, 2, -8, 8)
+    assert e.value.status == R.ERR_SHAPE
+    with pytest.raises(R.FriskHipError) as e:
+        R.copy_tiles(R.F16, 0x1000, 4, R.F16, 0x2000, 64, 8, 8, 2, 8, 8)                  # ld < tile cols
+    assert e.value.status == R.ERR_SHAPE
+    R.copy_tiles(R.F16, None, 64, R.F16, None, 64, 8, 8, 0, 8, 8)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", FLOATS, ids=[NAMES[d] for d in FLOATS])
+def test_elementwise_gpu(hip, dt):
+    """every opcode, walked / per-row / per-column / scalar operands, padded rows (vector path), odd extents and an element-
+    aligned pointer (scalar path), in place; against numpy float64 through the oracle's evaluator"""
+    import torch
+    tol = {O.F32: 3e-6, O.F16: 1e-3, O.BF16: 8e-3}[dt]
+    prog = [("input", 0), ("input", 1), "mul", ("input", 2), "sub", ("const", 0.75), "max", ("input", 3), "min", "neg", ("const", 3.0), "add", "log2",
+            ("input", 0), ("const", 0.125), "mul", "exp2", "div"]
+    for rows, cols, pad, shift in ((1, 8, 0, 0), (64, 256, 0, 0), (40, 136, 8, 0), (33, 100, 3, 1), (7, 5000, 0, 0), (1000, 3, 0, 0)):
+        ld = cols + pad
+        x = O.encode(dt, O.normal(rows * ld + shift, 95, 0, 1.0))
+        s = O.uniform(rows, 95, 1, 0.5, 1.5).astype(np.float32)
+        m = O.encode(dt, O.uniform(cols, 95, 2, -0.5, 0.5))
+        k = np.array([2.5], dtype=np.float32)
+        xf = O.decode(dt, x)[shift:].reshape(rows, ld)[:, :cols].astype(np.float64)
+        ins = [xf, s.astype(np.float64).reshape(rows, 1), O.decode(dt, m).astype(np.float64).reshape(1, cols), np.array([[2.5]])]
+        want = T.elementwise(prog, ins, rows, cols)
+        assert np.all(np.isfinite(want))
+        dx, ds, dm, dk = _dev(x), _dev(s), _dev(m), _dev(k)
+        es = O.NP_STORAGE[dt]().itemsize
+        dy = torch.full(((rows * ld + shift) * es,), 0xEE, dtype=torch.uint8, device="cuda")
+        desc = hip.make_elementwise_desc(prog, [(dt, ld, 1), (hip.F32, 1, 0), (dt, 0, 1), (hip.F32, 0, 0)], dt, rows, cols, out_ld=ld)
+        hip.elementwise(desc, [dx.data_ptr() + shift * es, ds.data_ptr(), dm.data_ptr(), dk.data_ptr()], dy.data_ptr() + shift * es, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        full = _host(dy, O.NP_STORAGE[dt])[shift:].reshape(rows, ld)
+        got = O.decode(dt, np.ascontiguousarray(full[:, :cols])).astype(np.float64).reshape(rows, cols)
+        err = np.abs(got - want) / np.maximum(np.abs(want), np.sqrt(np.mean(want ** 2)))
+        assert err.max() <= tol, (rows, cols, pad, shift, err.max())
+        if pad:
+            assert np.all(full[:, cols:].view(np.uint8) == 0xEE), "the kernel wrote into the padding"
+        # in place: the output over operand 0
+        hip.elementwise(desc, [dx.data_ptr() + shift * es, ds.data_ptr(), dm.data_ptr(), dk.data_ptr()], dx.data_ptr() + shift * es, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        again = _host(dx, O.NP_STORAGE[dt])[shift:].reshape(rows, ld)[:, :cols]
+        assert np.array_equal(again, full[:, :cols])
+
+
+@pytest.mark.gpu
+def test_copy_tiles_gpu(hip):
+    """tiles placed elsewhere than they came from: block-transposed, gathered at another pitch, converting on the way; bytes
+    between the destination tiles stay as they were"""
+    import torch
+    for sdt, ddt, tr, tc, n0, n1, sld, dld in ((O.F16, O.F16, 32, 32, 4, 4, 128, 128), (O.F32, O.BF16, 16, 24, 3, 5, 130, 80), (O.BF16, O.F32, 5, 7, 2, 3, 23, 40),
+                                               (O.F16, O.F16, 64, 512, 8, 1, 512, 600)):
+        src_rows, dst_rows = n0 * tr, n1 * tr if n1 > 1 else n0 * tr
+        x = O.encode(sdt, O.normal(src_rows * sld, 96, 0, 2.0)).reshape(src_rows, sld)
+        dx = _dev(x)
+        if n1 > 1:   # source tile (a, b) at rows a, columns b -> destination rows b, columns a
+            dst_cols_needed = n0 * tc
+            dld = max(dld, dst_cols_needed)
+            steps = dict(n0=n0, src_step0=tr * sld, dst_step0=tc, n1=n1, src_step1=tc, dst_step1=tr * dld)
+        else:        # one column of tiles copied at another row pitch
+            steps = dict(n0=n0, src_step0=tr * sld, dst_step0=tr * dld, n1=1, src_step1=0, dst_step1=0)
+        des = O.NP_STORAGE[ddt]().itemsize
+        dy = torch.full((dst_rows * dld * des,), 0xEE, dtype=torch.uint8, device="cuda")
+        hip.copy_tiles(sdt, dx.data_ptr(), sld, ddt, dy.data_ptr(), dld, tr, tc, stream=torch.cuda.current_stream().cuda_stream, **steps)
+        torch.cuda.synchronize()
+        want = np.frombuffer(bytes([0xEE]) * (dst_rows * dld * des), dtype=O.NP_STORAGE[ddt]).reshape(dst_rows, dld).copy()
+        conv = T.copy(sdt, x, ddt)
+        for a in range(n0):
+            for b in range(n1):
+                so, do = a * steps["src_step0"] + b * steps["src_step1"], a * steps["dst_step0"] + b * steps["dst_step1"]
+                sr, sc, dr, dc = so // sld, so % sld, do // dld, do % dld
+                want[dr:dr + tr, dc:dc + tc] = conv[sr:sr + tr, sc:sc + tc]
+        assert np.array_equal(_host(dy, O.NP_STORAGE[ddt]).reshape(dst_rows, dld), want), (sdt, ddt, tr, tc)
