@@ -478,6 +478,18 @@ def main():
         # the reference's @online_softmax sketch at the same size class: one read and one write of every element
         ms = time_op(lambda: R.softmax(R.F16, src16.data_ptr(), ocols, dst16.data_ptr(), ocols, orows, ocols, 1.25, None, cs))
         ops["softmax_rows"] = {"GB/s": round(2 * nbytes / (ms * 1e-3) / 1e9, 1), "frac_of_8TB/s": round(2 * nbytes / (ms * 1e-3) / 8e12, 4), "kernel_ms": round(ms, 5)}
+        # a free-standing frisk.block body through the interpreter: y = log2(max(x, c) / (x + c)), one read and one write per element
+        prog = [("input", 0), ("const", 0.5), "max", ("input", 0), ("const", 0.5), "add", "div", "log2"]
+        ew = R.make_elementwise_desc(prog, [(R.F16, ocols, 1)], R.F16, orows, ocols)
+        src16.abs_().add_(0.01)
+        ms = time_op(lambda: R.elementwise(ew, [src16.data_ptr()], dst16.data_ptr(), cs))
+        ops["block_body_log2_max_div"] = {"GB/s": round(2 * nbytes / (ms * 1e-3) / 1e9, 1), "frac_of_8TB/s": round(2 * nbytes / (ms * 1e-3) / 8e12, 4), "kernel_ms": round(ms, 5),
+                                          "program": "x0 c0.5 max x0 c0.5 add div log2 (8 steps, interpreted per 8 elements)"}
+        # tiles placed transposed: 64 x 64 tiles of the 8192 x 8192 head of the view, block (a, b) -> block (b, a)
+        tb = 8192 // 64
+        ms = time_op(lambda: R.copy_tiles(R.F16, src16.data_ptr(), ocols, R.F16, dst16.data_ptr(), ocols, 64, 64, tb, 64 * ocols, 64, tb, 64, 64 * ocols, cs))
+        moved = 2 * 8192 * 8192 * 2
+        ops["copy_tiles_transposed_8192x8192"] = {"GB/s": round(moved / (ms * 1e-3) / 1e9, 1), "frac_of_8TB/s": round(moved / (ms * 1e-3) / 8e12, 4), "kernel_ms": round(ms, 5)}
         del src16, dst16
         line["tile_ops_32768x8192_f16"] = ops
 
