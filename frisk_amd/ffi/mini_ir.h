@@ -1124,8 +1124,10 @@ inline GemmProgram match_tiled_gemm(Operation* kernel, Operation* module = nullp
 // induction variables: the windows of all iterations must then tile one rectangle of each side without gaps or overlap
 // (every index moves the window by whole tiles along one dimension); when every index moves both sides alike the copy is
 // lowered as one copy of that rectangle, otherwise (tiles placed transposed, say) as one tile-by-tile copy.  A tile may also pass through one frisk.alloc_buffer (global -> buffer -> global in
-// the same block, the buffer used by nothing else): the pair is lowered as the direct copy.  Fill and reduce take whole
-// arguments and must not be repeated by an enclosing grid or loop.
+// the same block, the buffer used by nothing else): the pair is lowered as the direct copy.  A staged tile may be reduced
+// on its way (copy -> buffer, reduce buffer -> vector buffer, copy vector buffer -> global) when the indices move it along
+// the kept dimension only: the tiles' reductions are then ONE reduction of the rectangle they cover.  Fill and reduce on
+// whole arguments must not be repeated by an enclosing grid or loop.
 struct TileOpDesc {
   enum Kind { Fill, Copy, Reduce, CopyTiles } kind = Fill;
   int arg_src = -1, arg_dst = -1;          // kernel argument positions (fill: arg_dst only)
@@ -1258,7 +1260,7 @@ inline std::vector<TileOpDesc> match_data_movement(Operation* kernel) {
 
   std::vector<TileOpDesc> out;
   std::vector<IndexRange> vars;
-  struct Staged { Value buffer; Operation* load; Block* block; };
+  struct Staged { Value buffer; Operation* load; Block* block; Operation* reduce = nullptr; };  // reduce: the tile was reduced into `buffer` on the way
   std::function<void(Block*)> walk = [&](Block* block) {
     std::vector<Staged> staged;  // tiles loaded into a buffer in this block and not yet stored
     for (Operation* op : block->ops) {
@@ -1319,7 +1321,43 @@ inline std::vector<TileOpDesc> match_data_movement(Operation* kernel) {
           if (at == staged.size()) fail("a copy stores a buffer that no copy in the same block has loaded");
           whole_buffer(op, false, src_v);
           load = staged[at].load;
+          Operation* reduced_by = staged[at].reduce;
           staged.erase(staged.begin() + (long)at);
+          if (reduced_by) {
+            // copy tile -> buffer; reduce buffer -> vector buffer; copy vector buffer -> global, under a grid or loop whose
+            // indices move the source tile along the kept dimension only: ONE reduction of the rectangle all tiles cover
+            View s = view_of(load->operands[0], "the reduce source"), t = view_of(dst_v, "the reduce destination");
+            if (s.rank != 2) fail("the source of a tiled reduction must have rank 2");
+            const Side ss = side_of(load, false, s.rank, vars, "source"), ts = side_of(op, true, t.rank, vars, "destination");
+            check_inside(ss, s, "source");
+            check_inside(ts, t, "destination");
+            d.kind = TileOpDesc::Reduce;
+            d.dim = reduced_by->int_attr("dim");
+            if (d.dim != 0 && d.dim != 1) fail("reduce dimension out of range");
+            if (!reduced_by->attr("clear")->b) fail("a tiled reduction must clear its staging vector (clear = true): the buffer holds nothing before");
+            const int kept_from_end = d.dim == 1 ? 1 : 0;   // the source dimension that survives, counted from the last
+            if ((d.dim == 1 ? ss.cols != ss.tc : ss.rows != ss.tr)) fail("the grid of a tiled reduction tiles the reduced dimension: partial results of different tiles would have to be combined");
+            const int64_t kept = d.dim == 1 ? ss.rows : ss.cols, kept_tile = d.dim == 1 ? ss.tr : ss.tc;
+            if (ts.rows != 1 && ts.cols != 1) fail("the destination windows of a tiled reduction do not form a vector");
+            const bool dst_along_cols = ts.rows == 1;
+            if ((dst_along_cols ? ts.cols : ts.rows) != kept || (dst_along_cols ? ts.tc : ts.tr) != kept_tile) fail("the destination of a tiled reduction does not hold one element per kept index");
+            if (!dst_along_cols && t.cols != 1) fail("the destination of a tiled reduction must be contiguous");
+            for (size_t v = 0; v < vars.size(); ++v) {
+              if (vars[v].count <= 1) continue;
+              if (ss.moves[v].first != kept_from_end) fail("an index of a tiled reduction does not move the source tile along the kept dimension");
+              if (ts.moves[v].first != (dst_along_cols ? 0 : 1) || ts.moves[v].second != ss.moves[v].second) fail("an index moves the source tile and the destination window of a tiled reduction differently");
+            }
+            if (!s.elem.equals(t.elem) || !s.elem.equals(load->operands[1].type().element()) || !t.elem.equals(src_v.type().element()))
+              fail("the element types of a tiled reduction differ between source, buffers and destination");
+            d.arg_src = s.arg; d.arg_dst = t.arg; d.elem_src = s.elem; d.elem_dst = t.elem;
+            d.rows = ss.rows; d.cols = ss.cols; d.src_ld = s.cols;
+            d.src_offset = ss.r0 * s.cols + ss.c0;
+            d.dst_offset = ts.r0 * t.cols + ts.c0;
+            d.reduce_kind = reduced_by->attr("kind")->s == "sum" ? "add" : reduced_by->attr("kind")->s;
+            d.clear = true;
+            out.push_back(d);
+            continue;
+          }
           const Type via = src_v.type().element();
           if (!via.equals(load->operands[0].type().element()) && !via.equals(dst_v.type().element())) fail("a staging buffer's element type is neither the source's nor the destination's");
         }
@@ -1366,6 +1404,21 @@ inline std::vector<TileOpDesc> match_data_movement(Operation* kernel) {
             }
           }
         }
+      } else if (op->name == "frisk.reduce" && kernel_arg_index(kernel, op->operands[0]) < 0) {
+        // a reduction of a staged tile into a second buffer: completed by the copy that stores that buffer
+        size_t at = staged.size();
+        for (size_t i = 0; i < staged.size(); ++i) if (staged[i].buffer == op->operands[0] && !staged[i].reduce) at = i;
+        if (at == staged.size()) fail("a reduce reads a buffer that no copy in the same block has loaded");
+        const Value vec = op->operands[1];
+        if (!vec.impl || !vec.impl->def || vec.impl->def->name != "frisk.alloc_buffer") fail("a reduce of a staged tile must write a frisk.alloc_buffer");
+        if (uses_of(vec) != 2) fail("the vector buffer of a tiled reduction must be used by exactly the reduce and one store");
+        const auto& tile_shape = op->operands[0].type().impl->shape;
+        const auto& vec_shape = vec.type().impl->shape;
+        const int64_t dim = op->int_attr("dim");
+        if (tile_shape.size() != 2 || vec_shape.size() != 1 || dim < 0 || dim > 1 || vec_shape[0] != tile_shape[(size_t)(1 - dim)]) fail("a reduce of a staged tile must go from a rank-2 buffer to a vector of the kept extent");
+        staged[at].buffer = vec;
+        staged[at].reduce = op;
+        continue;
       } else if (op->name == "frisk.reduce") {
         if (repeated) fail("a reduce under a grid or a loop would run once per iteration");
         View s = view_of(op->operands[0], "the reduce source"), t = view_of(op->operands[1], "the reduce destination");

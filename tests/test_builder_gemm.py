@@ -446,3 +446,51 @@ def test_tiled_copy_that_places_tiles_transposed_is_one_tile_by_tile_copy():
     b.create_for_op(0, 2, 1, loop)
     with pytest.raises(ValueError, match="at most two"):
         F.runtime.match_ops(kernel)
+
+
+def _tiled_reduce_kernel(h, *, rows=128, cols=256, dim=1, kind="max", dtype="fp16", tile=32, clear=True, tile_reduced_dim=False):
+    """kernel(x: rows x cols, v: kept extent): v := reduce(x along dim), written tile by tile: a grid over bands of `tile` kept
+    indices, every band through a shared tile, reduced into a shared vector, the vector stored to its place in v"""
+    b = h.builder
+    kept = rows if dim == 1 else cols
+    kernel, entry = h.new_kernel("tiled_reduce", [h.memref_type((rows, cols), dtype), h.memref_type((kept,), dtype)])
+    x, v = entry.get_argument(0), entry.get_argument(1)
+    grid = [kept // tile] + ([2] if tile_reduced_dim else [])
+    body = b.create_parallel_op(grid, 256).add_entry_block()
+    b.set_insertion_point_to_start(body)
+    band = body.get_argument(0)
+    red_extent = (cols if dim == 1 else rows) // (2 if tile_reduced_dim else 1)
+    shape = (tile, red_extent) if dim == 1 else (red_extent, tile)
+    buf = h.alloc_buffer(shape, dtype, space=F.MemorySpace.SHARED)
+    vec = h.alloc_buffer((tile,), dtype, space=F.MemorySpace.SHARED)
+    d0, d1 = b.get_affine_dim_expr(0), b.get_affine_dim_expr(1)
+    c = b.get_affine_constant_expr
+    idx = [band] + ([body.get_argument(1)] if tile_reduced_dim else [])
+    other = d1 * red_extent if tile_reduced_dim else c(0)
+    src_map = F.AffineMap.get(len(idx), 0, [d0 * tile, other] if dim == 1 else [other, d0 * tile])
+    b.create_copy_op(x, buf, idx, [], src_map, F.AffineMap.get(0, 0, [c(0), c(0)]), list(shape), list(shape))
+    b.create_reduce_op(buf, vec, kind, dim, clear)
+    b.create_copy_op(vec, v, [], [band], F.AffineMap.get(0, 0, [c(0)]), F.AffineMap.get(1, 0, [d0 * tile]), [tile], [tile])
+    return kernel
+
+
+def test_reduction_tiled_over_a_grid_is_one_reduction():
+    """copy tile -> buffer; reduce buffer -> vector; copy vector -> global under a grid that walks the kept dimension (FriskOps.td:412-441,
+    FriskOps.cpp:1725-1767): recognised as one reduction of the rectangle the tiles cover"""
+    for dim, kind in ((1, "max"), (0, "sum")):
+        h = F.create_session()
+        kernel = _tiled_reduce_kernel(h, dim=dim, kind=kind)
+        assert h.module.verify()
+        (op,) = F.runtime.match_ops(kernel)
+        assert op["op"] == "reduce" and (op["rows"], op["cols"], op["src_ld"]) == (128, 256, 256) and op["dim"] == dim
+        assert op["kind"] == ("max" if kind == "max" else "add") and op["clear"] and (op["src"], op["dst"], op["src_offset"], op["dst_offset"]) == (0, 1, 0, 0)
+    sessions = []
+
+    def refused(**kw):
+        h = F.create_session()
+        sessions.append(h)
+        with pytest.raises(ValueError) as e:
+            F.runtime.match_ops(_tiled_reduce_kernel(h, **kw))
+        return str(e.value)
+    assert "tiles the reduced dimension" in refused(tile_reduced_dim=True)
+    assert "must clear" in refused(clear=False)

@@ -123,3 +123,27 @@ def test_tiles_placed_transposed_through_the_builder(hip):
         nb = n // tile
         want = conv.reshape(nb, tile, nb, tile).transpose(2, 1, 0, 3).reshape(n, n)   # block indices swapped, tiles as they were
         assert np.array_equal(from_dev(dy, O.NP_STORAGE[out_code], (n, n)), want), (n, tile, dt)
+
+
+def test_reduction_tiled_over_a_grid_through_the_builder(hip):
+    """bands of rows (or columns) staged through a shared tile, reduced into a shared vector and stored to their place: one reduce
+    launch on the device, against the oracle's reduction of the whole view"""
+    import torch
+    from oracle import tile_ops as T
+    from test_builder_gemm import _tiled_reduce_kernel
+    for dim, kind, dt, code in ((1, "max", "fp16", O.F16), (0, "sum", "fp32", O.F32), (1, "sum", "bf16", O.BF16)):
+        h = F.create_session()
+        kernel = _tiled_reduce_kernel(h, rows=128, cols=256, dim=dim, kind=kind, dtype=dt)
+        x = O.encode(code, O.normal(128 * 256, 79, 0, 1.0)).reshape(128, 256)
+        kept = 128 if dim == 1 else 256
+        dx = to_dev(x)
+        dv = torch.full((kept * O.NP_STORAGE[code]().itemsize,), 0xEE, dtype=torch.uint8, device="cuda")
+        F.runtime.launch_ops(kernel, [dx.data_ptr(), dv.data_ptr()], torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        got = O.decode(code, from_dev(dv, O.NP_STORAGE[code], (kept,))).astype(np.float64)
+        want = T.reduce_f64(code, x, dim, "add" if kind == "sum" else kind)
+        if kind == "max":
+            assert np.array_equal(got, want)
+        else:
+            tol = {O.F32: 1e-5, O.F16: 1e-3, O.BF16: 8e-3}[code]
+            assert (np.abs(got - want) / np.maximum(np.abs(want), np.sqrt(np.mean(want ** 2)))).max() <= tol
