@@ -74,7 +74,7 @@ static int elem_size(int dt) {
     default: return 0;
   }
 }
-static int frag_bytes(int dt) { return dt == FRISK_E4M3 ? 32 : (dt == FRISK_F32 ? 4 : 16); }
+static int frag_bytes(int dt) { return dt == FRISK_E4M3 ? 32 : 16; }
 static int mfma_k(int dt) { return dt == FRISK_F32 ? 2 : (2 * frag_bytes(dt)) / elem_size(dt); }
 
 // Wave partition of a block tile: the reference's computeWarpPartition
@@ -156,7 +156,7 @@ static void fill_layout(frisk_lds_layout* L, bool kcontig, int es, int fragb, in
   L->row_shift2 = s.sh2;
   L->row_mask2 = s.mk2;
   L->chunk_shift2 = s.cs2;
-  L->read_instr = es == 4 ? 3 : (kcontig ? 0 : (es == 2 ? 1 : 2));
+  L->read_instr = kcontig ? 0 : (es == 4 ? 3 : (es == 2 ? 1 : 2));
   int atoms = mn / atom < 4 ? mn / atom : 4;
   int n_access = atoms * ((bk * es) / frag_kstep_bytes(fragb, atom)) * frag_instr_count(kcontig, es, fragb);
   // evaluating the bank model costs ~0.1 ms of host time: only when the caller asks for the plan
@@ -188,11 +188,10 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
   double c;  // cost of one K tile with the chip full
   const int64_t area = (int64_t)k->bm * k->bn;
   if (k->dtype == FRISK_F32) {
-    // 64x64: per K tile of 64 / 32; with K tiles of 128 split over two sets of waves 10 % less per unit of K when the grid is one round
-    // 128x128: K tiles of 16 in a ring of 4 cost 0.91 per tile against 1.93 for K tiles of 32 in a ring of 2, except with both operands
-    // K-contiguous (rows of 64 bytes double the L2 requests: 1032 against 998 us at 4096^3)
-    const double c128 = k->bk <= 16 ? ((!k->transA && k->transB) ? 1.0 : 0.91) : 1.93;
-    c = area >= 128 * 128 ? c128 : (k->wk > 1 ? (tiles <= 256 ? 1.8 : 2.3) : (k->bk >= 64 ? 1.0 : 0.55));
+    // Measured with 16-byte fragments (K-contiguous tiles read by ds_read_b128), us, NN: 1024^3 64x64x32 18.8, x64 19.4, x128 on 8 waves
+    // 19.5; 1536^3 69.4 / 73.8 / 78.6; 2048^3 128x128x32 120.8, x16 in a ring of 4 124.1, 64x64x32 123.3; 4096^3 928 / 941 / 962.
+    const double c128 = k->bk <= 16 ? ((!k->transA && k->transB) ? 1.0 : 0.91) : 1.74;
+    c = area >= 128 * 128 ? c128 : (k->wk > 1 ? (tiles <= 256 ? 1.8 : 2.3) : (k->bk >= 64 ? 1.0 : 0.44));
   } else if (k->bm == 32) {
     // 32x32 with a 4x deeper K tile; 32x128 (8-bit: 60.1 us for 256 tiles x 64 K tiles, the rate of the 32x32 kernel per K tile)
     c = k->wk > 1 ? 0.8 : (elem_size(k->dtype) == 1 ? 0.85 : 0.25);
@@ -522,7 +521,7 @@ int frisk_hip_lds_search_atom(const frisk_lds_layout* shape, int elem_bytes, int
   *best = *shape;
   best->row_shift = s.sh; best->row_mask = s.mk; best->chunk_shift = s.cs;
   best->row_shift2 = s.sh2; best->row_mask2 = s.mk2; best->chunk_shift2 = s.cs2;
-  best->read_instr = elem_bytes == 4 ? 3 : (kc ? 0 : (elem_bytes == 2 ? 1 : 2));
+  best->read_instr = elem_bytes == 4 ? (kc && frag_bytes >= 16 ? 0 : 3) : (kc ? 0 : (elem_bytes == 2 ? 1 : 2));
   best->read_cycles = (float)swizzle_read_cycles(t, s) / (float)n_access;
   best->write_cycles = 16.f;
   if (unswizzled_cycles) *unswizzled_cycles = (float)swizzle_read_cycles(t, Swizzle{0, 0, 0}) / (float)n_access;

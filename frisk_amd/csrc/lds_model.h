@@ -72,7 +72,8 @@ FRISK_HD int frag_addr_kc(int rowb, Swizzle s, int fragb, int lane, int mn0, int
 // The at / 16 blocks of a K-group sit side by side along the columns.
 // 32-bit elements read their single value directly.
 FRISK_HD int frag_addr_mc(int rowb, Swizzle s, int es, int fragb, int lane, int mn0, int kb0, int q, int at = 32) {
-  if (es == 4) return lds_offset(rowb, s, kb0 / 4 + (lane >> 5), (mn0 + (lane & 31)) * 4);
+  // 32-bit elements: instruction q of fragb / 4 reads the value at K index q of the lane's K group (fragb / 4 consecutive K)
+  if (es == 4) return lds_offset(rowb, s, kb0 / 4 + (lane >> 5) * (fragb / 4) + q, (mn0 + (lane & 31)) * 4);
   int kpi = es == 2 ? 4 : 8;
   int lpr = 16 / kpi;
   int blk = lane >> 4, l16 = lane & 15;
@@ -82,9 +83,11 @@ FRISK_HD int frag_addr_mc(int rowb, Swizzle s, int es, int fragb, int lane, int 
   int colbyte = (col0 + (l16 % lpr) * (8 / es)) * es;
   return lds_offset(rowb, s, krow, colbyte);
 }
-FRISK_HD int frag_instr_count(bool kcontig, int es, int fragb) { return (es == 4) ? 1 : (kcontig ? fragb / 16 : fragb / 8); }
-FRISK_HD int frag_instr_kind(bool kcontig, int es) { return es == 4 ? LDS_READ_B32 : (kcontig ? LDS_READ_B128 : LDS_READ_B64); }
-FRISK_HD int frag_instr_bytes(bool kcontig, int es) { return es == 4 ? 4 : (kcontig ? 16 : 8); }
+// 32-bit elements: a 16-byte fragment (4 consecutive K, feeding 4 MFMAs of K = 2: lanes 0-31 hold K 0..3, lanes 32-63 K 4..7 of
+// an 8-wide K group) is one ds_read_b128 on a K-contiguous tile and 4 ds_read_b32 on the other; a 4-byte fragment is one read
+FRISK_HD int frag_instr_count(bool kcontig, int es, int fragb) { return (es == 4) ? (kcontig || fragb < 8 ? 1 : fragb / 4) : (kcontig ? fragb / 16 : fragb / 8); }
+FRISK_HD int frag_instr_kind(bool kcontig, int es, int fragb = 16) { return es == 4 ? (kcontig && fragb >= 16 ? LDS_READ_B128 : LDS_READ_B32) : (kcontig ? LDS_READ_B128 : LDS_READ_B64); }
+FRISK_HD int frag_instr_bytes(bool kcontig, int es, int fragb = 16) { return es == 4 ? (kcontig && fragb >= 16 ? 16 : 4) : (kcontig ? 16 : 8); }
 
 // ---- cost of one wave-wide access; addr = 64 byte addresses
 // worst number of distinct dwords any bank must deliver to lanes [first, first+count)
@@ -144,7 +147,7 @@ FRISK_HD int swizzle_read_cycles(TileShape t, Swizzle s) {
   int kstep = frag_kstep_bytes(t.fragb, t.at);
   int ksteps = (t.bk * t.es) / kstep;
   int ninstr = frag_instr_count(t.kcontig, t.es, t.fragb);
-  int kind = frag_instr_kind(t.kcontig, t.es);
+  int kind = frag_instr_kind(t.kcontig, t.es, t.fragb);
   // bank behaviour repeats with the atom position beyond what the swizzle sees; sample the first atoms
   int atoms = t.mn / t.at < 4 ? t.mn / t.at : 4;
   for (int a = 0; a < atoms; ++a)
@@ -215,7 +218,6 @@ FRISK_HD Swizzle default_swizzle(bool kcontig, int es, int rowb, int at = 32) {
   if (kcontig) {
     // 16 consecutive rows must cover the 16 bank groups of 16 bytes: rows of 128 B
     // bring 2 groups by themselves, rows of 64 B bring 4, rows of 256 B none
-    if (es == 4) return Swizzle{0, chunks >= 8 ? 7 : chunks - 1, 0};
     if (chunks >= 16) return Swizzle{0, 15, 0};
     if (chunks == 8) return Swizzle{1, 7, 0};
     if (chunks == 4) return Swizzle{2, 3, 0};
