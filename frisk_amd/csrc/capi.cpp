@@ -201,7 +201,7 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
     // read by transpose reads (twice the LDS instructions) less of it is left (NN 104 against 108).  How full the round is decides:
     // 192 or 196 tiles, NN 78 against 82 us (3584^3) and 164 against 172 (4096x3072x8192), TN 79 against 85 and 169 against 182;
     // 144 tiles (3072^3), where the clock is not the limit, NN 61 against 59, TN even
-    if (k->atom == 16) c *= (!k->transA && k->transB) ? 0.93 : (tiles >= 176 ? 0.96 : 1.06);
+    if (k->atom == 16) c *= k->dtype == FRISK_E4M3 ? 0.96 : (!k->transA && k->transB) ? 0.93 : (tiles >= 176 ? 0.96 : 1.06);
   } else if (area >= 256 * 128) {
     c = 0.93;
   } else {
@@ -272,6 +272,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
         if (pm != k->wm || pn != k->wn) { policy_excluded = true; continue; }
       }
       if (want_split && !k->splitk) continue;
+      if ((d->K + k->bk - 1) / k->bk < k->min_k_tiles) continue;
       // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
       if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
       // ... and address a tile's chunks by 32-bit lane offsets from its first row: the stored rows of one tile must span

@@ -61,6 +61,7 @@ struct KernelEntry {
   int splitk;  // 1: compiled with the split-K store path
   int atom;  // rows and columns of the MFMA atom: 32 (32x32xK) or 16 (16x16x2K)
   int lds_bytes;
+  int min_k_tiles;  // fewest K tiles the kernel's loop is written for
   hipError_t (*launch)(const GemmParams&, hipStream_t);
   hipError_t (*prepare)();  // one-time, non-stream set-up of the kernel function (dynamic LDS limit)
 };

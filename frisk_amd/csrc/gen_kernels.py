@@ -52,7 +52,9 @@ VARIANTS = {
     "f16": ("FRISK_F16", "F16", square(64, atom16=True)),
     "bf16": ("FRISK_BF16", "BF16", square(64, atom16=True)),
     "i8": ("FRISK_I8", "I8", square(128, atom16=True)),
-    "e4m3": ("FRISK_E4M3", "E4M3", square(128)),
+    # 8-bit floats: the 256x256 NT variant once more on the 16x16x128 atom, whose K is the whole K tile (listed first: the planner's
+    # choice for B stored [N][K] from four K tiles on)
+    "e4m3": ("FRISK_E4M3", "E4M3", [(0, 1, 256, 256, 128, 2, 2, 2, 0, 0, 1, 3, 16)] + square(128)),
     # fp32: 128x128 for large problems; 64x64 (one atom per wave) fills the chip at 1024^3, K tiles of 64 measured 5 % faster than 32;
     # the same tile with K tiles of 128 shared by two sets of four waves (8 waves, two per SIMD) another 9 % at 1024^3 (21.6 against
     # 23.9 us), where a CU holds a single work-group and nothing else hides its waits
@@ -89,7 +91,7 @@ for tag, (enum, suffix, variants) in VARIANTS.items():
         cfg = cfg_of(enum, v)
         waves = f"w{wm}x{wn}" + (f"x{wk}" if wk > 1 else "")
         name = f"{tag}_{'t' if ta else 'n'}{'t' if tb else 'n'}_{bm}x{bn}x{bk}_{waves}_s{st}" + (f"x{sb}" if sb != st else "") + (f"_a{at}" if at != 32 else "") + ("_guard" if gd else "") + ("_splitk" if sk else "")
-        lines.append(f'    {{"{name}", {enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {sb}, {wk}, {gd}, {sk}, {at}, {cfg}::LDS_BYTES, &launch_gemm<{cfg}>, &prepare_gemm<{cfg}>}},')
+        lines.append(f'    {{"{name}", {enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {sb}, {wk}, {gd}, {sk}, {at}, {cfg}::LDS_BYTES, {cfg}::MIN_K_TILES, &launch_gemm<{cfg}>, &prepare_gemm<{cfg}>}},')
     lines.append("};")
     lines.append(f"const int kNumKernels{suffix} = sizeof(kKernels{suffix}) / sizeof(kKernels{suffix}[0]);")
     lines.append("#endif")

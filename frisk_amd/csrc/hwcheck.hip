@@ -192,10 +192,14 @@ template <int DT, int AT, int BMN, int BK> struct PathCfg {
     return hipGetLastError();
   }
   static hipError_t launch(int ta, int tb, const void* A, const void* B, void* D, hipStream_t s) {
+    // the atom whose K is the whole K tile exists for K-contiguous operands only (A [M][K], B [N][K])
+    if constexpr (DT == FRISK_E4M3 && AT == 16) return !ta && tb ? launch1<false, true>(A, B, D, s) : hipErrorInvalidValue;
+    else {
     if (!ta && !tb) return launch1<false, false>(A, B, D, s);
     if (!ta && tb) return launch1<false, true>(A, B, D, s);
     if (ta && !tb) return launch1<true, false>(A, B, D, s);
     return launch1<true, true>(A, B, D, s);
+    }
   }
 };
 
@@ -364,6 +368,7 @@ int frisk_hwcheck_fragment_path(int dtype, int atom, int transA, int transB, con
   if (dtype == FRISK_I8 && atom == 32) return (int)PathCfg<FRISK_I8, 32, 256, 128>::launch(transA, transB, A, B, D, s);
   if (dtype == FRISK_I8 && atom == 16) return (int)PathCfg<FRISK_I8, 16, 256, 128>::launch(transA, transB, A, B, D, s);
   if (dtype == FRISK_E4M3 && atom == 32) return (int)PathCfg<FRISK_E4M3, 32, 256, 128>::launch(transA, transB, A, B, D, s);
+  if (dtype == FRISK_E4M3 && atom == 16) return (int)PathCfg<FRISK_E4M3, 16, 256, 128>::launch(transA, transB, A, B, D, s);
   if (dtype == FRISK_F32 && atom == 32) return (int)PathCfg<FRISK_F32, 32, 128, 32>::launch(transA, transB, A, B, D, s);
   return -1;
 }

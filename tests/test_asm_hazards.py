@@ -21,6 +21,7 @@ template __global__ void gemm_kernel<GemmCfg<FRISK_F16, 0, 1, 256, 256, 64, 2, 2
 template __global__ void gemm_kernel<GemmCfg<FRISK_F16, 0, 0, 256, 256, 64, 2, 2, 2, false, true, 1, 3, 16>>(GemmParams);
 template __global__ void gemm_kernel<GemmCfg<FRISK_BF16, 1, 1, 256, 256, 64, 2, 2, 2, false, false, 1, 3, 16>>(GemmParams);
 template __global__ void gemm_kernel<GemmCfg<FRISK_I8, 1, 0, 256, 256, 128, 2, 2, 2, false, false, 1, 3, 16>>(GemmParams);
+template __global__ void gemm_kernel<GemmCfg<FRISK_E4M3, 0, 1, 256, 256, 128, 2, 2, 2, false, false, 1, 3, 16>>(GemmParams);
 }
 """
 
@@ -48,10 +49,15 @@ def hazards(listing, window_before=8, window_after=12):
                 continue
             ops = _operands(line)
             reads, result = _registers(",".join(ops)), _registers(ops[0])
+            multiplicands = _registers(",".join(ops[1:3])) - result
             for back in range(1, window_before + 1):
                 prev = lines[i - back] if i - back >= 0 else ""
-                if prev.startswith("v_") and not prev.startswith("v_mfma") and _registers((_operands(prev) or [""])[0]) & reads:
-                    found.append((name, prev, line))
+                if prev.startswith("v_") and not prev.startswith("v_mfma"):
+                    written = _registers((_operands(prev) or [""])[0]) & reads
+                    # a multiplicand written by an ordinary vector instruction is interlocked by the hardware (only the accumulator
+                    # operand needs wait states); keep two instructions of distance anyway
+                    if written - multiplicands or (written and back <= 2):
+                        found.append((name, prev, line))
             for fwd in range(1, window_after + 1):
                 nxt = lines[i + fwd] if i + fwd < len(lines) else ""
                 if nxt.startswith("v_") and not nxt.startswith("v_mfma") and _registers(",".join(_operands(nxt)[1:])) & result:
@@ -59,16 +65,24 @@ def hazards(listing, window_before=8, window_after=12):
     return found
 
 
-def foreign_m0_uses(listing):
-    """lines that name M0 outside the three-instruction transfer the kernels write themselves (s_add_u32 m0 / s_nop /
-    global_load_lds_dwordx4): the transfer writes M0 without telling the compiler, which is only sound while the
-    compiler has no use of M0 of its own in the kernel"""
+def foreign_m0_uses(listing, reach=6):
+    """lines that name M0 outside the transfers the kernels write themselves: s_add_u32 m0 followed, within a few
+    instructions that do not name M0 (an MFMA and scalar address arithmetic may sit between the two halves of a transfer), by
+    its global_load_lds_dwordx4.  The transfer writes M0 without telling the compiler, which is only sound while the
+    compiler has no use of M0 of its own in the kernel."""
     lines = [l.strip() for l in listing.split("\n") if l.startswith("\t") and not l.strip().startswith((".", ";"))]
     found = []
     for i, line in enumerate(lines):
         if not re.search(r"\bm0\b", line):
             continue
-        own = line.startswith("s_add_u32 m0, ") and lines[i + 1].startswith("s_nop") and lines[i + 2].startswith("global_load_lds_dwordx4")
+        own = False
+        if line.startswith("s_add_u32 m0, "):
+            for nxt in lines[i + 1:i + 1 + reach]:
+                if nxt.startswith("global_load_lds_dwordx4"):
+                    own = True
+                    break
+                if re.search(r"\bm0\b", nxt):
+                    break
         if not own:
             found.append(line)
     return found
@@ -79,6 +93,8 @@ def test_scanner_sees_both_patterns():
     got = hazards(listing)
     assert len(got) == 2 and got[0][1].startswith("v_accvgpr_mov") and got[1][2].startswith("v_accvgpr_read")
     assert foreign_m0_uses("\ts_add_u32 m0, s4, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 v1, s[2:3]\n\ts_mov_b32 m0, s7\n\tds_read_b32 v1, v2\n") == ["s_mov_b32 m0, s7"]
+    split = "\ts_add_u32 m0, s4, 0x400\n\tv_mfma_f32_16x16x32_f16 a[4:7], v[0:3], v[4:7], a[4:7]\n\ts_add_u32 s8, s8, s0\n\tglobal_load_lds_dwordx4 v1, s[8:9]\n"
+    assert foreign_m0_uses(split) == [] and foreign_m0_uses(split.replace("s_add_u32 s8, s8, s0", "s_add_u32 m0, s4, 0x800")) == ["s_add_u32 m0, s4, 0x400"]
     clean = "\n\t.globl\tk\nk:\n\tv_mfma_f32_16x16x32_f16 a[4:7], v[0:3], v[4:7], a[4:7]\n\tv_mfma_f32_16x16x32_f16 a[8:11], v[0:3], v[4:7], a[8:11]\n"
     assert hazards(clean) == []
 
@@ -94,6 +110,7 @@ def test_inline_assembly_mfma_kernels_keep_their_wait_states(tmp_path):
     assert r.returncode == 0, r.stderr[-2000:]
     listing = out.read_text()
     assert listing.count("v_mfma_f32_16x16x32_f16") > 300 and "v_mfma_i32_16x16x64_i8" in listing and "v_mfma_f32_16x16x32_bf16" in listing
+    assert listing.count("v_mfma_f32_16x16x128_f8f6f4") >= 64 * 7 and "scratch_" not in listing  # seven tile bodies, no spills
     bad = hazards(listing)
     assert not bad, "\n".join("%s: %s  ->  %s" % (n[:60], a, b) for n, a, b in bad[:10])
     assert listing.count("global_load_lds_dwordx4") > 100 and foreign_m0_uses(listing) == []

@@ -186,6 +186,48 @@ def test_fp8_tensor_scale_epilogue(hip):
     check(O.E4M3, O.BF16, got, ref)
 
 
+@pytest.mark.parametrize("k_tiles", [4, 5, 6, 7, 8, 9, 16])
+def test_fp8_whole_tile_atom_every_loop_path(hip, k_tiles):
+    """8-bit floats on the 16x16x128 atom (its K is the whole K tile).  The loop peels its first tile and its last three and
+    walks the tiles between them two at a time, with one more single tile or a move of the B fragments between the two
+    register buffers depending on the parity of the count: 4 .. 9 K tiles take every combination, 16 several rounds of the pair loop.
+    Exact check: integers up to 4 in magnitude (sums stay below 2^24), raw fp32 output."""
+    M, N, K = 512, 768, 128 * k_tiles
+    note(f"case fp8 16x16x128 atom, {k_tiles} K tiles, {M}x{N}x{K}")
+    rng = np.random.default_rng(900 + k_tiles)
+    Ai, Bi = rng.integers(-4, 5, size=(M, K)), rng.integers(-4, 5, size=(N, K))
+    A = O.encode(O.E4M3, Ai.astype(np.float32).reshape(-1)).reshape(M, K)
+    B = O.encode(O.E4M3, Bi.astype(np.float32).reshape(-1)).reshape(N, K)
+    got = run_gemm(hip, O.E4M3, A, B, 0, 1, O.F32, M, N, K, tile=(256, 256, 128), atom=16)
+    assert np.array_equal(got.astype(np.int64), Ai.astype(np.int64) @ Bi.astype(np.int64).T)
+    # random values, tensor scales, bf16 output, accumulation into C
+    xa, xb = O.normal(M * K, 40 + k_tiles, 0, 1.0), O.normal(N * K, 40 + k_tiles, 1, 1.0)
+    sA, sB = np.float32(np.abs(xa).max() / 448.0), np.float32(np.abs(xb).max() / 448.0)
+    A, B = O.encode(O.E4M3, xa / sA).reshape(M, K), O.encode(O.E4M3, xb / sB).reshape(N, K)
+    old = O.decode(O.BF16, O.encode(O.BF16, O.uniform(M * N, 41, 4, -2.0, 2.0))).reshape(M, N).astype(np.float64)
+    C0 = O.encode(O.BF16, old.astype(np.float32)).reshape(M, N)
+    ref = O.epilogue_tensor(O.gemm_f64(O.E4M3, A, B, False, True), sA, sB)
+    got = run_gemm(hip, O.E4M3, A, B, 0, 1, O.BF16, M, N, K, epilogue=hip.EPI_TENSOR_SCALE, sA=[sA], sB=[sB], tile=(256, 256, 128), atom=16)
+    check(O.E4M3, O.BF16, got, ref)
+    got = run_gemm(hip, O.E4M3, A, B, 0, 1, O.BF16, M, N, K, epilogue=hip.EPI_TENSOR_SCALE, sA=[sA], sB=[sB], C_init=C0, clear_accum=False,
+                   tile=(256, 256, 128), atom=16)
+    check(O.E4M3, O.BF16, got, ref + old)
+
+
+def test_fp8_whole_tile_atom_needs_four_k_tiles(hip):
+    """its loop is written for four or more K tiles: the planner offers it for none fewer, and a descriptor that names it is refused"""
+    for k_tiles, ok in ((3, False), (4, True)):
+        d = hip.make_desc(O.E4M3, 512, 512, 128 * k_tiles, dtype_out=O.BF16, transB=1, tile=(256, 256, 128), atom=16)
+        if ok:
+            assert hip.kernel_names()[hip.plan(d).kernel_id].endswith("_a16")
+        else:
+            with pytest.raises(hip.FriskHipError) as e:
+                hip.plan(d)
+            assert e.value.status == hip.ERR_TILE
+    p = hip.plan(hip.make_desc(O.E4M3, 512, 512, 384, dtype_out=O.BF16, transB=1))
+    assert not hip.kernel_names()[p.kernel_id].endswith("_a16")
+
+
 # ------------------------------------------------------------------ full-size configurations
 def test_config_fp32_1024(hip):
     M = N = K = 1024

@@ -50,7 +50,7 @@ def test_single_mfma_atom_against_host_product(hw, atom_id):
     assert np.array_equal(dD.cpu().numpy().astype(np.float64), want), name
 
 
-PATHS = [(O.F16, 32), (O.F16, 16), (O.BF16, 32), (O.BF16, 16), (O.I8, 32), (O.I8, 16), (O.E4M3, 32), (O.F32, 32)]
+PATHS = [(O.F16, 32), (O.F16, 16), (O.BF16, 32), (O.BF16, 16), (O.I8, 32), (O.I8, 16), (O.E4M3, 32), (O.E4M3, 16), (O.F32, 32)]
 
 
 @pytest.mark.parametrize("dtype,atom", PATHS)
@@ -58,6 +58,8 @@ PATHS = [(O.F16, 32), (O.F16, 16), (O.BF16, 32), (O.BF16, 16), (O.I8, 32), (O.I8
 def test_product_fragment_path_one_k_tile(hw, dtype, atom, transA, transB):
     import torch
     bmn, bk = (128, 32) if dtype == O.F32 else (256, 128 if dtype in (O.I8, O.E4M3) else 64)
+    if (dtype, atom) == (O.E4M3, 16) and (transA, transB) != (0, 1):
+        pytest.skip("the 16x16x128 atom is compiled for K-contiguous operands only (A [M][K], B [N][K])")
     note(f"case fragment path dtype {dtype} atom {atom} tA={transA} tB={transB} tile {bmn}x{bmn}x{bk}")
     rng = np.random.default_rng(7 * dtype + atom + 2 * transA + transB)
     maxv = {O.F16: 3, O.BF16: 3, O.I8: 127, O.E4M3: 4, O.F32: 100}[dtype]

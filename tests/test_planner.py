@@ -52,10 +52,9 @@ def test_plans_of_the_benchmark_configurations():
         assert p.grid_x == N // tile[1] and p.grid_y == M // tile[0]
         assert p.grid_x * p.grid_y >= 256 and p.xcd_remap == 1
         assert p.threads == 64 * p.waves_m * p.waves_n * p.waves_k and p.lds_bytes <= 160 * 1024
-        # the 16-bit and int8 256x256 defaults are built from 16-row atoms of twice the K depth (the part holds a higher clock on
-        # them), the rest from 32x32
-        atom = 16 if dt in (R.F16, R.BF16, R.I8) else 32
-        assert (p.mfma_m, p.mfma_n) == (atom, atom) and p.mfma_k == {R.F32: 2, R.F16: 32, R.BF16: 32, R.I8: 64, R.E4M3: 64}[dt]
+        # the 256x256 defaults are built from 16-row atoms of twice the K depth (the part holds a higher clock on them), fp32 from 32x32
+        atom = 16 if dt != R.F32 else 32
+        assert (p.mfma_m, p.mfma_n) == (atom, atom) and p.mfma_k == {R.F32: 2, R.F16: 32, R.BF16: 32, R.I8: 64, R.E4M3: 128}[dt]
         assert p.flops == 2.0 * M * N * K
         assert p.lds_a.k_contiguous == (0 if tA else 1) and p.lds_b.k_contiguous == (1 if tB else 0)
         assert p.workspace_bytes == 0 and p.kernel_id >= 0
@@ -80,7 +79,7 @@ SHAPES = [  # rows, row_bytes, k_contiguous, elem_bytes, frag_bytes, tile_mn, ti
     (256, 128, 1, 2, 16, 256, 64, 16), (64, 512, 0, 2, 16, 256, 64, 16), (256, 128, 1, 2, 16, 256, 64), (64, 512, 0, 2, 16, 256, 64), (128, 128, 1, 2, 16, 128, 64), (64, 256, 0, 2, 16, 128, 64),
     (256, 128, 1, 1, 16, 256, 128, 16), (128, 256, 0, 1, 16, 256, 128, 16),
     (256, 128, 1, 1, 16, 256, 128), (128, 256, 0, 1, 16, 256, 128), (128, 128, 1, 1, 16, 128, 128), (128, 128, 0, 1, 16, 128, 128),
-    (256, 128, 1, 1, 32, 256, 128), (128, 256, 0, 1, 32, 256, 128), (128, 128, 1, 1, 32, 128, 128), (128, 128, 0, 1, 32, 128, 128),
+    (256, 128, 1, 1, 32, 256, 128, 16), (256, 128, 1, 1, 32, 256, 128), (128, 256, 0, 1, 32, 256, 128), (128, 128, 1, 1, 32, 128, 128), (128, 128, 0, 1, 32, 128, 128),
     (128, 128, 1, 4, 16, 128, 32), (32, 512, 0, 4, 16, 128, 32), (64, 128, 1, 4, 16, 64, 32), (32, 256, 0, 4, 16, 64, 32),
     (64, 256, 1, 4, 16, 64, 64), (64, 256, 0, 4, 16, 64, 64), (64, 512, 1, 4, 16, 64, 128), (128, 64, 1, 4, 16, 128, 16),
 ]
@@ -98,6 +97,8 @@ def test_compiled_swizzle_is_what_the_cost_model_search_picks(shape):
             for M in (mn * 16,):
                 # the 16-bit and int8 256x256 tiles exist with both atoms: the descriptor names the one wanted
                 d = R.make_desc(dt, M, M, bk * 8, dtype_out=R.ACC_OF[dt] if dt != R.F16 else R.F16, transA=tA, transB=tB, tile=(mn, mn, bk), atom=atom)
+                if (dt, atom) == (R.E4M3, 16) and (tA, tB) != (0, 1):
+                    continue  # compiled for K-contiguous operands only
                 p = R.plan(d)
                 assert p.mfma_m == atom
                 for L in (p.lds_a, p.lds_b):
@@ -326,7 +327,7 @@ def test_planner_choices_for_the_benchmark_shapes_are_pinned():
         ((R.BF16, 8192, 8192, 8192, 1, R.BF16, R.EPI_NONE), "bf16_nt_256x256x64_w2x2_s2x3_a16"),
         ((R.I8, 4096, 4096, 4096, 0, R.F16, R.EPI_ROW_COL_SCALE), "i8_nn_256x256x128_w2x2_s2x3_a16"),
         ((R.E4M3, 32, 8192, 8192, 1, R.BF16, R.EPI_TENSOR_SCALE), "e4m3_nt_32x32x512_w1x1x4_s4_splitk"),
-        ((R.E4M3, 8192, 8192, 8192, 1, R.BF16, R.EPI_TENSOR_SCALE), "e4m3_nt_256x256x128_w2x2_s2x3"),
+        ((R.E4M3, 8192, 8192, 8192, 1, R.BF16, R.EPI_TENSOR_SCALE), "e4m3_nt_256x256x128_w2x2_s2x3_a16"),
     ]
     for (dt, M, N, K, tB, out, epi), name in want:
         p = R.plan(R.make_desc(dt, M, N, K, dtype_out=out, transB=tB, epilogue=epi))
