@@ -272,7 +272,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
         if (pm != k->wm || pn != k->wn) { policy_excluded = true; continue; }
       }
       if (want_split && !k->splitk) continue;
-      if ((d->K + k->bk - 1) / k->bk < k->min_k_tiles) continue;
+      if (k->min_k_tiles > 1 && (d->K + k->bk - 1) / k->bk < k->min_k_tiles) continue;
       // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
       if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
       // ... and address a tile's chunks by 32-bit lane offsets from its first row: the stored rows of one tile must span
