@@ -23,12 +23,12 @@ PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "i8": 5033.2, "e4m3": 5033.2, "f32
 FLOPS_PER_CU_CLK = {"f16": 4096, "bf16": 4096, "i8": 8192, "e4m3": 8192, "f32": 256}
 # L2-miss bytes of one fp16 4096^3 launch, a constant taken from rocprofv3 counters (not measured by this run):
 # FETCH_SIZE 98 426.0 KiB x 2.00 (the factor a 1 GiB copy shows for this counter) + WRITE_SIZE 32 774.8 KiB x 1.00
-TRAFFIC_BYTES_F16_4096 = int((98426.0 * 2.0 + 32774.8) * 1024)
+TRAFFIC_BYTES_F16_4096 = int((98508.0 * 2.0 + 32771.0) * 1024)
 TRAFFIC_SOURCE = "constant from profiles/bench_gemm_legs_f16_i8_bf16_fp8_f32.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE), not measured by this run"
 
 # duration of the register-only kernel (256 work-groups, 64 MFMAs, no memory) in a rocprofv3 kernel trace; event-timed back to
 # back the same launch takes longer by the gap between two launches
-REGISTER_ONLY_KERNEL_TRACE_MS = 0.00355
+REGISTER_ONLY_KERNEL_TRACE_MS = 0.00350
 
 SETTLE_MS = 100.0
 
