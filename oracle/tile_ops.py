@@ -1,4 +1,4 @@
-"""CPU restatement of frisk.fill, frisk.copy and frisk.reduce on rank-2 views -- TEST INFRASTRUCTURE ONLY.
+"""CPU restatement of frisk.fill, frisk.copy, frisk.reduce and elementwise frisk.block bodies on rank-2 views -- TEST INFRASTRUCTURE ONLY.
 
 The reference declares these ops and verifies their shapes (include/Dialect/Frisk/IR/FriskOps.td:348-441,
 lib/Dialect/Frisk/IR/FriskOps.cpp:1551-1767) but defines no arithmetic for them and holds no numerical
@@ -9,6 +9,12 @@ vectors: numerical parity against the reference is unpinned.  What this file fix
           type; clear = False combines the old destination value with the reduction (the accumulating form the
           online-softmax sketch of tmp/ir.mlir:33-57 relies on); shape rule of ReduceOp::verify (:1733-1767):
           destination rank = source rank - 1, the other extent is kept            (numpy's own reductions, closed forms)
+  elementwise  a frisk.block body (FriskOps.td:143-190; arith / math ops created by ffi/ir.cpp:383-394) as a postfix program
+          over operands read with a row stride and a column stride of 0 or 1, evaluated in float64 by numpy's own
+          add / subtract / multiply / divide / maximum / minimum / negative / exp2 / log2, rounded once to the output type
+          (the reference defines no arithmetic for block bodies either: parity unpinned; pinned here by closed forms --
+          identities such as log2(exp2(x)) = x, x / x = 1, max(x, x) = x -- and by numpy expressions written independently
+          in the tests)
 Arrays are in the storage types of oracle.NP_STORAGE (uint16 for f16 / bf16).
 """
 import numpy as np
