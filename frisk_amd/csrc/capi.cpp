@@ -201,7 +201,9 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
     // read by transpose reads (twice the LDS instructions) less of it is left (NN 104 against 108).  How full the round is decides:
     // 192 or 196 tiles, NN 78 against 82 us (3584^3) and 164 against 172 (4096x3072x8192), TN 79 against 85 and 169 against 182;
     // 144 tiles (3072^3), where the clock is not the limit, NN 61 against 59, TN even
-    if (k->atom == 16) c *= k->dtype == FRISK_E4M3 ? 0.96 : (!k->transA && k->transB) ? 0.93 : (tiles >= 176 ? 0.96 : 1.06);
+    // 8-bit floats on the 16x16x128 atom (NT only), us against the 32x32x64 atoms: 8192^3 331 / 351, 4096^3 45.1 / 48.8, 4096x4096x512
+    // 11.8 / 12.9, 4096x11008x4096 128 / 133, 6144^3 176 / 183; 3072^3 (144 tiles) 29.6 / 28.6
+    if (k->atom == 16) c *= k->dtype == FRISK_E4M3 ? (tiles >= 176 ? 0.94 : 1.04) : (!k->transA && k->transB) ? 0.93 : (tiles >= 176 ? 0.96 : 1.06);
   } else if (area >= 256 * 128) {
     c = 0.93;
   } else {
@@ -272,7 +274,8 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
         if (pm != k->wm || pn != k->wn) { policy_excluded = true; continue; }
       }
       if (want_split && !k->splitk) continue;
-      if (k->min_k_tiles > 1 && (d->K + k->bk - 1) / k->bk < k->min_k_tiles) continue;
+      // a kernel whose loop needs a minimum of K tiles: per slice when the descriptor asks for a split
+      if (k->min_k_tiles > 1 && (d->K + k->bk - 1) / k->bk / (want_split && d->split_k > 1 ? d->split_k : 1) < k->min_k_tiles) continue;
       // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
       if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
       // ... and address a tile's chunks by 32-bit lane offsets from its first row: the stored rows of one tile must span
@@ -327,6 +330,8 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   if (k->splitk && !no_split && d->K % k->bk == 0) {
     if (d->split_k > 1) {
       if (kt % d->split_k) return fail(FRISK_ERR_TILE, "split_k=%d does not divide the %lld K tiles", d->split_k, (long long)kt);
+      if (kt / d->split_k < k->min_k_tiles)
+        return fail(FRISK_ERR_TILE, "split_k=%d leaves %lld K tiles per slice, the chosen kernel %s needs %d", d->split_k, (long long)(kt / d->split_k), k->name, k->min_k_tiles);
       split = d->split_k;
     } else if (d->split_k == 0 && tiles < 256) {  // up to one work-group per CU, at least 4 K tiles per slice
       for (int c = 2; c <= 64; c *= 2)

@@ -53,8 +53,8 @@ VARIANTS = {
     "bf16": ("FRISK_BF16", "BF16", square(64, atom16=True)),
     "i8": ("FRISK_I8", "I8", square(128, atom16=True)),
     # 8-bit floats: the 256x256 NT variant once more on the 16x16x128 atom, whose K is the whole K tile (listed first: the planner's
-    # choice for B stored [N][K] from four K tiles on)
-    "e4m3": ("FRISK_E4M3", "E4M3", [(0, 1, 256, 256, 128, 2, 2, 2, 0, 0, 1, 3, 16)] + square(128)),
+    # choice for B stored [N][K] from four K tiles on), and its copy with the split-K store path
+    "e4m3": ("FRISK_E4M3", "E4M3", [(0, 1, 256, 256, 128, 2, 2, 2, 0, 0, 1, 3, 16), (0, 1, 256, 256, 128, 2, 2, 2, 0, 1, 1, 3, 16)] + square(128)),
     # fp32: 128x128 for large problems; 64x64 (one atom per wave) fills the chip at 1024^3, K tiles of 64 measured 5 % faster than 32;
     # the same tile with K tiles of 128 shared by two sets of four waves (8 waves, two per SIMD) another 9 % at 1024^3 (21.6 against
     # 23.9 us), where a CU holds a single work-group and nothing else hides its waits

@@ -226,6 +226,25 @@ def test_fp8_whole_tile_atom_needs_four_k_tiles(hip):
             assert e.value.status == hip.ERR_TILE
     p = hip.plan(hip.make_desc(O.E4M3, 512, 512, 384, dtype_out=O.BF16, transB=1))
     assert not hip.kernel_names()[p.kernel_id].endswith("_a16")
+    # an explicit split counts per slice (a full round of tiles, where the planner prefers the atom): 16 K tiles in 2 slices stay on it,
+    # in 8 slices they go to the 32-row atoms
+    names = hip.kernel_names()
+    assert names[hip.plan(hip.make_desc(O.E4M3, 4096, 4096, 2048, dtype_out=O.BF16, transB=1, tile=(256, 256, 128), split_k=2)).kernel_id].endswith("_a16_splitk")
+    assert names[hip.plan(hip.make_desc(O.E4M3, 4096, 4096, 2048, dtype_out=O.BF16, transB=1, tile=(256, 256, 128), split_k=8)).kernel_id].endswith("s2x3_splitk")
+
+
+def test_fp8_whole_tile_atom_split_k(hip):
+    """the 16x16x128 kernel with the split-K store path: 16 K tiles in 2 and 4 slices (8 and 4 tiles each) against the oracle, exact"""
+    M, N, K = 512, 512, 2048
+    rng = np.random.default_rng(77)
+    Ai, Bi = rng.integers(-4, 5, size=(M, K)), rng.integers(-4, 5, size=(N, K))
+    A = O.encode(O.E4M3, Ai.astype(np.float32).reshape(-1)).reshape(M, K)
+    B = O.encode(O.E4M3, Bi.astype(np.float32).reshape(-1)).reshape(N, K)
+    want = Ai.astype(np.int64) @ Bi.astype(np.int64).T
+    for split in (2, 4):
+        note(f"case fp8 16x16x128 atom, split_k={split}")
+        got = run_gemm(hip, O.E4M3, A, B, 0, 1, O.F32, M, N, K, tile=(256, 256, 128), atom=16, split_k=split)
+        assert np.array_equal(got.astype(np.int64), want)
 
 
 # ------------------------------------------------------------------ full-size configurations
