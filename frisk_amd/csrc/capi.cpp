@@ -200,10 +200,11 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
     // 16x16 atoms: the same cycles at a higher clock when most CUs are busy (fp16 4096^3 NT 100 against 112 us); with an operand
     // read by transpose reads (twice the LDS instructions) less of it is left (NN 104 against 108).  How full the round is decides:
     // 192 or 196 tiles, NN 78 against 82 us (3584^3) and 164 against 172 (4096x3072x8192), TN 79 against 85 and 169 against 182;
-    // 144 tiles (3072^3), where the clock is not the limit, NN 61 against 59, TN even
+    // 144 tiles (3072^3): NN 61 against 59 and TN even while the loop held several LDS reads per MFMA slot, NN 51.3 against 53.7
+    // (fp16), 50.4 against 51.3 (bf16), 30.6 against 31.2 (int8) since it holds one
     // 8-bit floats on the 16x16x128 atom (NT only), us against the 32x32x64 atoms: 8192^3 331 / 351, 4096^3 45.1 / 48.8, 4096x4096x512
     // 11.8 / 12.9, 4096x11008x4096 128 / 133, 6144^3 176 / 183; 3072^3 (144 tiles) 29.6 / 28.6
-    if (k->atom == 16) c *= k->dtype == FRISK_E4M3 ? (tiles >= 176 ? 0.94 : 1.04) : (!k->transA && k->transB) ? 0.93 : (tiles >= 176 ? 0.96 : 1.06);
+    if (k->atom == 16) c *= k->dtype == FRISK_E4M3 ? (tiles >= 176 ? 0.94 : 1.04) : (!k->transA && k->transB) ? 0.93 : (tiles >= 176 ? 0.96 : 0.98);
   } else if (area >= 256 * 128) {
     c = 0.93;
   } else {

@@ -94,11 +94,9 @@ def _frag_rows_cols(es, fragb, at, lane, mn0, q):
 def test_transpose_read_lane_maps_at_the_planners_addresses(hip, hw, dtype, atom):
     import torch
     es, fragb = (2, 16) if dtype == O.F16 else (1, 16)
-    # B stored [K][N]: its LDS tile has rows along K and is read by transpose reads.  A full round of 256 x 256 tiles takes
-    # the 16-row atoms for 16-bit operands, a grid below one round the 32-row atoms.
+    # B stored [K][N]: its LDS tile has rows along K and is read by transpose reads; the descriptor names the atom
     out_dt = O.F16 if dtype == O.F16 else O.I32
-    plans = [hip.plan(hip.make_desc(dtype, n, n, 4096, dtype_out=out_dt, tile=(256, 256, 0))) for n in (4096, 3072)]
-    p = next(q for q in plans if q.mfma_m == atom)
+    p = hip.plan(hip.make_desc(dtype, 4096, 4096, 4096, dtype_out=out_dt, tile=(256, 256, 0), atom=atom))
     assert p.mfma_m == atom and p.lds_b.k_contiguous == 0 and p.lds_b.read_instr == (1 if es == 2 else 2), (p.mfma_m, p.lds_b.read_instr)
     L = p.lds_b
     kpi = 4 if es == 2 else 8
