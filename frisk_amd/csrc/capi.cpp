@@ -191,7 +191,9 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
     // Measured with 16-byte fragments (K-contiguous tiles read by ds_read_b128), us, NN: 1024^3 64x64x32 18.8, x64 19.4, x128 on 8 waves
     // 19.5; 1536^3 69.4 / 73.8 / 78.6; 2048^3 128x128x32 120.8, x16 in a ring of 4 124.1, 64x64x32 123.3; 4096^3 928 / 941 / 962.
     const double c128 = k->bk <= 16 ? ((!k->transA && k->transB) ? 1.0 : 0.91) : 1.74;
-    c = area >= 128 * 128 ? c128 : (k->wk > 1 ? (tiles <= 256 ? 1.8 : 2.3) : (k->bk >= 64 ? 1.0 : 0.44));
+    // 64x64x32 per round and K tile of 32: 0.497 us over 9, 25 and 43 rounds (3072^3 429, 5120^3 1987, 4096x11008x4096 2779 us) against
+    // 1.81 us for a round of 128x128x32 (4096^3 926, 4096x11008x4096 2549): a quarter of the tile at 0.27 of the cost
+    c = area >= 128 * 128 ? c128 : (k->wk > 1 ? (tiles <= 256 ? 1.8 : 2.3) : (k->bk >= 64 ? 1.0 : (tiles <= 256 ? 0.44 : 0.465)));
   } else if (k->bm == 32) {
     // 32x32 with a 4x deeper K tile; 32x128 (8-bit: 60.1 us for 256 tiles x 64 K tiles, the rate of the 32x32 kernel per K tile)
     c = k->wk > 1 ? 0.8 : (elem_size(k->dtype) == 1 ? 0.85 : 0.25);
