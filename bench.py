@@ -234,7 +234,7 @@ def main():
     def gemm_launcher(desc, ptrs, ws=None, ws_bytes=0):
         return lambda: R.gemm(desc, *ptrs, ws, ws_bytes, cs)
 
-    # ---------------------------------------------------------------- headline: fp16 4096^3 NN (BASELINE configs[1])
+    # ---------------------------------------------------------------- headline: fp16 4096^3 NN (the configuration the metric is quoted on)
     M = N = K = 4096
     flops = 2.0 * M * N * K
     A = (torch.randn(M, K, device=dev, generator=g) / K ** 0.5).half()
