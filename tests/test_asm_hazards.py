@@ -114,3 +114,17 @@ def test_inline_assembly_mfma_kernels_keep_their_wait_states(tmp_path):
     bad = hazards(listing)
     assert not bad, "\n".join("%s: %s  ->  %s" % (n[:60], a, b) for n, a, b in bad[:10])
     assert listing.count("global_load_lds_dwordx4") > 100 and foreign_m0_uses(listing) == []
+
+
+@pytest.mark.skipif(not (os.path.exists(HIPCC) or shutil.which("hipcc")), reason="needs hipcc to produce the ISA listing")
+def test_attention_kernel_has_no_use_of_m0_besides_its_transfers(tmp_path):
+    """the attention kernel stages K and V with the same transfers (csrc/attention.hip: SK / SV issue_one): M0 is written by inline
+    assembly without a clobber, so the compiler must have no use of M0 of its own in that kernel either"""
+    out = tmp_path / "attention.s"
+    cmd = [HIPCC if os.path.exists(HIPCC) else "hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-Wno-unused-command-line-argument", "--cuda-device-only", "-S", os.path.join(CSRC, "attention.hip"), "-o", str(out)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    listing = out.read_text()
+    assert listing.count("global_load_lds_dwordx4") >= 4 * 16 and listing.count("v_mfma_f32_32x32x16") >= 4 * 32  # four kernels (f16 / bf16, two K layouts)
+    assert foreign_m0_uses(listing) == [] and "scratch_" not in listing

@@ -283,13 +283,13 @@ def test_plan_prints_lds_layouts_in_the_reference_debug_form(dtype, tile, trans_
     n = 4 * max(tile)
     kernel = h.tiled_gemm("g", n, n, n, dtype, tile=tile, trans_a=trans_a, trans_b=trans_b)
     p = F.runtime.plan(kernel, retile=False)
-    for text, (sh, mk, cs) in zip((p["lds_a"], p["lds_b"]), p["lds_swizzle"]):
+    for text, (sh, mk, cs), (sh2, mk2, cs2) in zip((p["lds_a"], p["lds_b"]), p["lds_swizzle"], p["lds_swizzle2"]):
         m = re.fullmatch(r"Layout\(shape=\[(\d+), (\d+)\], index=(affine_map<.*>)\)", text)
         assert m, text
         rows, cols = int(m.group(1)), int(m.group(2))
         i, j = L.grid(rows, cols)
         (idx,) = L.eval_affine_map(m.group(3), i, j)
-        lay = R.LdsLayout(rows=rows, row_bytes=cols * es, k_contiguous=1, row_shift=sh, row_mask=mk, chunk_shift=cs)
+        lay = R.LdsLayout(rows=rows, row_bytes=cols * es, k_contiguous=1, row_shift=sh, row_mask=mk, chunk_shift=cs, row_shift2=sh2, row_mask2=mk2, chunk_shift2=cs2)
         rr = np.random.default_rng(0).integers(0, rows, 300)
         cc = np.random.default_rng(1).integers(0, cols, 300)
         for r, c in zip(rr, cc):
