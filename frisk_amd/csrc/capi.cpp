@@ -238,6 +238,92 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
   return cost;
 }
 
+// Grids of at most 256 tiles of 128 x 128 (a few hundred rows, or a small square): no variant fills the chip with one
+// work-group per tile, so the choice is a (variant, split of K) pair.  Measured over 11 x 7 shapes (M 32 .. 2048, N and K
+// 1024 .. 16384, both layouts of B) with every variant at every split 1 .. 32, per element type: first the split of a variant
+// by rule -- the largest power of two that keeps tiles x split within `w` work-groups and `kmin` K tiles per slice (the
+// best split of a variant is within 2-5 % of this rule wherever the variant is competitive) -- then the variants compared
+// by a time model fitted to those points, in microseconds:
+//   launch + whole rounds x (K tiles x tk + ps) + a last round at K tiles x tk x (a + (1 - a) x fill) + the summing pass
+//   (r0 + r1 x megabytes of partial sums) when split.
+// The pair chosen this way is 3 % slower on average than the best pair of the sweep (worst case 1.4x); the one-size rule used
+// before lost 40 % on average on these grids.
+struct SmallGridModel { int cap, w, kmin; float launch, tk, a, r0, r1, ps; };
+static const SmallGridModel kSmallGrid[3][11] = {
+    {  // 16-bit
+        {512, 0, 0, 1.27f, 0.810f, 0.56f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
+        {256, 256, 16, 3.60f, 0.481f, 0.66f, 4.09f, 0.400f, 0.24f},  // 128x128 s3
+        {256, 0, 0, 4.78f, 0.756f, 0.80f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
+        {256, 0, 0, 4.36f, 0.773f, 0.79f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
+        {256, 256, 16, 5.49f, 1.263f, 0.57f, 6.06f, 0.255f, 9.73f},  // 256x256 s2
+        {256, 256, 16, 4.81f, 1.224f, 0.72f, 4.51f, 0.273f, 6.12f},  // 256x256 s2 a16
+        {256, 0, 0, 5.28f, 1.565f, 0.54f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
+        {128, 128, 16, 3.18f, 0.184f, 1.00f, 2.82f, 2.230f, 0.00f},  // 32x128 s3 n
+        {128, 128, 16, 3.10f, 0.191f, 1.00f, 2.91f, 2.152f, 0.00f},  // 32x128 s3 t
+        {512, 512, 16, 2.57f, 0.879f, 0.33f, 4.86f, 2.257f, 0.00f},  // 32x32 s2 t
+        {256, 128, 16, 2.63f, 0.508f, 0.65f, 3.85f, 0.948f, 0.28f},  // 32x32 s4 t
+    },
+    {  // int8
+        {512, 0, 0, 2.69f, 0.840f, 0.49f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
+        {256, 256, 16, 3.81f, 0.492f, 0.65f, 4.56f, 0.316f, 0.00f},  // 128x128 s3
+        {256, 0, 0, 5.35f, 0.763f, 0.80f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
+        {256, 0, 0, 4.97f, 0.779f, 0.79f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
+        {256, 256, 16, 4.38f, 1.710f, 0.53f, 5.49f, 0.170f, 6.61f},  // 256x256 s2
+        {256, 256, 16, 7.90f, 1.525f, 0.41f, 6.69f, 0.144f, 3.75f},  // 256x256 s2 a16
+        {256, 0, 0, 6.32f, 1.647f, 0.50f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
+        {128, 128, 16, 3.18f, 0.182f, 1.00f, 3.33f, 1.949f, 0.00f},  // 32x128 s3 n
+        {128, 128, 16, 3.33f, 0.173f, 1.00f, 3.80f, 1.483f, 0.00f},  // 32x128 s3 t
+        {512, 512, 16, 2.98f, 0.812f, 0.31f, 3.19f, 1.143f, 0.52f},  // 32x32 s2 t
+        {256, 128, 16, 3.08f, 0.461f, 0.62f, 3.55f, 0.000f, 0.55f},  // 32x32 s4 t
+    },
+    {  // 8-bit float
+        {512, 0, 0, 2.57f, 0.808f, 0.45f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
+        {256, 256, 16, 3.83f, 0.411f, 0.64f, 4.68f, 0.239f, 0.11f},  // 128x128 s3
+        {256, 0, 0, 5.19f, 0.670f, 0.77f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
+        {256, 0, 0, 5.14f, 0.678f, 0.75f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
+        {256, 256, 16, 6.82f, 1.427f, 0.57f, 3.84f, 0.170f, 4.62f},  // 256x256 s2
+        {256, 256, 16, 6.39f, 1.361f, 0.57f, 4.95f, 0.169f, 4.13f},  // 256x256 s2 a16
+        {256, 0, 0, 4.41f, 1.699f, 0.56f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
+        {128, 128, 16, 3.18f, 0.162f, 1.00f, 3.26f, 1.565f, 0.00f},  // 32x128 s3 n
+        {128, 128, 16, 3.18f, 0.162f, 1.00f, 3.26f, 1.565f, 0.00f},  // 32x128 s3 t
+        {512, 512, 16, 3.14f, 0.806f, 0.26f, 3.02f, 0.900f, 0.31f},  // 32x32 s2 t
+        {256, 128, 16, 3.30f, 0.436f, 0.50f, 3.13f, 0.000f, 0.40f},  // 32x32 s4 t
+    },
+};
+static int small_grid_class(const KernelEntry* k) {
+  if (k->bm == 32) return k->bn == 32 ? (k->stages >= 3 ? 10 : 9) : (k->transB ? 8 : 7);
+  if ((int64_t)k->bm * k->bn >= 256 * 256) return k->wm * k->wn > 4 ? 6 : (k->atom == 16 ? 5 : 4);
+  if (k->bm == 256) return 3;
+  if (k->bn == 256) return 2;
+  return k->stages >= 3 ? 1 : 0;
+}
+static bool small_grid(const frisk_gemm_desc* d) {
+  return d->dtype_ab != FRISK_F32 && d->split_k <= 1 && ((d->M + 127) / 128) * ((d->N + 127) / 128) <= 256;
+}
+static const SmallGridModel& small_grid_model(const KernelEntry* k) {
+  return kSmallGrid[k->dtype == FRISK_I8 ? 1 : (k->dtype == FRISK_E4M3 ? 2 : 0)][small_grid_class(k)];
+}
+static int small_grid_split(const KernelEntry* k, const frisk_gemm_desc* d, bool no_split) {
+  const SmallGridModel& m = small_grid_model(k);
+  if (!k->splitk || no_split || d->split_k == 1 || m.w == 0 || d->K % k->bk) return 1;
+  const int64_t tiles = ((d->M + k->bm - 1) / k->bm) * ((d->N + k->bn - 1) / k->bn), kt = d->K / k->bk;
+  int split = 1;
+  for (int c = 2; c <= 64; c *= 2)
+    if (tiles * c <= m.w && kt % c == 0 && kt / c >= std::max(m.kmin, k->min_k_tiles)) split = c;
+  return split;
+}
+static double small_grid_cost(const KernelEntry* k, const frisk_gemm_desc* d, bool no_split) {
+  const SmallGridModel& m = small_grid_model(k);
+  const int split = small_grid_split(k, d, no_split);
+  const int64_t tiles = ((d->M + k->bm - 1) / k->bm) * ((d->N + k->bn - 1) / k->bn);
+  const double kt = (double)((d->K + k->bk - 1) / k->bk) / split;
+  const int64_t wgs = tiles * split, full = wgs / m.cap, rest = wgs % m.cap;
+  double t = m.launch + (double)full * (kt * m.tk + m.ps);
+  if (rest) t += kt * m.tk * (m.a + (1.0 - m.a) * (double)rest / m.cap);
+  if (split > 1) t += m.r0 + m.r1 * ((double)d->M * (double)d->N * split * 4.0 / 1e6);
+  return k->guard ? 3.0 * t : t;
+}
+
 static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_model, bool force_guard = false, bool no_split = false) {
   int st = validate(d);
   if (st != FRISK_OK) return st;
@@ -257,6 +343,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
   double best_cost = 0.0;
   bool policy_excluded = false;
   bool any_layout = false, tile_requested = d->tile_m || d->tile_n || d->tile_k || d->waves_m || d->waves_n || d->stages || d->atom;
+  const bool small = small_grid(d);
   auto search = [&](bool want_split) {
     for (size_t i = 0; i < ks.size(); ++i) {
       const KernelEntry* k = ks[i];
@@ -286,7 +373,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
       const double span_a = (double)d->lda * es * (d->transA ? k->bk : k->bm), span_b = (double)d->ldb * es * (d->transB ? k->bn : k->bk);
       if (!k->guard && (span_a >= 4294967296.0 || span_b >= 4294967296.0)) continue;
       if (k->guard && best >= 0 && !ks[best]->guard) continue;  // never a guarded kernel when a fast one fits
-      const double cost = estimated_cost(k, d);
+      const double cost = small && !want_split ? small_grid_cost(k, d, no_split) : estimated_cost(k, d);
       // ties: the first listed variant is the tuned default
       if (best < 0 || (ks[best]->guard && !k->guard) || cost < best_cost) { best = (int)i; best_cost = cost; }
     }
@@ -336,6 +423,8 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
       if (kt / d->split_k < k->min_k_tiles)
         return fail(FRISK_ERR_TILE, "split_k=%d leaves %lld K tiles per slice, the chosen kernel %s needs %d", d->split_k, (long long)(kt / d->split_k), k->name, k->min_k_tiles);
       split = d->split_k;
+    } else if (small) {
+      split = small_grid_split(k, d, no_split);
     } else if (d->split_k == 0 && tiles < 256) {  // up to one work-group per CU, at least 4 K tiles per slice
       for (int c = 2; c <= 64; c *= 2)
         if (kt % c == 0 && kt / c >= 4 && tiles * c <= 256) split = c;

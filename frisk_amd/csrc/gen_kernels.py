@@ -33,6 +33,11 @@ def square(bk, atom16=False):
             if atom16:
                 out.append((ta, tb, 256, 256, bk, 2, 2, 2, 0, 1, 1, 3, 16))
             out.append((ta, tb, 256, 256, bk, 2, 2, 2, 0, 1, 1, 3))
+    # the 128x128 variant with 3 + 3 tiles once more with the split-K store path: grids of well under 256 tiles with a long K
+    # (M of a few hundred rows), where K is split over the idle CUs
+    for ta in (0, 1):
+        for tb in (0, 1):
+            out.append((ta, tb, 128, 128, bk, 2, 2, 3, 0, 1, 1, 3))
     # skinny variants (M a multiple of 32), bound by streaming B: K may be split over the grid's y dimension.
     #   B stored [N][K]: 32x32 tile, 512-byte K rows, the 4 waves split the K steps of a tile
     #   B stored [K][N]: 32x128 tile, 4 waves side by side

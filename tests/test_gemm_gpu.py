@@ -405,9 +405,10 @@ def test_empty_problems(hip):
 @pytest.mark.parametrize("transB", [0, 1])
 def test_skinny_split_k(hip, dtype, transB):
     """M = 32 and 64: a 32-row kernel runs (B stored [N][K]: 32x32 tile whose 4 waves split the K steps; B stored
-    [K][N]: 32x128 tile); every split factor gives the oracle's result (int8: the same bits)"""
+    [K][N]: 32x128 tile); every split factor gives the oracle's result (int8: the same bits).  K is deep enough for the planner to
+    split it by itself (slices of at least 16 K tiles)"""
     for M in (32, 64):
-        N, K = 384, 32 * BK[dtype]
+        N, K = 384, 128 * BK[dtype]
         sa, sb = stored_shapes(M, N, K, 0, transB)
         A = make_operand(dtype, *sa, seed=41, tensor=0, scale=0.5)
         B = make_operand(dtype, *sb, seed=41, tensor=1, scale=0.5)
@@ -425,6 +426,29 @@ def test_skinny_split_k(hip, dtype, transB):
                 check(dtype, out_dt, got, ref)
         # the planner's own split needs no workspace to be correct: without one the launch runs unsplit
         got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, workspace=False)
+        if dtype == O.I8:
+            assert np.array_equal(got, ref)
+        else:
+            check(dtype, out_dt, got, ref)
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.I8, O.E4M3])
+@pytest.mark.parametrize("transB", [0, 1])
+def test_small_grid_gets_a_split_of_128_tiles(hip, dtype, transB):
+    """a few hundred rows and a long K: the planner's small-grid model picks the 128x128 variant with the split-K store path and a
+    split of its own (16 tiles x 8 slices of 16 K tiles here); same result as the oracle, with and without a workspace"""
+    M, N, K = 512, 512, 128 * BK[dtype]
+    sa, sb = stored_shapes(M, N, K, 0, transB)
+    A = make_operand(dtype, *sa, seed=47, tensor=0, scale=0.5)
+    B = make_operand(dtype, *sb, seed=47, tensor=1, scale=0.5)
+    out_dt = DEFAULT_OUT[dtype]
+    ref = O.gemm_i32(A, B, 0, transB) if dtype == O.I8 else O.gemm_f64(dtype, A, B, 0, transB)
+    p = hip.plan(hip.make_desc(dtype, M, N, K, dtype_out=out_dt, transB=bool(transB)))
+    name = hip.kernel_names()[p.kernel_id]
+    assert (p.tile_m, p.tile_n, p.split_k) == (128, 128, 8) and name.endswith("_s3_splitk") and p.workspace_bytes == 8 * M * N * 4, (name, p.split_k)
+    for workspace in (True, False):
+        note(f"case small grid {NAMES[dtype]} tB={transB} M={M} N={N} K={K} workspace={workspace}")
+        got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, workspace=workspace)
         if dtype == O.I8:
             assert np.array_equal(got, ref)
         else:

@@ -244,9 +244,19 @@ def test_planner_ranks_variants_by_estimated_time():
     assert pick(R.BF16, 1024, 8192, 8192, transB=True) == "bf16_nt_256x128x64_w2x2_s3"
     assert pick(R.F16, 8192, 8192, 8192) == "f16_nn_256x256x64_w2x2_s2x3_a16"
     assert pick(R.E4M3, 32, 8192, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s4_splitk"
-    # more than 256 such tiles: the ring of 2, two work-groups per CU (29.3 us against 35.8 for 512 tiles, 52.8 against 60.1 for 1024)
-    assert pick(R.E4M3, 32, 16384, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s2_splitk"
-    assert pick(R.E4M3, 32, 32768, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s2_splitk"
+    # twice as wide: 128 work-groups of the 32x128 kernel (20.7 us; the 32x32 kernel with a ring of 2, two work-groups per CU, 29.3)
+    assert pick(R.E4M3, 32, 16384, 8192, transB=True) == "e4m3_nt_32x128x128_w1x4_s3_splitk"
+    assert pick(R.E4M3, 32, 32768, 8192, transB=True) == "e4m3_nt_32x128x128_w1x4_s3_splitk"
+    # grids of at most 256 tiles of 128x128: a (variant, split) pair from the small-grid model.  Measured, us, before -> now:
+    # 256x4096x4096 NT 41.9 -> 23.6 (64 tiles of 128x128 in 4 slices; 2 slices 21.6, the vendor library 18.9), 128x4096x4096 NN
+    # 25.4 -> 18.6, 512x2048x8192 NN 49.1 -> 35.5 (vendor 46.2)
+    p = R.plan(R.make_desc(R.F16, 256, 4096, 4096, transB=True))
+    assert (names[p.kernel_id], p.split_k, p.workspace_bytes) == ("f16_nt_128x128x64_w2x2_s3_splitk", 4, 4 * 256 * 4096 * 4)
+    p = R.plan(R.make_desc(R.F16, 512, 2048, 8192))
+    assert names[p.kernel_id] == "f16_nn_128x128x64_w2x2_s3_splitk" and p.split_k == 4
+    # ... and a descriptor that forbids splitting gets the best unsplit variant
+    p = R.plan(R.make_desc(R.F16, 512, 2048, 8192, split_k=1))
+    assert p.split_k == 1 and p.workspace_bytes == 0
     assert pick(R.F16, 1024, 1024, 1024) == "f16_nn_32x128x64_w1x4_s3_splitk"
     # 576 tiles = 2 rounds + 64: the variant with the split-K store path, its last 64 tiles as 4 work-groups each
     assert pick(R.I8, 6144, 6144, 6144) == "i8_nn_256x256x128_w2x2_s2x3_a16_splitk"
