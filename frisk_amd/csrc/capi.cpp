@@ -239,59 +239,63 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
 }
 
 // Grids of at most 256 tiles of 128 x 128 (a few hundred rows, or a small square): no variant fills the chip with one
-// work-group per tile, so the choice is a (variant, split of K) pair.  Measured over 11 x 7 shapes (M 32 .. 2048, N and K
-// 1024 .. 16384, both layouts of B) with every variant at every split 1 .. 32, per element type: first the split of a variant
-// by rule -- the largest power of two that keeps tiles x split within `w` work-groups and `kmin` K tiles per slice (the
-// best split of a variant is within 2-5 % of this rule wherever the variant is competitive) -- then the variants compared
-// by a time model fitted to those points, in microseconds:
+// work-group per tile, so the choice is a (variant, split of K) pair.  Measured over 11 x 7 + 4 shapes (M 32 .. 2048, N and K
+// 1024 .. 16384, both layouts of B) with every variant at every split 1 .. 32, per element type.  A variant's splits are the
+// powers of two that keep tiles x split within `w` work-groups and `kmin` K tiles per slice (the best split of a variant is
+// the largest of these or close to it wherever the variant is competitive); variants and splits are compared by a time model
+// fitted to those points, in microseconds:
 //   launch + whole rounds x (K tiles x tk + ps) + a last round at K tiles x tk x (a + (1 - a) x fill) + the summing pass
 //   (r0 + r1 x megabytes of partial sums) when split.
 // The pair chosen this way is 3 % slower on average than the best pair of the sweep (worst case 1.4x); the one-size rule used
 // before lost 40 % on average on these grids.
 struct SmallGridModel { int cap, w, kmin; float launch, tk, a, r0, r1, ps; };
-static const SmallGridModel kSmallGrid[3][11] = {
+static const SmallGridModel kSmallGrid[3][12] = {
     {  // 16-bit
-        {512, 0, 0, 1.27f, 0.810f, 0.56f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
-        {256, 256, 16, 3.60f, 0.481f, 0.66f, 4.09f, 0.400f, 0.24f},  // 128x128 s3
-        {256, 0, 0, 4.78f, 0.756f, 0.80f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
-        {256, 0, 0, 4.36f, 0.773f, 0.79f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
-        {256, 256, 16, 5.49f, 1.263f, 0.57f, 6.06f, 0.255f, 9.73f},  // 256x256 s2
-        {256, 256, 16, 4.81f, 1.224f, 0.72f, 4.51f, 0.273f, 6.12f},  // 256x256 s2 a16
-        {256, 0, 0, 5.28f, 1.565f, 0.54f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
-        {128, 128, 16, 3.18f, 0.184f, 1.00f, 2.82f, 2.230f, 0.00f},  // 32x128 s3 n
-        {128, 128, 16, 3.10f, 0.191f, 1.00f, 2.91f, 2.152f, 0.00f},  // 32x128 s3 t
-        {512, 512, 16, 2.57f, 0.879f, 0.33f, 4.86f, 2.257f, 0.00f},  // 32x32 s2 t
-        {256, 128, 16, 2.63f, 0.508f, 0.65f, 3.85f, 0.948f, 0.28f},  // 32x32 s4 t
+        {512, 0, 0, 1.30f, 0.805f, 0.56f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
+        {256, 256, 16, 3.59f, 0.475f, 0.68f, 4.51f, 0.300f, 0.79f},  // 128x128 s3
+        {256, 0, 0, 4.88f, 0.766f, 0.78f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
+        {256, 0, 0, 4.57f, 0.781f, 0.75f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
+        {256, 256, 16, 7.51f, 1.264f, 0.56f, 5.65f, 0.196f, 10.78f},  // 256x256 s2
+        {256, 256, 16, 6.99f, 1.219f, 0.62f, 5.04f, 0.220f, 6.68f},  // 256x256 s2 a16
+        {256, 0, 0, 5.22f, 1.563f, 0.54f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
+        {128, 128, 16, 2.58f, 0.216f, 1.00f, 5.56f, 0.300f, 0.00f},  // 32x128 s3 n
+        {128, 128, 16, 2.32f, 0.225f, 1.00f, 6.02f, 0.300f, 0.00f},  // 32x128 s3 t
+        {512, 512, 16, 1.95f, 1.024f, 0.35f, 6.11f, 0.300f, 0.00f},  // 32x32 s2 t
+        {256, 128, 16, 2.61f, 0.558f, 0.52f, 4.28f, 0.000f, 0.00f},  // 32x32 s4 t
+        {512, 256, 16, 2.67f, 0.481f, 0.45f, 5.30f, 0.300f, 4.54f},  // 64x128 s3
     },
     {  // int8
-        {512, 0, 0, 2.69f, 0.840f, 0.49f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
-        {256, 256, 16, 3.81f, 0.492f, 0.65f, 4.56f, 0.316f, 0.00f},  // 128x128 s3
-        {256, 0, 0, 5.35f, 0.763f, 0.80f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
-        {256, 0, 0, 4.97f, 0.779f, 0.79f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
-        {256, 256, 16, 4.38f, 1.710f, 0.53f, 5.49f, 0.170f, 6.61f},  // 256x256 s2
-        {256, 256, 16, 7.90f, 1.525f, 0.41f, 6.69f, 0.144f, 3.75f},  // 256x256 s2 a16
-        {256, 0, 0, 6.32f, 1.647f, 0.50f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
-        {128, 128, 16, 3.18f, 0.182f, 1.00f, 3.33f, 1.949f, 0.00f},  // 32x128 s3 n
-        {128, 128, 16, 3.33f, 0.173f, 1.00f, 3.80f, 1.483f, 0.00f},  // 32x128 s3 t
-        {512, 512, 16, 2.98f, 0.812f, 0.31f, 3.19f, 1.143f, 0.52f},  // 32x32 s2 t
-        {256, 128, 16, 3.08f, 0.461f, 0.62f, 3.55f, 0.000f, 0.55f},  // 32x32 s4 t
+        {512, 0, 0, 2.69f, 0.812f, 0.50f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
+        {256, 256, 16, 3.72f, 0.485f, 0.67f, 4.67f, 0.300f, 0.43f},  // 128x128 s3
+        {256, 0, 0, 5.30f, 0.773f, 0.78f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
+        {256, 0, 0, 4.99f, 0.777f, 0.78f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
+        {256, 256, 16, 14.92f, 1.460f, 0.44f, 0.00f, 0.142f, 9.60f},  // 256x256 s2
+        {256, 256, 16, 7.65f, 1.409f, 0.51f, 5.50f, 0.182f, 4.66f},  // 256x256 s2 a16
+        {256, 0, 0, 6.25f, 1.689f, 0.48f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
+        {128, 128, 16, 2.76f, 0.217f, 1.00f, 5.44f, 0.300f, 0.00f},  // 32x128 s3 n
+        {128, 128, 16, 3.05f, 0.193f, 1.00f, 5.80f, 0.300f, 0.00f},  // 32x128 s3 t
+        {512, 512, 16, 3.07f, 0.903f, 0.26f, 3.71f, 0.300f, 0.00f},  // 32x32 s2 t
+        {256, 128, 16, 3.20f, 0.498f, 0.52f, 3.38f, 0.000f, 0.27f},  // 32x32 s4 t
+        {512, 256, 16, 3.02f, 0.524f, 0.41f, 4.98f, 0.300f, 2.17f},  // 64x128 s3
     },
     {  // 8-bit float
-        {512, 0, 0, 2.57f, 0.808f, 0.45f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
-        {256, 256, 16, 3.83f, 0.411f, 0.64f, 4.68f, 0.239f, 0.11f},  // 128x128 s3
-        {256, 0, 0, 5.19f, 0.670f, 0.77f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
-        {256, 0, 0, 5.14f, 0.678f, 0.75f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
-        {256, 256, 16, 6.82f, 1.427f, 0.57f, 3.84f, 0.170f, 4.62f},  // 256x256 s2
-        {256, 256, 16, 6.39f, 1.361f, 0.57f, 4.95f, 0.169f, 4.13f},  // 256x256 s2 a16
-        {256, 0, 0, 4.41f, 1.699f, 0.56f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
-        {128, 128, 16, 3.18f, 0.162f, 1.00f, 3.26f, 1.565f, 0.00f},  // 32x128 s3 n
-        {128, 128, 16, 3.18f, 0.162f, 1.00f, 3.26f, 1.565f, 0.00f},  // 32x128 s3 t
-        {512, 512, 16, 3.14f, 0.806f, 0.26f, 3.02f, 0.900f, 0.31f},  // 32x32 s2 t
-        {256, 128, 16, 3.30f, 0.436f, 0.50f, 3.13f, 0.000f, 0.40f},  // 32x32 s4 t
+        {512, 0, 0, 2.74f, 0.791f, 0.43f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
+        {256, 256, 16, 3.70f, 0.406f, 0.69f, 4.14f, 0.300f, 0.51f},  // 128x128 s3
+        {256, 0, 0, 5.20f, 0.662f, 0.78f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
+        {256, 0, 0, 5.11f, 0.672f, 0.75f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
+        {256, 256, 16, 8.03f, 1.287f, 0.53f, 5.18f, 0.151f, 7.09f},  // 256x256 s2
+        {256, 256, 16, 7.13f, 1.237f, 0.59f, 5.61f, 0.165f, 4.45f},  // 256x256 s2 a16
+        {256, 0, 0, 5.18f, 1.644f, 0.51f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
+        {128, 128, 16, 2.80f, 0.192f, 1.00f, 5.19f, 0.300f, 0.00f},  // 32x128 s3 n
+        {128, 128, 16, 2.80f, 0.192f, 1.00f, 5.19f, 0.300f, 0.00f},  // 32x128 s3 t
+        {512, 512, 16, 3.00f, 0.895f, 0.26f, 3.27f, 0.300f, 0.00f},  // 32x32 s2 t
+        {256, 128, 16, 3.22f, 0.484f, 0.45f, 2.93f, 0.000f, 0.14f},  // 32x32 s4 t
+        {512, 256, 16, 3.01f, 0.438f, 0.46f, 4.52f, 0.300f, 2.45f},  // 64x128 s3
     },
 };
 static int small_grid_class(const KernelEntry* k) {
   if (k->bm == 32) return k->bn == 32 ? (k->stages >= 3 ? 10 : 9) : (k->transB ? 8 : 7);
+  if (k->bm == 64) return 11;
   if ((int64_t)k->bm * k->bn >= 256 * 256) return k->wm * k->wn > 4 ? 6 : (k->atom == 16 ? 5 : 4);
   if (k->bm == 256) return 3;
   if (k->bn == 256) return 2;
@@ -303,18 +307,7 @@ static bool small_grid(const frisk_gemm_desc* d) {
 static const SmallGridModel& small_grid_model(const KernelEntry* k) {
   return kSmallGrid[k->dtype == FRISK_I8 ? 1 : (k->dtype == FRISK_E4M3 ? 2 : 0)][small_grid_class(k)];
 }
-static int small_grid_split(const KernelEntry* k, const frisk_gemm_desc* d, bool no_split) {
-  const SmallGridModel& m = small_grid_model(k);
-  if (!k->splitk || no_split || d->split_k == 1 || m.w == 0 || d->K % k->bk) return 1;
-  const int64_t tiles = ((d->M + k->bm - 1) / k->bm) * ((d->N + k->bn - 1) / k->bn), kt = d->K / k->bk;
-  int split = 1;
-  for (int c = 2; c <= 64; c *= 2)
-    if (tiles * c <= m.w && kt % c == 0 && kt / c >= std::max(m.kmin, k->min_k_tiles)) split = c;
-  return split;
-}
-static double small_grid_cost(const KernelEntry* k, const frisk_gemm_desc* d, bool no_split) {
-  const SmallGridModel& m = small_grid_model(k);
-  const int split = small_grid_split(k, d, no_split);
+static double small_grid_time(const SmallGridModel& m, const KernelEntry* k, const frisk_gemm_desc* d, int split) {
   const int64_t tiles = ((d->M + k->bm - 1) / k->bm) * ((d->N + k->bn - 1) / k->bn);
   const double kt = (double)((d->K + k->bk - 1) / k->bk) / split;
   const int64_t wgs = tiles * split, full = wgs / m.cap, rest = wgs % m.cap;
@@ -322,6 +315,27 @@ static double small_grid_cost(const KernelEntry* k, const frisk_gemm_desc* d, bo
   if (rest) t += kt * m.tk * (m.a + (1.0 - m.a) * (double)rest / m.cap);
   if (split > 1) t += m.r0 + m.r1 * ((double)d->M * (double)d->N * split * 4.0 / 1e6);
   return k->guard ? 3.0 * t : t;
+}
+// the split of a variant: among the powers of two the rule admits, the one the model makes fastest; *cost receives its time
+static int small_grid_split(const KernelEntry* k, const frisk_gemm_desc* d, bool no_split, double* cost = nullptr) {
+  const SmallGridModel& m = small_grid_model(k);
+  int best = 1;
+  double best_t = small_grid_time(m, k, d, 1);
+  if (k->splitk && !no_split && d->split_k != 1 && m.w != 0 && d->K % k->bk == 0) {
+    const int64_t tiles = ((d->M + k->bm - 1) / k->bm) * ((d->N + k->bn - 1) / k->bn), kt = d->K / k->bk;
+    for (int c = 2; c <= 64; c *= 2)
+      if (tiles * c <= m.w && kt % c == 0 && kt / c >= std::max(m.kmin, k->min_k_tiles)) {
+        const double t = small_grid_time(m, k, d, c);
+        if (t < best_t) { best = c; best_t = t; }
+      }
+  }
+  if (cost) *cost = best_t;
+  return best;
+}
+static double small_grid_cost(const KernelEntry* k, const frisk_gemm_desc* d, bool no_split) {
+  double t = 0.0;
+  small_grid_split(k, d, no_split, &t);
+  return t;
 }
 
 static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_model, bool force_guard = false, bool no_split = false) {

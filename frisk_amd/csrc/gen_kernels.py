@@ -47,6 +47,10 @@ def square(bk, atom16=False):
     out.append((0, 1, 32, 32, 4 * bk, 1, 1, 2, 0, 1, 4))
     for tb in (0, 1):
         out.append((0, tb, 32, 128, bk, 1, 4, 3, 0, 1, 1))
+    # 64 rows: from M = 64 to a few hundred rows a 32-row tile streams B once per 32 rows of A (fp16 64x8192x8192 NT 34.2 us, the
+    # vendor library 26.6); with 64-row tiles 26.6, 128x8192x8192 28.6 against 47.4, 256x4096x4096 18.3 against 23.6
+    for tb in (0, 1):
+        out.append((0, tb, 64, 128, bk, 2, 2, 3, 0, 1, 1))
     # guarded variants: any shape, any leading dimension, element-aligned pointers
     for ta in (0, 1):
         for tb in (0, 1):

@@ -404,8 +404,8 @@ def test_empty_problems(hip):
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.I8, O.E4M3])
 @pytest.mark.parametrize("transB", [0, 1])
 def test_skinny_split_k(hip, dtype, transB):
-    """M = 32 and 64: a 32-row kernel runs (B stored [N][K]: 32x32 tile whose 4 waves split the K steps; B stored
-    [K][N]: 32x128 tile); every split factor gives the oracle's result (int8: the same bits).  K is deep enough for the planner to
+    """M = 32 and 64: a 32- or 64-row kernel runs (32 rows, B stored [N][K]: 32x32 tile whose 4 waves split the K steps; B stored
+    [K][N]: 32x128 tile; 64 rows: 64x128); every split factor gives the oracle's result (int8: the same bits).  K is deep enough for the planner to
     split it by itself (slices of at least 16 K tiles)"""
     for M in (32, 64):
         N, K = 384, 128 * BK[dtype]
@@ -416,10 +416,11 @@ def test_skinny_split_k(hip, dtype, transB):
         ref = O.gemm_i32(A, B, 0, transB) if dtype == O.I8 else O.gemm_f64(dtype, A, B, 0, transB)
         d = hip.make_desc(dtype, M, N, K, dtype_out=out_dt, transB=bool(transB))
         p = hip.plan(d)
-        assert p.tile_m == 32 and p.split_k > 1 and p.workspace_bytes == p.split_k * M * N * 4, (p.tile_m, p.split_k, p.workspace_bytes)
-        for split in (0, 1, 2, 4, 8):
-            note(f"case skinny {NAMES[dtype]} tB={transB} M={M} N={N} K={K} split_k={split}")
-            got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, split_k=split)
+        assert p.tile_m in (32, 64) and p.tile_m <= M and p.split_k > 1 and p.workspace_bytes == p.split_k * M * N * 4, (p.tile_m, p.split_k, p.workspace_bytes)
+        # the planner's variant at every split, then the 32-row kernels by name (at M = 64 the planner prefers 64-row tiles)
+        for split, rows in ((0, 0), (1, 0), (2, 0), (4, 0), (8, 0), (0, 32), (2, 32)):
+            note(f"case skinny {NAMES[dtype]} tB={transB} M={M} N={N} K={K} split_k={split} tile_m={rows}")
+            got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, split_k=split, tile=(rows, 0, 0))
             if dtype == O.I8:
                 assert np.array_equal(got, ref)
             else:
@@ -434,9 +435,10 @@ def test_skinny_split_k(hip, dtype, transB):
 
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.I8, O.E4M3])
 @pytest.mark.parametrize("transB", [0, 1])
-def test_small_grid_gets_a_split_of_128_tiles(hip, dtype, transB):
-    """a few hundred rows and a long K: the planner's small-grid model picks the 128x128 variant with the split-K store path and a
-    split of its own (16 tiles x 8 slices of 16 K tiles here); same result as the oracle, with and without a workspace"""
+def test_small_grid_gets_a_split_of_its_own(hip, dtype, transB):
+    """a few hundred rows and a long K: the planner's small-grid model picks a variant with the split-K store path and a split of
+    its own; same result as the oracle with the planner's pair, without a workspace (one pass), and with the 128x128 and 64x128
+    variants named by the descriptor at splits 2 and 4"""
     M, N, K = 512, 512, 128 * BK[dtype]
     sa, sb = stored_shapes(M, N, K, 0, transB)
     A = make_operand(dtype, *sa, seed=47, tensor=0, scale=0.5)
@@ -445,10 +447,12 @@ def test_small_grid_gets_a_split_of_128_tiles(hip, dtype, transB):
     ref = O.gemm_i32(A, B, 0, transB) if dtype == O.I8 else O.gemm_f64(dtype, A, B, 0, transB)
     p = hip.plan(hip.make_desc(dtype, M, N, K, dtype_out=out_dt, transB=bool(transB)))
     name = hip.kernel_names()[p.kernel_id]
-    assert (p.tile_m, p.tile_n, p.split_k) == (128, 128, 8) and name.endswith("_s3_splitk") and p.workspace_bytes == 8 * M * N * 4, (name, p.split_k)
-    for workspace in (True, False):
-        note(f"case small grid {NAMES[dtype]} tB={transB} M={M} N={N} K={K} workspace={workspace}")
-        got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, workspace=workspace)
+    assert p.tile_m in (64, 128) and p.split_k > 1 and name.endswith("_s3_splitk") and p.workspace_bytes == p.split_k * M * N * 4, (name, p.split_k)
+    cases = [dict(workspace=True), dict(workspace=False)]
+    cases += [dict(tile=(bm, 128, BK[dtype]), split_k=sk) for bm in (64, 128) for sk in (2, 4)]
+    for kw in cases:
+        note(f"case small grid {NAMES[dtype]} tB={transB} M={M} N={N} K={K} {kw}")
+        got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, **kw)
         if dtype == O.I8:
             assert np.array_equal(got, ref)
         else:

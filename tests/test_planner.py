@@ -248,16 +248,20 @@ def test_planner_ranks_variants_by_estimated_time():
     assert pick(R.E4M3, 32, 16384, 8192, transB=True) == "e4m3_nt_32x128x128_w1x4_s3_splitk"
     assert pick(R.E4M3, 32, 32768, 8192, transB=True) == "e4m3_nt_32x128x128_w1x4_s3_splitk"
     # grids of at most 256 tiles of 128x128: a (variant, split) pair from the small-grid model.  Measured, us, before -> now:
-    # 256x4096x4096 NT 41.9 -> 23.6 (64 tiles of 128x128 in 4 slices; 2 slices 21.6, the vendor library 18.9), 128x4096x4096 NN
-    # 25.4 -> 18.6, 512x2048x8192 NN 49.1 -> 35.5 (vendor 46.2)
-    p = R.plan(R.make_desc(R.F16, 256, 4096, 4096, transB=True))
-    assert (names[p.kernel_id], p.split_k, p.workspace_bytes) == ("f16_nt_128x128x64_w2x2_s3_splitk", 4, 4 * 256 * 4096 * 4)
+    # 64x8192x8192 NT 40.1 -> 26.5 (64-row tiles, K in 4 slices; the vendor library 26.4), 128x8192x8192 NT 47.4 -> 30.5 (vendor
+    # 37.4), 256x4096x4096 NT 41.9 -> 20.2 (vendor 18.8), 512x2048x8192 NN 49.1 -> 31.2 (vendor 47.1)
+    p = R.plan(R.make_desc(R.F16, 64, 8192, 8192, transB=True))
+    assert (names[p.kernel_id], p.split_k, p.workspace_bytes) == ("f16_nt_64x128x64_w2x2_s3_splitk", 4, 4 * 64 * 8192 * 4)
+    p = R.plan(R.make_desc(R.F16, 128, 8192, 8192, transB=True))
+    assert (names[p.kernel_id], p.split_k) == ("f16_nt_128x128x64_w2x2_s3_splitk", 4)
+    assert pick(R.F16, 256, 4096, 4096, transB=True) == "f16_nt_64x128x64_w2x2_s3_splitk"
     p = R.plan(R.make_desc(R.F16, 512, 2048, 8192))
     assert names[p.kernel_id] == "f16_nn_128x128x64_w2x2_s3_splitk" and p.split_k == 4
     # ... and a descriptor that forbids splitting gets the best unsplit variant
     p = R.plan(R.make_desc(R.F16, 512, 2048, 8192, split_k=1))
     assert p.split_k == 1 and p.workspace_bytes == 0
-    assert pick(R.F16, 1024, 1024, 1024) == "f16_nn_32x128x64_w1x4_s3_splitk"
+    # 1024^3: 128 work-groups of 64x128 (6.8 us, the same as 256 of 32x128; 128x128 tiles 9.0, the vendor library 17.6)
+    assert pick(R.F16, 1024, 1024, 1024) == "f16_nn_64x128x64_w2x2_s3_splitk"
     # 576 tiles = 2 rounds + 64: the variant with the split-K store path, its last 64 tiles as 4 work-groups each
     assert pick(R.I8, 6144, 6144, 6144) == "i8_nn_256x256x128_w2x2_s2x3_a16_splitk"
     p = R.plan(R.make_desc(R.I8, 6144, 6144, 6144, dtype_out=R.I32))

@@ -40,7 +40,7 @@ def test_static_workspace_matches_caller_workspace_on_two_calls_in_a_row(hip):
     assert hip.static_workspace_bytes() == 32 << 20
     # first call: int8 64 x 2048 x 8192 NN, the planner splits K (skinny problem); dequantising epilogue
     # second call: a smaller problem of the same kind, then an fp16 one with an explicit split on the 256 x 256 tile
-    cases = [(O.I8, 64, 2048, 8192, 0, O.F16, 0, hip.EPI_ROW_COL_SCALE), (O.I8, 32, 512, 4096, 0, O.I32, 0, hip.EPI_NONE),
+    cases = [(O.I8, 64, 2048, 8192, 0, O.F16, 0, hip.EPI_ROW_COL_SCALE), (O.I8, 32, 512, 8192, 0, O.I32, 0, hip.EPI_NONE),
              (O.F16, 512, 512, 2048, 1, O.F16, 4, hip.EPI_NONE)]
     for n, (dt, M, N, K, tB, out_dt, split, epi) in enumerate(cases):
         A = make_operand(dt, M, K, 40 + n, 0, scale=0.05)
