@@ -239,58 +239,59 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
 }
 
 // Grids of at most 256 tiles of 128 x 128 (a few hundred rows, or a small square): no variant fills the chip with one
-// work-group per tile, so the choice is a (variant, split of K) pair.  Measured over 11 x 7 + 4 shapes (M 32 .. 2048, N and K
-// 1024 .. 16384, both layouts of B) with every variant at every split 1 .. 32, per element type.  A variant's splits are the
-// powers of two that keep tiles x split within `w` work-groups and `kmin` K tiles per slice (the best split of a variant is
-// the largest of these or close to it wherever the variant is competitive); variants and splits are compared by a time model
-// fitted to those points, in microseconds:
+// work-group per tile, so the choice is a (variant, split of K) pair.  Measured per element type over 81 skinny shapes (M 32 ..
+// 2048, N and K 1024 .. 28672) and 90 squarish ones (sides 768 .. 2048, K 1024 .. 8192), both layouts of B, every variant at
+// every split 1 .. 32.  A variant's splits are the powers of two that keep tiles x split within `w` work-groups and `kmin` K
+// tiles per slice; variants and splits are compared by a time model fitted to the sweep, in microseconds:
 //   launch + whole rounds x (K tiles x tk + ps) + a last round at K tiles x tk x (a + (1 - a) x fill) + the summing pass
-//   (r0 + r1 x megabytes of partial sums) when split.
-// The pair chosen this way is 3 % slower on average than the best pair of the sweep (worst case 1.4x); the one-size rule used
-// before lost 40 % on average on these grids.
-struct SmallGridModel { int cap, w, kmin; float launch, tk, a, r0, r1, ps; };
+//   (r0 + r1 x megabytes of partial sums) when split;
+// variants of which a CU holds two work-groups (`cap` 512) pay tk2 per K tile more once any CU holds its second one:
+// K tiles x tk2 x (a2 + (1 - a2) x fill of the second half).  The pair chosen this way is 1-2 % slower on average than the
+// best pair of the sweep (worst case 1.3x, more than 1.2x in 5 of 483 cases); the one-size rule used before lost 35-40 % on
+// average on the skinny shapes.
+struct SmallGridModel { int cap, w, kmin; float launch, tk, a, r0, r1, ps, tk2, a2; };
 static const SmallGridModel kSmallGrid[3][12] = {
     {  // 16-bit
-        {512, 0, 0, 1.30f, 0.805f, 0.56f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
-        {256, 256, 16, 3.59f, 0.475f, 0.68f, 4.51f, 0.300f, 0.79f},  // 128x128 s3
-        {256, 0, 0, 4.88f, 0.766f, 0.78f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
-        {256, 0, 0, 4.57f, 0.781f, 0.75f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
-        {256, 256, 16, 7.51f, 1.264f, 0.56f, 5.65f, 0.196f, 10.78f},  // 256x256 s2
-        {256, 256, 16, 6.99f, 1.219f, 0.62f, 5.04f, 0.220f, 6.68f},  // 256x256 s2 a16
-        {256, 0, 0, 5.22f, 1.563f, 0.54f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
-        {128, 128, 16, 2.58f, 0.216f, 1.00f, 5.56f, 0.300f, 0.00f},  // 32x128 s3 n
-        {128, 128, 16, 2.32f, 0.225f, 1.00f, 6.02f, 0.300f, 0.00f},  // 32x128 s3 t
-        {512, 512, 16, 1.95f, 1.024f, 0.35f, 6.11f, 0.300f, 0.00f},  // 32x32 s2 t
-        {256, 128, 16, 2.61f, 0.558f, 0.52f, 4.28f, 0.000f, 0.00f},  // 32x32 s4 t
-        {512, 256, 16, 2.67f, 0.481f, 0.45f, 5.30f, 0.300f, 4.54f},  // 64x128 s3
+        {512, 0, 0, 1.10f, 0.645f, 0.72f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
+        {256, 256, 16, 3.40f, 0.471f, 0.70f, 4.39f, 0.300f, 1.75f, 0.000f, 0.00f},  // 128x128 s3
+        {256, 0, 0, 4.99f, 0.759f, 0.81f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
+        {256, 0, 0, 4.51f, 0.767f, 0.80f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
+        {256, 256, 16, 9.96f, 1.343f, 0.52f, 0.00f, 0.300f, 6.73f, 0.000f, 0.00f},  // 256x256 s2
+        {256, 256, 16, 6.84f, 1.231f, 0.63f, 2.46f, 0.300f, 3.47f, 0.000f, 0.00f},  // 256x256 s2 a16
+        {256, 0, 0, 5.67f, 1.578f, 0.53f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
+        {512, 128, 16, 1.65f, 0.343f, 0.71f, 4.92f, 0.300f, 0.00f, 0.202f, 0.44f},  // 32x128 s3 n
+        {512, 128, 16, 1.36f, 0.371f, 0.67f, 5.09f, 0.300f, 0.00f, 0.172f, 0.45f},  // 32x128 s3 t
+        {512, 256, 16, 2.07f, 0.644f, 0.59f, 6.13f, 0.300f, 0.00f, 0.286f, 1.00f},  // 32x32 s2 t
+        {256, 128, 16, 2.66f, 0.541f, 0.54f, 4.38f, 0.000f, 0.10f, 0.000f, 0.00f},  // 32x32 s4 t
+        {512, 256, 16, 2.56f, 0.325f, 0.69f, 5.82f, 0.300f, 0.57f, 0.292f, 0.66f},  // 64x128 s3
     },
     {  // int8
-        {512, 0, 0, 2.69f, 0.812f, 0.50f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
-        {256, 256, 16, 3.72f, 0.485f, 0.67f, 4.67f, 0.300f, 0.43f},  // 128x128 s3
-        {256, 0, 0, 5.30f, 0.773f, 0.78f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
-        {256, 0, 0, 4.99f, 0.777f, 0.78f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
-        {256, 256, 16, 14.92f, 1.460f, 0.44f, 0.00f, 0.142f, 9.60f},  // 256x256 s2
-        {256, 256, 16, 7.65f, 1.409f, 0.51f, 5.50f, 0.182f, 4.66f},  // 256x256 s2 a16
-        {256, 0, 0, 6.25f, 1.689f, 0.48f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
-        {128, 128, 16, 2.76f, 0.217f, 1.00f, 5.44f, 0.300f, 0.00f},  // 32x128 s3 n
-        {128, 128, 16, 3.05f, 0.193f, 1.00f, 5.80f, 0.300f, 0.00f},  // 32x128 s3 t
-        {512, 512, 16, 3.07f, 0.903f, 0.26f, 3.71f, 0.300f, 0.00f},  // 32x32 s2 t
-        {256, 128, 16, 3.20f, 0.498f, 0.52f, 3.38f, 0.000f, 0.27f},  // 32x32 s4 t
-        {512, 256, 16, 3.02f, 0.524f, 0.41f, 4.98f, 0.300f, 2.17f},  // 64x128 s3
+        {512, 0, 0, 2.19f, 0.638f, 0.73f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
+        {256, 256, 16, 3.61f, 0.485f, 0.68f, 4.86f, 0.300f, 0.93f, 0.000f, 0.00f},  // 128x128 s3
+        {256, 0, 0, 5.14f, 0.776f, 0.80f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
+        {256, 0, 0, 4.87f, 0.770f, 0.81f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
+        {256, 256, 16, 10.06f, 1.408f, 0.55f, 0.00f, 0.300f, 5.92f, 0.000f, 0.00f},  // 256x256 s2
+        {256, 256, 16, 7.05f, 1.400f, 0.56f, 3.42f, 0.276f, 1.59f, 0.000f, 0.00f},  // 256x256 s2 a16
+        {256, 0, 0, 6.29f, 1.631f, 0.51f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
+        {512, 128, 16, 2.26f, 0.354f, 0.68f, 4.64f, 0.300f, 0.11f, 0.164f, 0.68f},  // 32x128 s3 n
+        {512, 128, 16, 2.41f, 0.351f, 0.63f, 4.80f, 0.134f, 0.33f, 0.135f, 0.85f},  // 32x128 s3 t
+        {512, 256, 16, 3.12f, 0.530f, 0.49f, 3.60f, 0.300f, 0.32f, 0.314f, 1.00f},  // 32x32 s2 t
+        {256, 128, 16, 3.15f, 0.479f, 0.57f, 3.42f, 0.000f, 0.51f, 0.000f, 0.00f},  // 32x32 s4 t
+        {512, 256, 16, 2.95f, 0.341f, 0.66f, 5.45f, 0.300f, 0.00f, 0.323f, 0.56f},  // 64x128 s3
     },
     {  // 8-bit float
-        {512, 0, 0, 2.74f, 0.791f, 0.43f, 5.00f, 0.300f, 1.00f},  // 128x128 s2
-        {256, 256, 16, 3.70f, 0.406f, 0.69f, 4.14f, 0.300f, 0.51f},  // 128x128 s3
-        {256, 0, 0, 5.20f, 0.662f, 0.78f, 5.00f, 0.300f, 1.00f},  // 128x256 s3
-        {256, 0, 0, 5.11f, 0.672f, 0.75f, 5.00f, 0.300f, 1.00f},  // 256x128 s3
-        {256, 256, 16, 8.03f, 1.287f, 0.53f, 5.18f, 0.151f, 7.09f},  // 256x256 s2
-        {256, 256, 16, 7.13f, 1.237f, 0.59f, 5.61f, 0.165f, 4.45f},  // 256x256 s2 a16
-        {256, 0, 0, 5.18f, 1.644f, 0.51f, 5.00f, 0.300f, 1.00f},  // 256x256 s2 w8
-        {128, 128, 16, 2.80f, 0.192f, 1.00f, 5.19f, 0.300f, 0.00f},  // 32x128 s3 n
-        {128, 128, 16, 2.80f, 0.192f, 1.00f, 5.19f, 0.300f, 0.00f},  // 32x128 s3 t
-        {512, 512, 16, 3.00f, 0.895f, 0.26f, 3.27f, 0.300f, 0.00f},  // 32x32 s2 t
-        {256, 128, 16, 3.22f, 0.484f, 0.45f, 2.93f, 0.000f, 0.14f},  // 32x32 s4 t
-        {512, 256, 16, 3.01f, 0.438f, 0.46f, 4.52f, 0.300f, 2.45f},  // 64x128 s3
+        {512, 0, 0, 2.06f, 0.617f, 0.67f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
+        {256, 256, 16, 3.54f, 0.415f, 0.71f, 3.74f, 0.300f, 0.95f, 0.000f, 0.00f},  // 128x128 s3
+        {256, 0, 0, 5.00f, 0.659f, 0.82f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
+        {256, 0, 0, 4.82f, 0.662f, 0.80f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
+        {256, 256, 16, 7.77f, 1.244f, 0.63f, 1.61f, 0.267f, 5.93f, 0.000f, 0.00f},  // 256x256 s2
+        {256, 256, 16, 6.67f, 1.222f, 0.66f, 2.81f, 0.263f, 1.55f, 0.000f, 0.00f},  // 256x256 s2 a16
+        {256, 0, 0, 5.36f, 1.029f, 1.00f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
+        {512, 128, 16, 2.31f, 0.327f, 0.66f, 4.06f, 0.300f, 0.21f, 0.145f, 1.00f},  // 32x128 s3 n
+        {512, 128, 16, 2.31f, 0.327f, 0.66f, 4.06f, 0.300f, 0.21f, 0.145f, 1.00f},  // 32x128 s3 t
+        {512, 256, 16, 3.09f, 0.528f, 0.48f, 3.11f, 0.300f, 0.30f, 0.297f, 1.00f},  // 32x32 s2 t
+        {256, 128, 16, 3.24f, 0.455f, 0.50f, 3.04f, 0.000f, 0.43f, 0.000f, 0.00f},  // 32x32 s4 t
+        {512, 256, 16, 3.00f, 0.301f, 0.72f, 4.51f, 0.300f, 0.16f, 0.258f, 0.70f},  // 64x128 s3
     },
 };
 static int small_grid_class(const KernelEntry* k) {
@@ -311,8 +312,15 @@ static double small_grid_time(const SmallGridModel& m, const KernelEntry* k, con
   const int64_t tiles = ((d->M + k->bm - 1) / k->bm) * ((d->N + k->bn - 1) / k->bn);
   const double kt = (double)((d->K + k->bk - 1) / k->bk) / split;
   const int64_t wgs = tiles * split, full = wgs / m.cap, rest = wgs % m.cap;
-  double t = m.launch + (double)full * (kt * m.tk + m.ps);
-  if (rest) t += kt * m.tk * (m.a + (1.0 - m.a) * (double)rest / m.cap);
+  double t = m.launch, whole = kt * m.tk + m.ps, last = 0.0;
+  if (m.cap == 512) {  // two work-groups per CU: the second one of any CU sets the pace of the round
+    whole += kt * m.tk2;
+    const double f1 = (double)std::min<int64_t>(rest, 256) / 256.0, f2 = (double)std::max<int64_t>(rest - 256, 0) / 256.0;
+    last = kt * (m.tk * (m.a + (1.0 - m.a) * f1) + (rest > 256 ? m.tk2 * (m.a2 + (1.0 - m.a2) * f2) : 0.0));
+  } else {
+    last = kt * m.tk * (m.a + (1.0 - m.a) * (double)rest / m.cap);
+  }
+  t += (double)full * whole + (rest ? last : 0.0);
   if (split > 1) t += m.r0 + m.r1 * ((double)d->M * (double)d->N * split * 4.0 / 1e6);
   return k->guard ? 3.0 * t : t;
 }

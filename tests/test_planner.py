@@ -244,8 +244,9 @@ def test_planner_ranks_variants_by_estimated_time():
     assert pick(R.BF16, 1024, 8192, 8192, transB=True) == "bf16_nt_256x128x64_w2x2_s3"
     assert pick(R.F16, 8192, 8192, 8192) == "f16_nn_256x256x64_w2x2_s2x3_a16"
     assert pick(R.E4M3, 32, 8192, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s4_splitk"
-    # twice as wide: 128 work-groups of the 32x128 kernel (20.7 us; the 32x32 kernel with a ring of 2, two work-groups per CU, 29.3)
-    assert pick(R.E4M3, 32, 16384, 8192, transB=True) == "e4m3_nt_32x128x128_w1x4_s3_splitk"
+    # twice as wide, 512 such tiles: the ring of 2, two work-groups per CU (21.4 us; 128 work-groups of the 32x128 kernel 20.4); four
+    # times as wide: the 32x128 kernel (28672 columns: 35.1 us)
+    assert pick(R.E4M3, 32, 16384, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s2_splitk"
     assert pick(R.E4M3, 32, 32768, 8192, transB=True) == "e4m3_nt_32x128x128_w1x4_s3_splitk"
     # grids of at most 256 tiles of 128x128: a (variant, split) pair from the small-grid model.  Measured, us, before -> now:
     # 64x8192x8192 NT 40.1 -> 26.5 (64-row tiles, K in 4 slices; the vendor library 26.4), 128x8192x8192 NT 47.4 -> 30.5 (vendor
