@@ -173,8 +173,12 @@ static int tail_split_of(const KernelEntry* k, int64_t tiles, int64_t kt, bool w
   if (!k->splitk || k->bm < 128 || k->wk > 1 || !whole_k_tiles || tiles <= 256) return 1;
   const int64_t rest = tiles % 256;
   if (rest == 0 || rest > 128) return 1;
+  // shallower slices do not repay the second launch (measured); the 8-bit kernels run a K tile of twice the depth in the same
+  // time, so the summing pass weighs twice as much against their slices (fp8 5120x4096x4096: 64 tiles in 4 slices of 8 K tiles
+  // 92.4 us, unsplit 84, 256x128 tiles 81.4)
+  const int min_slice = elem_size(k->dtype) == 1 ? 16 : 8;
   for (int s = 8; s >= 2; s /= 2)
-    if (rest * s <= 256 && kt % s == 0 && kt / s >= 8) return s;  // shallower slices do not repay the second launch (measured)
+    if (rest * s <= 256 && kt % s == 0 && kt / s >= min_slice) return s;
   return 1;
 }
 
@@ -182,7 +186,16 @@ static int tail_split_of(const KernelEntry* k, int64_t tiles, int64_t kt, bool w
 // (256); a K tile of a 256x256 tile costs 1.5 units when every CU runs one, and less when the chip is partly idle
 // (less contention in the L2 and a higher clock): factor 0.6 + 0.4 * fill.  The constants are measured on fp16 problems
 // between 1024^3 and 8192^3 and carry over to the 8-bit types, whose K tiles hold the same number of bytes.
-static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
+// the split the planner gives a grid below one round of a variant with the split-K store path: up to one work-group per CU,
+// at least 4 K tiles per slice
+static int sub_round_split(const KernelEntry* k, int64_t tiles, int64_t kt) {
+  int split = 1;
+  for (int c = 2; c <= 64; c *= 2)
+    if (kt % c == 0 && kt / c >= std::max(4, k->min_k_tiles) && tiles * c <= 256) split = c;
+  return split;
+}
+
+static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d, bool may_split = false) {
   const int64_t tiles = ((d->M + k->bm - 1) / k->bm) * ((d->N + k->bn - 1) / k->bn);
   const double kt = (double)((d->K + k->bk - 1) / k->bk);
   double c;  // cost of one K tile with the chip full
@@ -223,6 +236,14 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d) {
   }
   const int64_t full = tiles / 256, rest = tiles % 256;
   const double rest_fill = (double)rest / 256.0;
+  if (may_split && k->splitk && k->bm >= 128 && tiles < 256 && d->K % k->bk == 0) {
+    // below one round with a deep K the planner splits K over the idle CUs (2048x4096x16384 fp16: 128 tiles of 256x256 in 2
+    // slices 209.5 us, 256 tiles of 256x128 unsplit 243.6): the slices' K tiles at the fill they reach, plus the summing pass
+    const int cs = sub_round_split(k, tiles, (int64_t)kt);
+    // (measured: the slices' loops 8 % above the per-K-tile rate of a long loop, the pass at 256 KiB per tile and slice in 0.07 us;
+    // 1024x8192x8192 comes out even with 256x128 tiles unsplit, 123.7 against 123.9 us, and stays unsplit)
+    if (cs > 1) return kt / cs * c * (0.6 + 0.4 * rest_fill * cs) * 1.08 + 5.0 + 0.07 * (double)(tiles * cs);
+  }
   double cost = (double)full * kt * c;
   if (const int ts = tail_split_of(k, tiles, (int64_t)kt, d->K % k->bk == 0); ts > 1) {
     // the last `rest` tiles as ts work-groups each, a ts-th of the K tiles apiece, plus the pass that sums them
@@ -395,7 +416,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
       const double span_a = (double)d->lda * es * (d->transA ? k->bk : k->bm), span_b = (double)d->ldb * es * (d->transB ? k->bn : k->bk);
       if (!k->guard && (span_a >= 4294967296.0 || span_b >= 4294967296.0)) continue;
       if (k->guard && best >= 0 && !ks[best]->guard) continue;  // never a guarded kernel when a fast one fits
-      const double cost = small && !want_split ? small_grid_cost(k, d, no_split) : estimated_cost(k, d);
+      const double cost = small && !want_split ? small_grid_cost(k, d, no_split) : estimated_cost(k, d, !want_split && !no_split && d->split_k == 0);
       // ties: the first listed variant is the tuned default
       if (best < 0 || (ks[best]->guard && !k->guard) || cost < best_cost) { best = (int)i; best_cost = cost; }
     }
@@ -447,9 +468,8 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
       split = d->split_k;
     } else if (small) {
       split = small_grid_split(k, d, no_split);
-    } else if (d->split_k == 0 && tiles < 256) {  // up to one work-group per CU, at least 4 K tiles per slice
-      for (int c = 2; c <= 64; c *= 2)
-        if (kt % c == 0 && kt / c >= 4 && tiles * c <= 256) split = c;
+    } else if (d->split_k == 0 && tiles < 256) {
+      split = sub_round_split(k, tiles, kt);
     } else if (d->split_k == 0) {
       const int ts = tail_split_of(k, tiles, kt, true);
       if (ts > 1) {

@@ -504,8 +504,8 @@ def test_split_k_status_codes(hip):
 @pytest.mark.parametrize("dtype,transA,transB", [(O.F16, 0, 0), (O.BF16, 0, 1), (O.F16, 1, 0), (O.BF16, 1, 1), (O.I8, 0, 0), (O.E4M3, 0, 1)])
 def test_tail_split(hip, dtype, transA, transB):
     """17 x 17 = 289 tiles of 256 x 256: one round of 256 and 33 left over, which run as 4 work-groups each (a quarter of the
-    32 K tiles apiece) and are summed through the workspace; without a workspace the same launch runs unsplit.  Both give
-    the oracle's result (int8: the same bits)"""
+    32 K tiles apiece; the 8-bit types as 2 each, their slices hold at least 16 K tiles) and are summed through the workspace;
+    without a workspace the same launch runs unsplit.  Both give the oracle's result (int8: the same bits)"""
     M = N = 17 * 256
     K = 32 * BK[dtype]
     sa, sb = stored_shapes(M, N, K, transA, transB)
@@ -514,7 +514,8 @@ def test_tail_split(hip, dtype, transA, transB):
     out_dt = DEFAULT_OUT[dtype]
     ref = O.gemm_i32(A, B, transA, transB) if dtype == O.I8 else O.gemm_f64(dtype, A, B, transA, transB)
     p = hip.plan(hip.make_desc(dtype, M, N, K, dtype_out=out_dt, transA=bool(transA), transB=bool(transB)))
-    assert (p.tile_m, p.tile_n, p.tail_tiles, p.tail_split) == (256, 256, 33, 4) and p.workspace_bytes == 4 * 33 * 256 * 256 * 4
+    ts = 2 if dtype in (O.I8, O.E4M3) else 4
+    assert (p.tile_m, p.tile_n, p.tail_tiles, p.tail_split) == (256, 256, 33, ts) and p.workspace_bytes == ts * 33 * 256 * 256 * 4
     for workspace in (True, False):
         note(f"case tail split {NAMES[dtype]} tA={transA} tB={transB} {M}x{N}x{K} workspace={workspace}")
         got = run_gemm(hip, dtype, A, B, transA, transB, out_dt, M, N, K, workspace=workspace)

@@ -263,10 +263,17 @@ def test_planner_ranks_variants_by_estimated_time():
     assert p.split_k == 1 and p.workspace_bytes == 0
     # 1024^3: 128 work-groups of 64x128 (6.8 us, the same as 256 of 32x128; 128x128 tiles 9.0, the vendor library 17.6)
     assert pick(R.F16, 1024, 1024, 1024) == "f16_nn_64x128x64_w2x2_s3_splitk"
-    # 576 tiles = 2 rounds + 64: the variant with the split-K store path, its last 64 tiles as 4 work-groups each
+    # 576 tiles = 2 rounds + 64: the variant with the split-K store path, its last 64 tiles as 2 work-groups each (8-bit types:
+    # slices of at least 16 K tiles; 186 us against 192 with 4 slices of 12), fp16 as 4 each (slices of at least 8)
     assert pick(R.I8, 6144, 6144, 6144) == "i8_nn_256x256x128_w2x2_s2x3_a16_splitk"
     p = R.plan(R.make_desc(R.I8, 6144, 6144, 6144, dtype_out=R.I32))
+    assert (p.tail_tiles, p.tail_split, p.split_k) == (64, 2, 1) and p.workspace_bytes == 2 * 64 * 256 * 256 * 4
+    p = R.plan(R.make_desc(R.F16, 6144, 6144, 6144))
     assert (p.tail_tiles, p.tail_split, p.split_k) == (64, 4, 1) and p.workspace_bytes == 4 * 64 * 256 * 256 * 4
+    # below one round of 256x256 tiles with a deep K: K in slices over the idle CUs (2048x4096x16384: 128 tiles x 2 slices 200 us,
+    # 256 tiles of 256x128 unsplit 243); 1024x8192x8192 comes out even (123.7 against 123.9 us) and stays unsplit
+    p = R.plan(R.make_desc(R.F16, 2048, 4096, 16384))
+    assert (names[p.kernel_id], p.split_k) == ("f16_nn_256x256x64_w2x2_s2x3_a16_splitk", 2)
     # whole rounds, more than half a round left over, or a descriptor that forbids splitting: no tail
     for shape, kw in (((8192, 8192, 8192), {}), ((5120, 5120, 5120), {}), ((6144, 6144, 6144), {"split_k": 1})):
         p = R.plan(R.make_desc(R.F16, *shape, **kw))
