@@ -447,6 +447,42 @@ def main():
                           "launch_floor_ms + bytes / streaming rate"})
         del Bf
 
+        # grids far below one round of tiles (a few hundred rows against an 8192 x 8192 fp16 B stored [N][K], rotating over 3 buffers of
+        # 128 MiB): the planner's small-grid choice of a (variant, split-K) pair, beside the vendor library on the same tensors
+        small = {}
+        Bs = [(torch.randn(8192, 8192, device=dev, generator=g) / 64).half() for _ in range(3)]
+        for Msm in (64, 256):
+            Asm = (torch.randn(Msm, 8192, device=dev, generator=g) / 64).half()
+            Csm = torch.empty(Msm, 8192, device=dev, dtype=torch.float16)
+            Cvm = torch.empty_like(Csm)
+            dsm = R.make_desc(R.F16, Msm, 8192, 8192, dtype_out=R.F16, transB=True)
+            psm = R.plan(dsm)
+            wsm_bytes = R.workspace_bytes(dsm)
+            wsm = torch.empty(max(wsm_bytes, 16), dtype=torch.uint8, device=dev)
+            turn = [0, 0]
+
+            def ours_small():
+                b_ = Bs[turn[0] % len(Bs)]
+                turn[0] += 1
+                R.gemm(dsm, Asm.data_ptr(), b_.data_ptr(), Csm.data_ptr(), None, None, wsm.data_ptr() if wsm_bytes else None, wsm_bytes, cs)
+
+            def vendor_small():
+                b_ = Bs[turn[1] % len(Bs)]
+                turn[1] += 1
+                return torch.matmul(Asm, b_.t(), out=Cvm)
+            tsm = time_launches(torch, ours_small, a.steps, a.warmup, stream)
+            sm_bytes = 2 * (Msm * 8192 + 8192 * 8192 + Msm * 8192)
+            key = "%dx8192x8192" % Msm
+            small[key] = {"kernel": R.kernel_names()[psm.kernel_id], "split_k": psm.split_k, "workspace_bytes": wsm_bytes,
+                          "kernel_ms": round(tsm["mean_ms"], 5), "kernel_ms_median": round(tsm["median_ms"], 5), "kernel_ms_min": round(tsm["min_ms"], 5),
+                          "algorithmic_GBps": round(sm_bytes / (tsm["mean_ms"] * 1e-3) / 1e9, 1),
+                          "TFLOPs": round(2.0 * Msm * 8192 * 8192 / (tsm["mean_ms"] * 1e-3) / 1e12, 1)}
+            vendor["fp16_small_grid_" + key + "_nt"] = vendor_leg(torch, "torch.matmul(A, Bt.t(), out=C), fp16 %s NT, B rotating over the same 3 buffers" % key,
+                                                                  vendor_small, 2.0 * Msm * 8192 * 8192, a.steps, a.warmup, stream, tsm["mean_ms"])
+            del Asm, Csm, Cvm, wsm
+        legs["fp16_small_grid_nt"] = small
+        del Bs
+
         # the dialect's data-movement ops on a 32768 x 8192 f16 view (512 MiB per array: twice the last-level cache)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 

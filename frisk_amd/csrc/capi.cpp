@@ -262,57 +262,58 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d, boo
 // Grids of at most 256 tiles of 128 x 128 (a few hundred rows, or a small square): no variant fills the chip with one
 // work-group per tile, so the choice is a (variant, split of K) pair.  Measured per element type over 81 skinny shapes (M 32 ..
 // 2048, N and K 1024 .. 28672) and 90 squarish ones (sides 768 .. 2048, K 1024 .. 8192), both layouts of B, every variant at
-// every split 1 .. 32.  A variant's splits are the powers of two that keep tiles x split within `w` work-groups and `kmin` K
+// every split 1 .. 32, B taken in turn from as many copies as fill 400 MiB so that it streams from HBM as the weights of a model
+// do (with one B of at most 128 MiB the last-level cache serves it: 26.5 instead of 38 us at fp16 64x8192x8192).  A variant's splits are the powers of two that keep tiles x split within `w` work-groups and `kmin` K
 // tiles per slice; variants and splits are compared by a time model fitted to the sweep, in microseconds:
 //   launch + whole rounds x (K tiles x tk + ps) + a last round at K tiles x tk x (a + (1 - a) x fill) + the summing pass
 //   (r0 + r1 x megabytes of partial sums) when split;
 // variants of which a CU holds two work-groups (`cap` 512) pay tk2 per K tile more once any CU holds its second one:
-// K tiles x tk2 x (a2 + (1 - a2) x fill of the second half).  The pair chosen this way is 1-2 % slower on average than the
-// best pair of the sweep (worst case 1.3x, more than 1.2x in 5 of 483 cases); the one-size rule used before lost 35-40 % on
+// K tiles x tk2 x (a2 + (1 - a2) x fill of the second half).  The pair chosen this way is 2 % slower on average than the
+// best pair of the sweep (more than 1.2x in 24 of 966 cases); the one-size rule used before lost 35-40 % on
 // average on the skinny shapes.
 struct SmallGridModel { int cap, w, kmin; float launch, tk, a, r0, r1, ps, tk2, a2; };
 static const SmallGridModel kSmallGrid[3][12] = {
     {  // 16-bit
-        {512, 0, 0, 1.10f, 0.645f, 0.72f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
-        {256, 256, 16, 3.40f, 0.471f, 0.70f, 4.39f, 0.300f, 1.75f, 0.000f, 0.00f},  // 128x128 s3
-        {256, 0, 0, 4.99f, 0.759f, 0.81f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
-        {256, 0, 0, 4.51f, 0.767f, 0.80f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
-        {256, 256, 16, 9.96f, 1.343f, 0.52f, 0.00f, 0.300f, 6.73f, 0.000f, 0.00f},  // 256x256 s2
-        {256, 256, 16, 6.84f, 1.231f, 0.63f, 2.46f, 0.300f, 3.47f, 0.000f, 0.00f},  // 256x256 s2 a16
-        {256, 0, 0, 5.67f, 1.578f, 0.53f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
-        {512, 128, 16, 1.65f, 0.343f, 0.71f, 4.92f, 0.300f, 0.00f, 0.202f, 0.44f},  // 32x128 s3 n
-        {512, 128, 16, 1.36f, 0.371f, 0.67f, 5.09f, 0.300f, 0.00f, 0.172f, 0.45f},  // 32x128 s3 t
-        {512, 256, 16, 2.07f, 0.644f, 0.59f, 6.13f, 0.300f, 0.00f, 0.286f, 1.00f},  // 32x32 s2 t
-        {256, 128, 16, 2.66f, 0.541f, 0.54f, 4.38f, 0.000f, 0.10f, 0.000f, 0.00f},  // 32x32 s4 t
-        {512, 256, 16, 2.56f, 0.325f, 0.69f, 5.82f, 0.300f, 0.57f, 0.292f, 0.66f},  // 64x128 s3
+        {512, 0, 0, 0.53f, 0.784f, 0.77f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
+        {256, 256, 16, 2.10f, 0.545f, 0.76f, 5.70f, 0.300f, 3.26f, 0.000f, 0.00f},  // 128x128 s3
+        {256, 0, 0, 3.54f, 0.882f, 0.76f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
+        {256, 0, 0, 4.08f, 0.829f, 0.75f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
+        {256, 256, 16, 9.22f, 1.460f, 0.54f, 0.00f, 0.300f, 9.07f, 0.000f, 0.00f},  // 256x256 s2
+        {256, 256, 16, 5.66f, 1.306f, 0.66f, 3.18f, 0.300f, 7.33f, 0.000f, 0.00f},  // 256x256 s2 a16
+        {256, 0, 0, 0.59f, 2.078f, 0.52f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
+        {512, 128, 16, 0.42f, 0.455f, 0.73f, 6.44f, 0.300f, 0.00f, 0.189f, 1.00f},  // 32x128 s3 n
+        {512, 128, 16, 0.15f, 0.464f, 0.76f, 6.40f, 0.300f, 0.00f, 0.168f, 1.00f},  // 32x128 s3 t
+        {512, 256, 16, 2.35f, 0.747f, 0.69f, 7.36f, 0.000f, 0.00f, 0.231f, 0.70f},  // 32x32 s2 t
+        {256, 128, 16, 2.87f, 0.578f, 0.66f, 6.52f, 0.000f, 0.06f, 0.000f, 0.00f},  // 32x32 s4 t
+        {512, 256, 16, 1.38f, 0.435f, 0.72f, 7.11f, 0.300f, 2.05f, 0.303f, 0.41f},  // 64x128 s3
     },
     {  // int8
-        {512, 0, 0, 2.19f, 0.638f, 0.73f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
-        {256, 256, 16, 3.61f, 0.485f, 0.68f, 4.86f, 0.300f, 0.93f, 0.000f, 0.00f},  // 128x128 s3
-        {256, 0, 0, 5.14f, 0.776f, 0.80f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
-        {256, 0, 0, 4.87f, 0.770f, 0.81f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
-        {256, 256, 16, 10.06f, 1.408f, 0.55f, 0.00f, 0.300f, 5.92f, 0.000f, 0.00f},  // 256x256 s2
-        {256, 256, 16, 7.05f, 1.400f, 0.56f, 3.42f, 0.276f, 1.59f, 0.000f, 0.00f},  // 256x256 s2 a16
-        {256, 0, 0, 6.29f, 1.631f, 0.51f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
-        {512, 128, 16, 2.26f, 0.354f, 0.68f, 4.64f, 0.300f, 0.11f, 0.164f, 0.68f},  // 32x128 s3 n
-        {512, 128, 16, 2.41f, 0.351f, 0.63f, 4.80f, 0.134f, 0.33f, 0.135f, 0.85f},  // 32x128 s3 t
-        {512, 256, 16, 3.12f, 0.530f, 0.49f, 3.60f, 0.300f, 0.32f, 0.314f, 1.00f},  // 32x32 s2 t
-        {256, 128, 16, 3.15f, 0.479f, 0.57f, 3.42f, 0.000f, 0.51f, 0.000f, 0.00f},  // 32x32 s4 t
-        {512, 256, 16, 2.95f, 0.341f, 0.66f, 5.45f, 0.300f, 0.00f, 0.323f, 0.56f},  // 64x128 s3
+        {512, 0, 0, 2.57f, 0.722f, 0.77f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
+        {256, 256, 16, 3.40f, 0.540f, 0.68f, 5.54f, 0.300f, 4.29f, 0.000f, 0.00f},  // 128x128 s3
+        {256, 0, 0, 4.92f, 0.906f, 0.71f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
+        {256, 0, 0, 4.92f, 0.824f, 0.76f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
+        {256, 256, 16, 8.15f, 1.580f, 0.58f, 0.00f, 0.300f, 8.69f, 0.000f, 0.00f},  // 256x256 s2
+        {256, 256, 16, 6.58f, 1.490f, 0.58f, 2.68f, 0.296f, 5.09f, 0.000f, 0.00f},  // 256x256 s2 a16
+        {256, 0, 0, 4.67f, 1.877f, 0.55f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
+        {512, 128, 16, 1.97f, 0.461f, 0.65f, 4.84f, 0.300f, 0.00f, 0.212f, 0.79f},  // 32x128 s3 n
+        {512, 128, 16, 1.95f, 0.435f, 0.68f, 5.19f, 0.300f, 0.00f, 0.176f, 1.00f},  // 32x128 s3 t
+        {512, 256, 16, 2.98f, 0.681f, 0.72f, 4.19f, 0.300f, 0.68f, 0.194f, 1.00f},  // 32x32 s2 t
+        {256, 128, 16, 3.18f, 0.531f, 0.68f, 3.96f, 0.000f, 0.60f, 0.000f, 0.00f},  // 32x32 s4 t
+        {512, 256, 16, 2.67f, 0.439f, 0.67f, 6.27f, 0.300f, 1.60f, 0.362f, 0.36f},  // 64x128 s3
     },
     {  // 8-bit float
-        {512, 0, 0, 2.06f, 0.617f, 0.67f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
-        {256, 256, 16, 3.54f, 0.415f, 0.71f, 3.74f, 0.300f, 0.95f, 0.000f, 0.00f},  // 128x128 s3
-        {256, 0, 0, 5.00f, 0.659f, 0.82f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
-        {256, 0, 0, 4.82f, 0.662f, 0.80f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
-        {256, 256, 16, 7.77f, 1.244f, 0.63f, 1.61f, 0.267f, 5.93f, 0.000f, 0.00f},  // 256x256 s2
-        {256, 256, 16, 6.67f, 1.222f, 0.66f, 2.81f, 0.263f, 1.55f, 0.000f, 0.00f},  // 256x256 s2 a16
-        {256, 0, 0, 5.36f, 1.029f, 1.00f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
-        {512, 128, 16, 2.31f, 0.327f, 0.66f, 4.06f, 0.300f, 0.21f, 0.145f, 1.00f},  // 32x128 s3 n
-        {512, 128, 16, 2.31f, 0.327f, 0.66f, 4.06f, 0.300f, 0.21f, 0.145f, 1.00f},  // 32x128 s3 t
-        {512, 256, 16, 3.09f, 0.528f, 0.48f, 3.11f, 0.300f, 0.30f, 0.297f, 1.00f},  // 32x32 s2 t
-        {256, 128, 16, 3.24f, 0.455f, 0.50f, 3.04f, 0.000f, 0.43f, 0.000f, 0.00f},  // 32x32 s4 t
-        {512, 256, 16, 3.00f, 0.301f, 0.72f, 4.51f, 0.300f, 0.16f, 0.258f, 0.70f},  // 64x128 s3
+        {512, 0, 0, 2.52f, 0.715f, 0.75f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
+        {256, 256, 16, 3.25f, 0.483f, 0.69f, 4.62f, 0.300f, 1.09f, 0.000f, 0.00f},  // 128x128 s3
+        {256, 0, 0, 4.69f, 0.853f, 0.64f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
+        {256, 0, 0, 4.55f, 0.802f, 0.67f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
+        {256, 256, 16, 7.06f, 1.310f, 0.66f, 0.85f, 0.291f, 6.15f, 0.000f, 0.00f},  // 256x256 s2
+        {256, 256, 16, 6.43f, 1.253f, 0.70f, 1.82f, 0.289f, 3.59f, 0.000f, 0.00f},  // 256x256 s2 a16
+        {256, 0, 0, 6.30f, 0.977f, 1.00f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
+        {512, 128, 16, 1.89f, 0.424f, 0.69f, 5.13f, 0.300f, 0.00f, 0.165f, 1.00f},  // 32x128 s3 n
+        {512, 128, 16, 1.89f, 0.424f, 0.69f, 5.13f, 0.300f, 0.00f, 0.165f, 1.00f},  // 32x128 s3 t
+        {512, 256, 16, 3.18f, 0.668f, 0.70f, 5.09f, 0.000f, 0.40f, 0.223f, 1.00f},  // 32x32 s2 t
+        {256, 128, 16, 3.21f, 0.510f, 0.72f, 4.53f, 0.000f, 0.57f, 0.000f, 0.00f},  // 32x32 s4 t
+        {512, 256, 16, 2.75f, 0.389f, 0.74f, 5.18f, 0.300f, 0.61f, 0.295f, 0.41f},  // 64x128 s3
     },
 };
 static int small_grid_class(const KernelEntry* k) {

@@ -248,14 +248,17 @@ def test_planner_ranks_variants_by_estimated_time():
     # times as wide: the 32x128 kernel (28672 columns: 35.1 us)
     assert pick(R.E4M3, 32, 16384, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s2_splitk"
     assert pick(R.E4M3, 32, 32768, 8192, transB=True) == "e4m3_nt_32x128x128_w1x4_s3_splitk"
-    # grids of at most 256 tiles of 128x128: a (variant, split) pair from the small-grid model.  Measured, us, before -> now:
-    # 64x8192x8192 NT 40.1 -> 26.5 (64-row tiles, K in 4 slices; the vendor library 26.4), 128x8192x8192 NT 47.4 -> 30.5 (vendor
-    # 37.4), 256x4096x4096 NT 41.9 -> 20.2 (vendor 18.8), 512x2048x8192 NN 49.1 -> 31.2 (vendor 47.1)
+    # grids of at most 256 tiles of 128x128: a (variant, split) pair from the small-grid model.  Measured with B streamed from HBM
+    # (taken in turn from copies that fill 400 MiB), us, the former choice -> now: 64x8192x8192 NT 42.0 -> 38.7 (64-row tiles, K in 4
+    # slices; the vendor library 32.2), 128x8192x8192 NT 55.5 -> 41.9 (vendor 47.0), 256x4096x4096 NT 43.5 -> 24.8 (vendor 22.5),
+    # 512x2048x8192 NN 34.7 (vendor 56.1); with one B that the last-level cache holds: 40.1 -> 26.5 (vendor 26.4), 47.4 -> 30.5
+    # (37.4), 41.9 -> 23.6 (18.8)
     p = R.plan(R.make_desc(R.F16, 64, 8192, 8192, transB=True))
     assert (names[p.kernel_id], p.split_k, p.workspace_bytes) == ("f16_nt_64x128x64_w2x2_s3_splitk", 4, 4 * 64 * 8192 * 4)
     p = R.plan(R.make_desc(R.F16, 128, 8192, 8192, transB=True))
     assert (names[p.kernel_id], p.split_k) == ("f16_nt_128x128x64_w2x2_s3_splitk", 4)
-    assert pick(R.F16, 256, 4096, 4096, transB=True) == "f16_nt_64x128x64_w2x2_s3_splitk"
+    p = R.plan(R.make_desc(R.F16, 256, 4096, 4096, transB=True))
+    assert (names[p.kernel_id], p.split_k) == ("f16_nt_128x128x64_w2x2_s3_splitk", 4)
     p = R.plan(R.make_desc(R.F16, 512, 2048, 8192))
     assert names[p.kernel_id] == "f16_nn_128x128x64_w2x2_s3_splitk" and p.split_k == 4
     # ... and a descriptor that forbids splitting gets the best unsplit variant
