@@ -272,53 +272,60 @@ static double estimated_cost(const KernelEntry* k, const frisk_gemm_desc* d, boo
 // best pair of the sweep (more than 1.2x in 24 of 966 cases); the one-size rule used before lost 35-40 % on
 // average on the skinny shapes.
 struct SmallGridModel { int cap, w, kmin; float launch, tk, a, r0, r1, ps, tk2, a2; };
-static const SmallGridModel kSmallGrid[3][12] = {
+static const SmallGridModel kSmallGrid[3][14] = {
     {  // 16-bit
-        {512, 0, 0, 0.53f, 0.784f, 0.77f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
-        {256, 256, 16, 2.10f, 0.545f, 0.76f, 5.70f, 0.300f, 3.26f, 0.000f, 0.00f},  // 128x128 s3
-        {256, 0, 0, 3.54f, 0.882f, 0.76f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
-        {256, 0, 0, 4.08f, 0.829f, 0.75f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
-        {256, 256, 16, 9.22f, 1.460f, 0.54f, 0.00f, 0.300f, 9.07f, 0.000f, 0.00f},  // 256x256 s2
-        {256, 256, 16, 5.66f, 1.306f, 0.66f, 3.18f, 0.300f, 7.33f, 0.000f, 0.00f},  // 256x256 s2 a16
-        {256, 0, 0, 0.59f, 2.078f, 0.52f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
-        {512, 128, 16, 0.42f, 0.455f, 0.73f, 6.44f, 0.300f, 0.00f, 0.189f, 1.00f},  // 32x128 s3 n
-        {512, 128, 16, 0.15f, 0.464f, 0.76f, 6.40f, 0.300f, 0.00f, 0.168f, 1.00f},  // 32x128 s3 t
-        {512, 256, 16, 2.35f, 0.747f, 0.69f, 7.36f, 0.000f, 0.00f, 0.231f, 0.70f},  // 32x32 s2 t
-        {256, 128, 16, 2.87f, 0.578f, 0.66f, 6.52f, 0.000f, 0.06f, 0.000f, 0.00f},  // 32x32 s4 t
-        {512, 256, 16, 1.38f, 0.435f, 0.72f, 7.11f, 0.300f, 2.05f, 0.303f, 0.41f},  // 64x128 s3
+        {512, 0, 0, 0.57f, 0.783f, 0.77f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
+        {256, 256, 16, 2.32f, 0.551f, 0.73f, 5.64f, 0.300f, 4.27f, 0.000f, 0.00f},  // 128x128 s3
+        {256, 0, 0, 3.66f, 0.879f, 0.76f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
+        {256, 0, 0, 4.17f, 0.833f, 0.74f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
+        {256, 256, 16, 9.37f, 1.496f, 0.52f, 0.00f, 0.300f, 8.37f, 0.000f, 0.00f},  // 256x256 s2
+        {256, 256, 16, 5.82f, 1.307f, 0.66f, 2.98f, 0.300f, 8.84f, 0.000f, 0.00f},  // 256x256 s2 a16
+        {256, 0, 0, 0.83f, 2.046f, 0.53f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
+        {512, 128, 16, 0.36f, 0.456f, 0.74f, 6.46f, 0.300f, 0.00f, 0.211f, 0.88f},  // 32x128 s3 n
+        {512, 128, 16, 0.12f, 0.465f, 0.76f, 6.43f, 0.300f, 0.00f, 0.170f, 1.00f},  // 32x128 s3 t
+        {512, 256, 16, 2.40f, 0.744f, 0.68f, 7.68f, 0.000f, 0.00f, 0.222f, 0.72f},  // 32x32 s2 t
+        {256, 128, 16, 2.88f, 0.580f, 0.65f, 6.64f, 0.000f, 0.03f, 0.000f, 0.00f},  // 32x32 s4 t
+        {512, 256, 16, 1.56f, 0.436f, 0.69f, 7.25f, 0.300f, 2.21f, 0.315f, 0.41f},  // 64x128 s3
+        {256, 256, 16, 3.28f, 0.638f, 0.82f, 6.76f, 0.000f, 1.01f, 0.000f, 0.00f},  // 64x32 s3
+        {256, 256, 16, 2.59f, 0.851f, 0.83f, 5.42f, 0.065f, 0.79f, 0.000f, 0.00f},  // 128x64 s3
     },
     {  // int8
-        {512, 0, 0, 2.57f, 0.722f, 0.77f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
-        {256, 256, 16, 3.40f, 0.540f, 0.68f, 5.54f, 0.300f, 4.29f, 0.000f, 0.00f},  // 128x128 s3
-        {256, 0, 0, 4.92f, 0.906f, 0.71f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
-        {256, 0, 0, 4.92f, 0.824f, 0.76f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
-        {256, 256, 16, 8.15f, 1.580f, 0.58f, 0.00f, 0.300f, 8.69f, 0.000f, 0.00f},  // 256x256 s2
-        {256, 256, 16, 6.58f, 1.490f, 0.58f, 2.68f, 0.296f, 5.09f, 0.000f, 0.00f},  // 256x256 s2 a16
-        {256, 0, 0, 4.67f, 1.877f, 0.55f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
-        {512, 128, 16, 1.97f, 0.461f, 0.65f, 4.84f, 0.300f, 0.00f, 0.212f, 0.79f},  // 32x128 s3 n
-        {512, 128, 16, 1.95f, 0.435f, 0.68f, 5.19f, 0.300f, 0.00f, 0.176f, 1.00f},  // 32x128 s3 t
-        {512, 256, 16, 2.98f, 0.681f, 0.72f, 4.19f, 0.300f, 0.68f, 0.194f, 1.00f},  // 32x32 s2 t
-        {256, 128, 16, 3.18f, 0.531f, 0.68f, 3.96f, 0.000f, 0.60f, 0.000f, 0.00f},  // 32x32 s4 t
-        {512, 256, 16, 2.67f, 0.439f, 0.67f, 6.27f, 0.300f, 1.60f, 0.362f, 0.36f},  // 64x128 s3
+        {512, 0, 0, 2.56f, 0.726f, 0.76f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
+        {256, 256, 16, 3.38f, 0.558f, 0.65f, 5.70f, 0.300f, 4.52f, 0.000f, 0.00f},  // 128x128 s3
+        {256, 0, 0, 4.88f, 0.908f, 0.71f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
+        {256, 0, 0, 4.92f, 0.827f, 0.76f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
+        {256, 256, 16, 8.27f, 1.618f, 0.56f, 0.00f, 0.300f, 7.84f, 0.000f, 0.00f},  // 256x256 s2
+        {256, 256, 16, 6.65f, 1.471f, 0.60f, 2.63f, 0.300f, 5.73f, 0.000f, 0.00f},  // 256x256 s2 a16
+        {256, 0, 0, 4.80f, 1.741f, 0.61f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
+        {512, 128, 16, 2.00f, 0.461f, 0.65f, 4.98f, 0.300f, 0.00f, 0.222f, 0.70f},  // 32x128 s3 n
+        {512, 128, 16, 1.96f, 0.436f, 0.69f, 5.27f, 0.300f, 0.00f, 0.188f, 0.88f},  // 32x128 s3 t
+        {512, 256, 16, 3.09f, 0.678f, 0.71f, 4.29f, 0.300f, 0.59f, 0.199f, 1.00f},  // 32x32 s2 t
+        {256, 128, 16, 3.29f, 0.532f, 0.66f, 4.15f, 0.000f, 0.53f, 0.000f, 0.00f},  // 32x32 s4 t
+        {512, 256, 16, 2.72f, 0.443f, 0.65f, 6.47f, 0.300f, 1.56f, 0.377f, 0.36f},  // 64x128 s3
+        {256, 256, 16, 3.47f, 0.646f, 0.87f, 4.48f, 0.300f, 1.19f, 0.000f, 0.00f},  // 64x32 s3
+        {256, 256, 16, 3.04f, 0.844f, 0.83f, 4.14f, 0.300f, 0.89f, 0.000f, 0.00f},  // 128x64 s3
     },
     {  // 8-bit float
-        {512, 0, 0, 2.52f, 0.715f, 0.75f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
-        {256, 256, 16, 3.25f, 0.483f, 0.69f, 4.62f, 0.300f, 1.09f, 0.000f, 0.00f},  // 128x128 s3
-        {256, 0, 0, 4.69f, 0.853f, 0.64f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
-        {256, 0, 0, 4.55f, 0.802f, 0.67f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
-        {256, 256, 16, 7.06f, 1.310f, 0.66f, 0.85f, 0.291f, 6.15f, 0.000f, 0.00f},  // 256x256 s2
-        {256, 256, 16, 6.43f, 1.253f, 0.70f, 1.82f, 0.289f, 3.59f, 0.000f, 0.00f},  // 256x256 s2 a16
-        {256, 0, 0, 6.30f, 0.977f, 1.00f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
-        {512, 128, 16, 1.89f, 0.424f, 0.69f, 5.13f, 0.300f, 0.00f, 0.165f, 1.00f},  // 32x128 s3 n
-        {512, 128, 16, 1.89f, 0.424f, 0.69f, 5.13f, 0.300f, 0.00f, 0.165f, 1.00f},  // 32x128 s3 t
-        {512, 256, 16, 3.18f, 0.668f, 0.70f, 5.09f, 0.000f, 0.40f, 0.223f, 1.00f},  // 32x32 s2 t
-        {256, 128, 16, 3.21f, 0.510f, 0.72f, 4.53f, 0.000f, 0.57f, 0.000f, 0.00f},  // 32x32 s4 t
-        {512, 256, 16, 2.75f, 0.389f, 0.74f, 5.18f, 0.300f, 0.61f, 0.295f, 0.41f},  // 64x128 s3
+        {512, 0, 0, 2.63f, 0.708f, 0.74f, 5.00f, 0.200f, 1.00f, 0.300f, 0.50f},  // 128x128 s2
+        {256, 256, 16, 3.32f, 0.485f, 0.67f, 4.85f, 0.300f, 2.07f, 0.000f, 0.00f},  // 128x128 s3
+        {256, 0, 0, 4.85f, 0.854f, 0.62f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 128x256 s3
+        {256, 0, 0, 4.62f, 0.802f, 0.67f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x128 s3
+        {256, 256, 16, 7.47f, 1.283f, 0.68f, 0.41f, 0.300f, 7.22f, 0.000f, 0.00f},  // 256x256 s2
+        {256, 256, 16, 6.48f, 1.195f, 0.74f, 1.99f, 0.300f, 6.48f, 0.000f, 0.00f},  // 256x256 s2 a16
+        {256, 0, 0, 4.17f, 1.217f, 1.00f, 5.00f, 0.200f, 1.00f, 0.000f, 0.00f},  // 256x256 s2 w8
+        {512, 128, 16, 1.98f, 0.421f, 0.67f, 5.23f, 0.300f, 0.00f, 0.148f, 1.00f},  // 32x128 s3 n
+        {512, 128, 16, 1.98f, 0.421f, 0.67f, 5.23f, 0.300f, 0.00f, 0.148f, 1.00f},  // 32x128 s3 t
+        {512, 256, 16, 2.79f, 0.698f, 0.71f, 4.93f, 0.000f, 0.57f, 0.225f, 1.00f},  // 32x32 s2 t
+        {256, 128, 16, 2.98f, 0.514f, 0.73f, 4.23f, 0.000f, 0.67f, 0.000f, 0.00f},  // 32x32 s4 t
+        {512, 256, 16, 2.79f, 0.386f, 0.74f, 5.38f, 0.300f, 0.88f, 0.302f, 0.44f},  // 64x128 s3
+        {256, 256, 16, 3.53f, 0.630f, 0.89f, 4.81f, 0.291f, 1.23f, 0.000f, 0.00f},  // 64x32 s3
+        {256, 256, 16, 3.26f, 0.649f, 0.80f, 5.42f, 0.095f, 1.14f, 0.000f, 0.00f},  // 128x64 s3
     },
 };
 static int small_grid_class(const KernelEntry* k) {
   if (k->bm == 32) return k->bn == 32 ? (k->stages >= 3 ? 10 : 9) : (k->transB ? 8 : 7);
-  if (k->bm == 64) return 11;
+  if (k->bm == 64) return k->wk > 1 ? 12 : 11;
+  if (k->bm == 128 && k->bn == 64) return 13;
   if ((int64_t)k->bm * k->bn >= 256 * 256) return k->wm * k->wn > 4 ? 6 : (k->atom == 16 ? 5 : 4);
   if (k->bm == 256) return 3;
   if (k->bn == 256) return 2;

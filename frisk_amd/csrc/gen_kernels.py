@@ -51,6 +51,11 @@ def square(bk, atom16=False):
     # vendor library 26.6); with 64-row tiles 26.6, 128x8192x8192 28.6 against 47.4, 256x4096x4096 18.3 against 23.6
     for tb in (0, 1):
         out.append((0, tb, 64, 128, bk, 2, 2, 3, 0, 1, 1))
+    # B stored [N][K] streamed from HBM against 64 and 128 rows (fp16, B rotating over 400 MiB, us): the 32x32 kernel's shape with 64
+    # rows, the 4 waves splitting the K steps, 64x8192x8192 31.6 against 36.2 for 64x128 tiles (the vendor library 34.1); a
+    # 128x64 tile with K tiles twice as deep, 128x16384x4096 35.2 against 39.6 (vendor 36.0), 128x4096x16384 40.5 against 42.8
+    out.append((0, 1, 64, 32, 4 * bk, 1, 1, 3, 0, 1, 4))
+    out.append((0, 1, 128, 64, 2 * bk, 2, 2, 3, 0, 1, 1))
     # guarded variants: any shape, any leading dimension, element-aligned pointers
     for ta in (0, 1):
         for tb in (0, 1):

@@ -439,8 +439,8 @@ def test_skinny_split_k(hip, dtype, transB):
 @pytest.mark.parametrize("transB", [0, 1])
 def test_small_grid_gets_a_split_of_its_own(hip, dtype, transB):
     """a few hundred rows and a long K: the planner's small-grid model picks a variant with the split-K store path and a split of
-    its own; same result as the oracle with the planner's pair, without a workspace (one pass), and with the 128x128 and 64x128
-    variants named by the descriptor at splits 2 and 4"""
+    its own; same result as the oracle with the planner's pair, without a workspace (one pass), and with the small-grid variants
+    (128x128, 64x128, 64x32 with waves splitting K, 128x64) named by the descriptor at several splits"""
     M, N, K = 512, 512, 128 * BK[dtype]
     sa, sb = stored_shapes(M, N, K, 0, transB)
     A = make_operand(dtype, *sa, seed=47, tensor=0, scale=0.5)
@@ -452,6 +452,8 @@ def test_small_grid_gets_a_split_of_its_own(hip, dtype, transB):
     assert p.tile_m in (64, 128) and p.split_k > 1 and name.endswith("_s3_splitk") and p.workspace_bytes == p.split_k * M * N * 4, (name, p.split_k)
     cases = [dict(workspace=True), dict(workspace=False)]
     cases += [dict(tile=(bm, 128, BK[dtype]), split_k=sk) for bm in (64, 128) for sk in (2, 4)]
+    if transB:  # the two variants that stream a B stored [N][K]: 64x32 with the waves splitting K, 128x64 with K tiles twice as deep
+        cases += [dict(tile=(64, 32, 4 * BK[dtype]), split_k=sk) for sk in (1, 2)] + [dict(tile=(128, 64, 2 * BK[dtype]), split_k=sk) for sk in (1, 4)]
     for kw in cases:
         note(f"case small grid {NAMES[dtype]} tB={transB} M={M} N={N} K={K} {kw}")
         got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, **kw)

@@ -249,16 +249,15 @@ def test_planner_ranks_variants_by_estimated_time():
     assert pick(R.E4M3, 32, 16384, 8192, transB=True) == "e4m3_nt_32x32x512_w1x1x4_s2_splitk"
     assert pick(R.E4M3, 32, 32768, 8192, transB=True) == "e4m3_nt_32x128x128_w1x4_s3_splitk"
     # grids of at most 256 tiles of 128x128: a (variant, split) pair from the small-grid model.  Measured with B streamed from HBM
-    # (taken in turn from copies that fill 400 MiB), us, the former choice -> now: 64x8192x8192 NT 42.0 -> 38.7 (64-row tiles, K in 4
-    # slices; the vendor library 32.2), 128x8192x8192 NT 55.5 -> 41.9 (vendor 47.0), 256x4096x4096 NT 43.5 -> 24.8 (vendor 22.5),
-    # 512x2048x8192 NN 34.7 (vendor 56.1); with one B that the last-level cache holds: 40.1 -> 26.5 (vendor 26.4), 47.4 -> 30.5
-    # (37.4), 41.9 -> 23.6 (18.8)
+    # (taken in turn from copies that fill 400 MiB), us, the former choice -> now: 64x8192x8192 NT 42.0 -> 30.7 (64 rows against
+    # 32 columns of B, the 4 waves splitting the K steps; the vendor library 31.7), 128x8192x8192 NT 55.5 -> 41.4 (vendor 46.7),
+    # 256x4096x4096 NT 43.5 -> 22.5 (128x64 tiles with K tiles of 128, 2 slices; vendor 22.4), 512x2048x8192 NN 34.7 (vendor 56.1)
     p = R.plan(R.make_desc(R.F16, 64, 8192, 8192, transB=True))
-    assert (names[p.kernel_id], p.split_k, p.workspace_bytes) == ("f16_nt_64x128x64_w2x2_s3_splitk", 4, 4 * 64 * 8192 * 4)
+    assert (names[p.kernel_id], p.split_k, p.workspace_bytes) == ("f16_nt_64x32x256_w1x1x4_s3_splitk", 1, 0)
     p = R.plan(R.make_desc(R.F16, 128, 8192, 8192, transB=True))
     assert (names[p.kernel_id], p.split_k) == ("f16_nt_128x128x64_w2x2_s3_splitk", 4)
     p = R.plan(R.make_desc(R.F16, 256, 4096, 4096, transB=True))
-    assert (names[p.kernel_id], p.split_k) == ("f16_nt_128x128x64_w2x2_s3_splitk", 4)
+    assert (names[p.kernel_id], p.split_k, p.workspace_bytes) == ("f16_nt_128x64x128_w2x2_s3_splitk", 2, 2 * 256 * 4096 * 4)
     p = R.plan(R.make_desc(R.F16, 512, 2048, 8192))
     assert names[p.kernel_id] == "f16_nn_128x128x64_w2x2_s3_splitk" and p.split_k == 4
     # ... and a descriptor that forbids splitting gets the best unsplit variant
