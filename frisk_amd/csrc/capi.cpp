@@ -322,6 +322,30 @@ static const SmallGridModel kSmallGrid[3][14] = {
         {256, 256, 16, 3.26f, 0.649f, 0.80f, 5.42f, 0.095f, 1.14f, 0.000f, 0.00f},  // 128x64 s3
     },
 };
+// fp32: one 64x64 work-group of four waves already keeps a CU's matrix pipe busy (a 32x32x2 MFMA is 64 cycles), so time follows
+// the work of the busiest CU and idle CUs are lost outright: 256x256x8192 runs 127 us on its 16 tiles and 23 us with K split 16
+// ways.  Fitted to 70 skinny and 50 squarish shapes, both layouts of B, B from HBM.
+static const SmallGridModel kSmallGridF32[11] = {
+    {512, 0, 0, 4.84f, 1.832f, 0.94f, 0.00f, 0.000f, 1.00f, 0.300f, 0.50f},  // 128x128x32 s2
+    {512, 0, 0, 4.95f, 0.944f, 0.91f, 0.00f, 0.000f, 1.00f, 0.300f, 0.50f},  // 128x128x16 s4
+    {512, 0, 0, 2.36f, 0.612f, 0.73f, 0.00f, 0.000f, 0.00f, 0.398f, 0.87f},  // 64x64x32 s2
+    {512, 4096, 8, 3.95f, 0.536f, 0.72f, 5.54f, 0.071f, 1.66f, 0.443f, 0.83f},  // 64x64x32 s3
+    {512, 0, 0, 2.38f, 1.208f, 0.82f, 0.00f, 0.000f, 0.00f, 0.905f, 0.87f},  // 64x64x64 s2
+    {256, 0, 0, 4.18f, 2.138f, 0.87f, 0.00f, 0.000f, 1.27f, 0.000f, 0.00f},  // 64x64x128 s2, 8 waves
+    {512, 512, 8, 3.12f, 0.630f, 0.76f, 4.56f, 0.817f, 0.00f, 0.635f, 0.48f},  // 32x128x32 s3 n
+    {512, 512, 8, 2.58f, 0.639f, 0.72f, 5.36f, 0.534f, 0.36f, 0.594f, 0.53f},  // 32x128x32 s3 t
+    {512, 512, 4, 2.35f, 0.857f, 0.78f, 4.01f, 0.947f, 0.00f, 0.573f, 0.50f},  // 32x32x128 s2 t
+    {256, 256, 4, 3.06f, 0.735f, 0.89f, 3.36f, 1.485f, 1.05f, 0.000f, 0.00f},  // 32x32x128 s4 t
+    {256, 256, 4, 3.32f, 1.127f, 0.98f, 4.25f, 0.048f, 2.24f, 0.000f, 0.00f},  // 64x32x128 s3 t
+};
+static int small_grid_class_f32(const KernelEntry* k) {
+  if (k->bm == 32) return k->bn == 32 ? (k->stages >= 3 ? 9 : 8) : (k->transB ? 7 : 6);
+  if (k->bn == 32) return 10;
+  if (k->bm == 128) return k->bk <= 16 ? 1 : 0;
+  if (k->bk >= 128) return 5;
+  if (k->bk >= 64) return 4;
+  return k->stages >= 3 ? 3 : 2;
+}
 static int small_grid_class(const KernelEntry* k) {
   if (k->bm == 32) return k->bn == 32 ? (k->stages >= 3 ? 10 : 9) : (k->transB ? 8 : 7);
   if (k->bm == 64) return k->wk > 1 ? 12 : 11;
@@ -332,9 +356,10 @@ static int small_grid_class(const KernelEntry* k) {
   return k->stages >= 3 ? 1 : 0;
 }
 static bool small_grid(const frisk_gemm_desc* d) {
-  return d->dtype_ab != FRISK_F32 && d->split_k <= 1 && ((d->M + 127) / 128) * ((d->N + 127) / 128) <= 256;
+  return d->split_k <= 1 && ((d->M + 127) / 128) * ((d->N + 127) / 128) <= 256;
 }
 static const SmallGridModel& small_grid_model(const KernelEntry* k) {
+  if (k->dtype == FRISK_F32) return kSmallGridF32[small_grid_class_f32(k)];
   return kSmallGrid[k->dtype == FRISK_I8 ? 1 : (k->dtype == FRISK_E4M3 ? 2 : 0)][small_grid_class(k)];
 }
 static double small_grid_time(const SmallGridModel& m, const KernelEntry* k, const frisk_gemm_desc* d, int split) {
@@ -360,7 +385,7 @@ static int small_grid_split(const KernelEntry* k, const frisk_gemm_desc* d, bool
   double best_t = small_grid_time(m, k, d, 1);
   if (k->splitk && !no_split && d->split_k != 1 && m.w != 0 && d->K % k->bk == 0) {
     const int64_t tiles = ((d->M + k->bm - 1) / k->bm) * ((d->N + k->bn - 1) / k->bn), kt = d->K / k->bk;
-    for (int c = 2; c <= 64; c *= 2)
+    for (int c = 2; c <= (k->dtype == FRISK_F32 ? 32 : 64); c *= 2)  // the sweeps behind the tables: fp32 up to 32 slices
       if (tiles * c <= m.w && kt % c == 0 && kt / c >= std::max(m.kmin, k->min_k_tiles)) {
         const double t = small_grid_time(m, k, d, c);
         if (t < best_t) { best = c; best_t = t; }

@@ -77,6 +77,13 @@ VARIANTS = {
     "f32": ("FRISK_F32", "F32", [(ta, tb, 128, 128, 16, 2, 2, 4, 0, 0, 1) for ta in (0, 1) for tb in (0, 1)]
             + [(ta, tb, bm, bn, bk, 2, 2, 2, 0, 0, 1) for bm, bn, bk in ((128, 128, 32), (64, 64, 64), (64, 64, 32)) for ta in (0, 1) for tb in (0, 1)]
             + [(ta, tb, 64, 64, 128, 2, 2, 2, 0, 0, 2) for ta in (0, 1) for tb in (0, 1)]
+            # grids that leave CUs idle, or a few rows against a large B streamed from HBM: K split over the idle CUs (one 64x64 work-group of
+            # four waves keeps a CU's matrix pipe busy, so 64 tiles on 256 CUs run at a quarter of the rate).  64x64x32 in a ring of 3
+            # (256x4096x4096, B from HBM: 70 against 82 us for the ring of 2); 32x128x32 for 32 rows; for B stored [N][K] 32x32x128 and
+            # 64x32x128 with the four waves splitting the K tile (512-byte rows of B: 32x16384x4096 47.5 against 61.4 us)
+            + [(ta, tb, 64, 64, 32, 2, 2, 3, 0, 1, 1) for ta in (0, 1) for tb in (0, 1)]
+            + [(0, tb, 32, 128, 32, 1, 4, 3, 0, 1, 1) for tb in (0, 1)]
+            + [(0, 1, 32, 32, 128, 1, 1, 4, 0, 1, 4), (0, 1, 32, 32, 128, 1, 1, 2, 0, 1, 4), (0, 1, 64, 32, 128, 1, 1, 3, 0, 1, 4)]
             + [(ta, tb, 64, 64, 32, 2, 2, 2, 1, 0, 1) for ta in (0, 1) for tb in (0, 1)]),
 }
 

@@ -463,6 +463,40 @@ def test_small_grid_gets_a_split_of_its_own(hip, dtype, transB):
             check(dtype, out_dt, got, ref)
 
 
+@pytest.mark.parametrize("transA,transB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_fp32_small_grids_split_k(hip, transA, transB):
+    """fp32 on grids that leave CUs idle: one 64x64 work-group already keeps a CU's matrix pipe busy, so the planner splits K over
+    the idle CUs (32-row tiles for 32 rows).  The planner's own pair, the same without a workspace (one pass), and every fp32
+    variant with the split-K store path named by the descriptor at several splits, all against the oracle at 1e-4; accumulation
+    into C through the split path"""
+    K = 128 * BK[O.F32]
+    for M, N in ((32, 384), (64, 256), (256, 384)):
+        if transA and M % 64:
+            continue
+        sa, sb = stored_shapes(M, N, K, transA, transB)
+        A = make_operand(O.F32, *sa, seed=53, tensor=0, scale=0.5)
+        B = make_operand(O.F32, *sb, seed=53, tensor=1, scale=0.5)
+        ref = O.gemm_f64(O.F32, A, B, transA, transB)
+        p = hip.plan(hip.make_desc(O.F32, M, N, K, dtype_out=O.F32, transA=bool(transA), transB=bool(transB)))
+        name = hip.kernel_names()[p.kernel_id]
+        assert p.split_k > 1 and name.endswith("_splitk") and p.tile_m <= M and p.workspace_bytes == p.split_k * M * N * 4, (name, p.split_k)
+        cases = [dict(workspace=True), dict(workspace=False)]
+        if M % 64 == 0:
+            cases += [dict(tile=(64, 64, 32), stages=3, split_k=sk) for sk in (2, 4, 16)]
+        if not transA:
+            cases += [dict(tile=(32, 128, 32), split_k=sk) for sk in (1, 2, 8)]
+            if transB:  # B stored [N][K]: the four waves split the K tile
+                cases += [dict(tile=(32, 32, 128), stages=st, split_k=sk) for st in (2, 4) for sk in (1, 2, 4)]
+                if M % 64 == 0:
+                    cases += [dict(tile=(64, 32, 128), split_k=sk) for sk in (1, 4)]
+        for kw in cases:
+            note(f"case fp32 small grid tA={transA} tB={transB} M={M} N={N} K={K} {kw}")
+            check(O.F32, O.F32, run_gemm(hip, O.F32, A, B, transA, transB, O.F32, M, N, K, **kw), ref)
+        C0 = O.uniform(M * N, 53, 2, -1.0, 1.0).reshape(M, N).astype(np.float32)
+        note(f"case fp32 small grid accumulate tA={transA} tB={transB} M={M} N={N}")
+        check(O.F32, O.F32, run_gemm(hip, O.F32, A, B, transA, transB, O.F32, M, N, K, C_init=C0, clear_accum=False), ref + C0)
+
+
 def test_split_k_epilogues_and_accumulate(hip):
     M, N, K = 32, 256, 2048
     A = make_operand(O.I8, M, K, seed=42, tensor=0)
@@ -494,11 +528,13 @@ def test_split_k_status_codes(hip):
     with pytest.raises(hip.FriskHipError) as e:
         hip.gemm(d, buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), None, None, None, 0, None)
     assert e.value.status == hip.ERR_WORKSPACE
-    # no fp32 kernel has the split path: an explicit split is refused
-    d = hip.make_desc(O.F32, 256, 256, 2048, split_k=4)
+    # a tile named by the descriptor whose variants have no split path: an explicit split is refused
+    d = hip.make_desc(O.F32, 256, 256, 2048, tile=(128, 128, 32), split_k=4)
     with pytest.raises(hip.FriskHipError) as e:
         hip.plan(d)
     assert e.value.status == hip.ERR_TILE
+    p = hip.plan(hip.make_desc(O.F32, 256, 256, 2048, split_k=4))
+    assert p.split_k == 4 and hip.kernel_names()[p.kernel_id].endswith("_splitk")
     # an explicit split looks for a variant that can split: the 256 x 256 tile has one in every layout
     p = hip.plan(hip.make_desc(O.F16, 256, 256, 2048, transA=True, split_k=4))
     assert p.split_k == 4 and hip.kernel_names()[p.kernel_id].endswith("_splitk")

@@ -276,6 +276,17 @@ def test_planner_ranks_variants_by_estimated_time():
     # 256 tiles of 256x128 unsplit 243); 1024x8192x8192 comes out even (123.7 against 123.9 us) and stays unsplit
     p = R.plan(R.make_desc(R.F16, 2048, 4096, 16384))
     assert (names[p.kernel_id], p.split_k) == ("f16_nn_256x256x64_w2x2_s2x3_a16_splitk", 2)
+    # fp32: a 64x64 work-group keeps a CU's matrix pipe busy, so grids that leave CUs idle get K split over them (B from HBM, us,
+    # before -> now | the vendor library): 32x4096x4096 241 (the guarded kernel) -> 21.6 | 26.1, 64x4096x4096 NT 83.8 -> 26.4 | 24.9,
+    # 256x256x8192 135 -> 22.9 | 27.5, 32x16384x4096 NT (512-byte rows of B, the 4 waves splitting the K tile) 92 -> 47.5 | 51.8,
+    # 256x4096x4096 (256 tiles, a ring of 3) 82 -> 70 | 69
+    for (M, N, K, tB), want in (((32, 4096, 4096, 0), ("f32_nn_32x128x32_w1x4_s3_splitk", 8)), ((32, 16384, 4096, 1), ("f32_nt_32x32x128_w1x1x4_s2_splitk", 1)),
+                                ((64, 4096, 4096, 1), ("f32_nt_64x64x32_w2x2_s3_splitk", 4)), ((256, 256, 8192, 0), ("f32_nn_64x64x32_w2x2_s3_splitk", 16)),
+                                ((256, 4096, 4096, 0), ("f32_nn_64x64x32_w2x2_s3_splitk", 1)), ((2048, 2048, 2048, 0), ("f32_nn_128x128x32_w2x2_s2", 1))):
+        p = R.plan(R.make_desc(R.F32, M, N, K, dtype_out=R.F32, transB=bool(tB)))
+        assert (names[p.kernel_id], p.split_k) == want and p.workspace_bytes == (p.split_k * M * N * 4 if p.split_k > 1 else 0), (M, N, K, names[p.kernel_id], p.split_k)
+    p = R.plan(R.make_desc(R.F32, 256, 256, 8192, dtype_out=R.F32, split_k=1))
+    assert p.split_k == 1 and p.workspace_bytes == 0
     # whole rounds, more than half a round left over, or a descriptor that forbids splitting: no tail
     for shape, kw in (((8192, 8192, 8192), {}), ((5120, 5120, 5120), {}), ((6144, 6144, 6144), {"split_k": 1})):
         p = R.plan(R.make_desc(R.F16, *shape, **kw))
@@ -346,7 +357,7 @@ def test_tiles_whose_rows_span_4_gib_are_not_given_to_the_fast_kernels():
 def test_planner_choices_for_the_benchmark_shapes_are_pinned():
     """the kernels bench.py times: a change of the cost table that moves one of them must show here"""
     want = [
-        ((R.F32, 1024, 1024, 1024, 0, R.F32, R.EPI_NONE), "f32_nn_64x64x32_w2x2_s2"),
+        ((R.F32, 1024, 1024, 1024, 0, R.F32, R.EPI_NONE), "f32_nn_64x64x32_w2x2_s3_splitk"),
         ((R.F16, 4096, 4096, 4096, 0, R.F16, R.EPI_NONE), "f16_nn_256x256x64_w2x2_s2x3_a16"),
         ((R.F16, 4096, 4096, 4096, 1, R.F16, R.EPI_NONE), "f16_nt_256x256x64_w2x2_s2x3_a16"),
         ((R.BF16, 8192, 8192, 8192, 1, R.BF16, R.EPI_NONE), "bf16_nt_256x256x64_w2x2_s2x3_a16"),
