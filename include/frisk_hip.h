@@ -163,7 +163,8 @@ int frisk_hip_gemm(const frisk_gemm_desc* desc, const void* A, const void* B, vo
  * harnesses that forbid hipMalloc) and therefore have no workspace to pass.  No counterpart in the reference.  The
  * partial sums of a split-K or tail-split plan go to a fixed array of FRISK_HIP_STATIC_WS_BYTES that lives in the
  * library's device image (one copy per GPU, held until the process ends); neither this call nor anything it calls
- * allocates or frees.  Same planner, kernels and results as frisk_hip_gemm with a large enough workspace, with two
+ * allocates or frees.  (The HIP runtime places a device image on a GPU when it is first used there, which takes device
+ * memory once: call frisk_hip_init() on each GPU beforehand and that has happened before the first launch.)  Same planner, kernels and results as frisk_hip_gemm with a large enough workspace, with two
  * exceptions for plans that need more than the array holds: an explicit split_k > 1 in the descriptor is refused with
  * FRISK_ERR_WORKSPACE, and a split the planner chose itself (split_k = 0: the tail split of a large grid can want
  * 64 MiB) is dropped, the launch running as a single pass exactly as frisk_hip_gemm does without a workspace.  All calls on one GPU share the array: calls that may overlap on that GPU (different streams,

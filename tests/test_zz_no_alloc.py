@@ -37,6 +37,7 @@ def _static(hip, dtype, A, B, transB, dtype_out, M, N, K, split_k=0, epilogue=0,
 
 
 def test_static_workspace_matches_caller_workspace_on_two_calls_in_a_row(hip):
+    hip.init()  # the set-up call: places the library's device image (the array is part of it) on the GPU, once
     assert hip.static_workspace_bytes() == 32 << 20
     # first call: int8 64 x 2048 x 8192 NN, the planner splits K (skinny problem); dequantising epilogue
     # second call: a smaller problem of the same kind, then an fp16 one with an explicit split on the 256 x 256 tile
@@ -59,6 +60,7 @@ def test_static_workspace_matches_caller_workspace_on_two_calls_in_a_row(hip):
 
 
 def test_static_workspace_tail_split_and_unsplit_plans(hip):
+    hip.init()
     # a tail split that fits the array: 4352 x 4096 x 4096 fp16 NT has 272 tiles, the last 16 split 8 ways = 32 MiB
     M, N, K = 4352, 4096, 4096
     d = hip.make_desc(O.F16, M, N, K, transB=True)
