@@ -23,7 +23,7 @@ template <bool INT_ACC> __global__ void __launch_bounds__(256) splitk_reduce_ker
   const char* src = (const char*)p.partial + ((size_t)m * p.N + n) * 4;
   if (whole) {
     // the slices' quads are fetched eight at a time and then added in slice order: one memory latency per eight slices instead
-    // of one per slice (16 slices of a 256 x 256 result: 9.9 -> 3 us), the same sum
+    // of one per slice (16 slices of a 256 x 256 result: 9.9 -> 4.4 us in a kernel trace), the same sum
     for (int z0 = 0; z0 < p.split_k; z0 += 8) {
       r_v4i t[8];
 #pragma unroll
