@@ -12,7 +12,7 @@ import os
 # atom16: the default 256x256 variant (and its split-K copy) exists once more built from 16x16 atoms of twice the K depth: the
 # part holds a higher clock on them (fp16 4096^3 NT 100 against 112 us, NN 104 against 108; int8 gains nothing).  Listed first;
 # the planner prefers the 32x32 atoms where the clock is not the limit (grids below one round with a transpose-read operand)
-def square(bk, atom16=False):
+def square(bk, atom16=False, skinny_ta=(0,)):
     out = []
     # The first variant of a tile size is the planner's default.  256x256: 4 waves of 128x128 (fewest LDS reads per MFMA)
     # with 2 LDS tiles of A and 3 of B (160 KiB), B fetched two tiles ahead and spread over the K tile; then the same
@@ -45,12 +45,16 @@ def square(bk, atom16=False):
     # the same with a ring of 2 tiles (64 KiB): two work-groups share a CU, for grids of more than 256 tiles, where the
     # start of one work-group then overlaps the steady state of another
     out.append((0, 1, 32, 32, 4 * bk, 1, 1, 2, 0, 1, 4))
-    for tb in (0, 1):
-        out.append((0, tb, 32, 128, bk, 1, 4, 3, 0, 1, 1))
+    # (16-bit types: A stored [K][M] too, or a 32- or 64-row problem with A transposed falls to the guarded kernel, 10x slower; the
+    # 8-bit types' transposed rows of 32 and 64 bytes are shorter than their LDS swizzle needs)
+    for ta in skinny_ta:
+        for tb in (0, 1):
+            out.append((ta, tb, 32, 128, bk, 1, 4, 3, 0, 1, 1))
     # 64 rows: from M = 64 to a few hundred rows a 32-row tile streams B once per 32 rows of A (fp16 64x8192x8192 NT 34.2 us, the
     # vendor library 26.6); with 64-row tiles 26.6, 128x8192x8192 28.6 against 47.4, 256x4096x4096 18.3 against 23.6
-    for tb in (0, 1):
-        out.append((0, tb, 64, 128, bk, 2, 2, 3, 0, 1, 1))
+    for ta in skinny_ta:
+        for tb in (0, 1):
+            out.append((ta, tb, 64, 128, bk, 2, 2, 3, 0, 1, 1))
     # B stored [N][K] streamed from HBM against 64 and 128 rows (fp16, B rotating over 400 MiB, us): the 32x32 kernel's shape with 64
     # rows, the 4 waves splitting the K steps, 64x8192x8192 31.6 against 36.2 for 64x128 tiles (the vendor library 34.1); a
     # 128x64 tile with K tiles twice as deep, 128x16384x4096 35.2 against 39.6 (vendor 36.0), 128x4096x16384 40.5 against 42.8
@@ -63,8 +67,8 @@ def square(bk, atom16=False):
     return out
 
 VARIANTS = {
-    "f16": ("FRISK_F16", "F16", square(64, atom16=True)),
-    "bf16": ("FRISK_BF16", "BF16", square(64, atom16=True)),
+    "f16": ("FRISK_F16", "F16", square(64, atom16=True, skinny_ta=(0, 1))),
+    "bf16": ("FRISK_BF16", "BF16", square(64, atom16=True, skinny_ta=(0, 1))),
     "i8": ("FRISK_I8", "I8", square(128, atom16=True)),
     # 8-bit floats: the 256x256 NT variant once more on the 16x16x128 atom, whose K is the whole K tile (listed first: the planner's
     # choice for B stored [N][K] from four K tiles on), and its copy with the split-K store path
@@ -82,7 +86,7 @@ VARIANTS = {
             # (256x4096x4096, B from HBM: 70 against 82 us for the ring of 2); 32x128x32 for 32 rows; for B stored [N][K] 32x32x128 and
             # 64x32x128 with the four waves splitting the K tile (512-byte rows of B: 32x16384x4096 47.5 against 61.4 us)
             + [(ta, tb, 64, 64, 32, 2, 2, 3, 0, 1, 1) for ta in (0, 1) for tb in (0, 1)]
-            + [(0, tb, 32, 128, 32, 1, 4, 3, 0, 1, 1) for tb in (0, 1)]
+            + [(ta, tb, 32, 128, 32, 1, 4, 3, 0, 1, 1) for ta in (0, 1) for tb in (0, 1)]
             + [(0, 1, 32, 32, 128, 1, 1, 4, 0, 1, 4), (0, 1, 32, 32, 128, 1, 1, 2, 0, 1, 4), (0, 1, 64, 32, 128, 1, 1, 3, 0, 1, 4)]
             + [(ta, tb, 64, 64, 32, 2, 2, 2, 1, 0, 1) for ta in (0, 1) for tb in (0, 1)]),
 }

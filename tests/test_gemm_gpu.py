@@ -403,32 +403,32 @@ def test_empty_problems(hip):
 
 
 # ------------------------------------------------------------------ skinny problems: 32-row tiles, K split over work-groups
-@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.I8, O.E4M3])
+@pytest.mark.parametrize("dtype,transA", [(O.F16, 0), (O.BF16, 0), (O.I8, 0), (O.E4M3, 0), (O.F16, 1), (O.BF16, 1)])
 @pytest.mark.parametrize("transB", [0, 1])
-def test_skinny_split_k(hip, dtype, transB):
+def test_skinny_split_k(hip, dtype, transA, transB):
     """M = 32 and 64: a 32- or 64-row kernel runs (32 rows, B stored [N][K]: 32x32 tile whose 4 waves split the K steps; B stored
     [K][N]: 32x128 tile; 64 rows: 64x128); every split factor gives the oracle's result (int8: the same bits).  K is deep enough for the planner to
-    split it by itself (slices of at least 16 K tiles)"""
+    split it by itself (slices of at least 16 K tiles).  The 16-bit types have the 32x128 and 64x128 tiles for A stored [K][M] too."""
     for M in (32, 64):
         N, K = 384, 128 * BK[dtype]
-        sa, sb = stored_shapes(M, N, K, 0, transB)
+        sa, sb = stored_shapes(M, N, K, transA, transB)
         A = make_operand(dtype, *sa, seed=41, tensor=0, scale=0.5)
         B = make_operand(dtype, *sb, seed=41, tensor=1, scale=0.5)
         out_dt = DEFAULT_OUT[dtype]
-        ref = O.gemm_i32(A, B, 0, transB) if dtype == O.I8 else O.gemm_f64(dtype, A, B, 0, transB)
-        d = hip.make_desc(dtype, M, N, K, dtype_out=out_dt, transB=bool(transB))
+        ref = O.gemm_i32(A, B, transA, transB) if dtype == O.I8 else O.gemm_f64(dtype, A, B, transA, transB)
+        d = hip.make_desc(dtype, M, N, K, dtype_out=out_dt, transA=bool(transA), transB=bool(transB))
         p = hip.plan(d)
         assert p.tile_m in (32, 64) and p.tile_m <= M and p.split_k > 1 and p.workspace_bytes == p.split_k * M * N * 4, (p.tile_m, p.split_k, p.workspace_bytes)
         # the planner's variant at every split, then the 32-row kernels by name (at M = 64 the planner prefers 64-row tiles)
         for split, rows in ((0, 0), (1, 0), (2, 0), (4, 0), (8, 0), (0, 32), (2, 32)):
-            note(f"case skinny {NAMES[dtype]} tB={transB} M={M} N={N} K={K} split_k={split} tile_m={rows}")
-            got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, split_k=split, tile=(rows, 0, 0))
+            note(f"case skinny {NAMES[dtype]} tA={transA} tB={transB} M={M} N={N} K={K} split_k={split} tile_m={rows}")
+            got = run_gemm(hip, dtype, A, B, transA, transB, out_dt, M, N, K, split_k=split, tile=(rows, 0, 0))
             if dtype == O.I8:
                 assert np.array_equal(got, ref)
             else:
                 check(dtype, out_dt, got, ref)
         # the planner's own split needs no workspace to be correct: without one the launch runs unsplit
-        got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, workspace=False)
+        got = run_gemm(hip, dtype, A, B, transA, transB, out_dt, M, N, K, workspace=False)
         if dtype == O.I8:
             assert np.array_equal(got, ref)
         else:
@@ -471,8 +471,6 @@ def test_fp32_small_grids_split_k(hip, transA, transB):
     into C through the split path"""
     K = 128 * BK[O.F32]
     for M, N in ((32, 384), (64, 256), (256, 384)):
-        if transA and M % 64:
-            continue
         sa, sb = stored_shapes(M, N, K, transA, transB)
         A = make_operand(O.F32, *sa, seed=53, tensor=0, scale=0.5)
         B = make_operand(O.F32, *sb, seed=53, tensor=1, scale=0.5)
@@ -483,12 +481,11 @@ def test_fp32_small_grids_split_k(hip, transA, transB):
         cases = [dict(workspace=True), dict(workspace=False)]
         if M % 64 == 0:
             cases += [dict(tile=(64, 64, 32), stages=3, split_k=sk) for sk in (2, 4, 16)]
-        if not transA:
-            cases += [dict(tile=(32, 128, 32), split_k=sk) for sk in (1, 2, 8)]
-            if transB:  # B stored [N][K]: the four waves split the K tile
-                cases += [dict(tile=(32, 32, 128), stages=st, split_k=sk) for st in (2, 4) for sk in (1, 2, 4)]
-                if M % 64 == 0:
-                    cases += [dict(tile=(64, 32, 128), split_k=sk) for sk in (1, 4)]
+        cases += [dict(tile=(32, 128, 32), split_k=sk) for sk in (1, 2, 8)]
+        if not transA and transB:  # A stored [M][K], B stored [N][K]: the four waves split the K tile
+            cases += [dict(tile=(32, 32, 128), stages=st, split_k=sk) for st in (2, 4) for sk in (1, 2, 4)]
+            if M % 64 == 0:
+                cases += [dict(tile=(64, 32, 128), split_k=sk) for sk in (1, 4)]
         for kw in cases:
             note(f"case fp32 small grid tA={transA} tB={transB} M={M} N={N} K={K} {kw}")
             check(O.F32, O.F32, run_gemm(hip, O.F32, A, B, transA, transB, O.F32, M, N, K, **kw), ref)

@@ -287,6 +287,13 @@ def test_planner_ranks_variants_by_estimated_time():
         assert (names[p.kernel_id], p.split_k) == want and p.workspace_bytes == (p.split_k * M * N * 4 if p.split_k > 1 else 0), (M, N, K, names[p.kernel_id], p.split_k)
     p = R.plan(R.make_desc(R.F32, 256, 256, 8192, dtype_out=R.F32, split_k=1))
     assert p.split_k == 1 and p.workspace_bytes == 0
+    # A stored [K][M]: fp32 and the 16-bit types have the 32- and 64-row tiles for it too (fp32 32x4096x4096: 249 us on the guarded
+    # kernel before, 23.9 now, the vendor library 26.3); the 8-bit types do not (their transposed rows are shorter than the LDS
+    # swizzle needs) and take the guarded kernel there
+    for dt, (M, N, K, tB), want in ((R.F32, (32, 4096, 4096, 0), "f32_tn_32x128x32_w1x4_s3_splitk"), (R.F16, (32, 8192, 8192, 0), "f16_tn_32x128x64_w1x4_s3_splitk"),
+                                    (R.F16, (64, 8192, 8192, 1), "f16_tt_64x128x64_w2x2_s3_splitk"), (R.BF16, (96, 4096, 4096, 0), "bf16_tn_32x128x64_w1x4_s3_splitk")):
+        assert pick(dt, M, N, K, transA=True, transB=bool(tB)) == want
+    assert pick(R.I8, 32, 4096, 4096, transA=True).endswith("_guard")
     # whole rounds, more than half a round left over, or a descriptor that forbids splitting: no tail
     for shape, kw in (((8192, 8192, 8192), {}), ((5120, 5120, 5120), {}), ((6144, 6144, 6144), {"split_k": 1})):
         p = R.plan(R.make_desc(R.F16, *shape, **kw))
