@@ -442,8 +442,10 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
       if (want_split && !k->splitk) continue;
       // a kernel whose loop needs a minimum of K tiles: per slice when the descriptor asks for a split
       if (k->min_k_tiles > 1 && (d->K + k->bk - 1) / k->bk / (want_split && d->split_k > 1 ? d->split_k : 1) < k->min_k_tiles) continue;
-      // the fast kernels need whole tiles and rows that start on 16-byte boundaries; the guarded ones take anything
-      if (!k->guard && (force_guard || !rows_aligned || d->M % k->bm || d->N % k->bn || d->K % k->bk)) continue;
+      // the fast kernels need whole tiles and rows that start on 16-byte boundaries; their edge variants take any M and N (and
+      // are left out where the plain twin fits); the guarded ones take anything
+      const bool whole_mn = d->M % k->bm == 0 && d->N % k->bn == 0;
+      if (!k->guard && (force_guard || !rows_aligned || d->K % k->bk || (k->edge ? whole_mn : !whole_mn))) continue;
       // ... and address a tile's chunks by 32-bit lane offsets from its first row: the stored rows of one tile must span
       // less than 4 GiB
       const double span_a = (double)d->lda * es * (d->transA ? k->bk : k->bm), span_b = (double)d->ldb * es * (d->transB ? k->bn : k->bk);

@@ -60,6 +60,7 @@ struct KernelEntry {
   int guard;  // 1: handles any shape / leading dimension (slower staging)
   int splitk;  // 1: compiled with the split-K store path
   int atom;  // rows and columns of the MFMA atom: 32 (32x32xK) or 16 (16x16x2K)
+  int edge;  // 1: M and N need not be multiples of the tile (K, and the alignment of rows and pointers, as for the plain kernels)
   int lds_bytes;
   int min_k_tiles;  // fewest K tiles the kernel's loop is written for
   hipError_t (*launch)(const GemmParams&, hipStream_t);

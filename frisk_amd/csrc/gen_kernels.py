@@ -8,6 +8,22 @@ committed so a build needs only hipcc.
 """
 import os
 
+def full(v):
+    """(…, WK) -> (…, WK, stages of B, atom, edge): B has as many stages as A, the atom is 32x32 and the kernel wants whole tiles
+    unless the variant says otherwise"""
+    v = tuple(v)
+    if len(v) == 11:
+        v += (v[7],)
+    if len(v) == 12:
+        v += (32,)
+    return v if len(v) == 14 else v + (0,)
+
+
+def edge(v):
+    """the variant once more for M and N that are not multiples of the tile"""
+    return full(v)[:13] + (1,)
+
+
 # a variant: (transA, transB, BM, BN, BK, WM, WN, stages of A, guard, split-K, WK, stages of B[, MFMA atom])
 # atom16: the default 256x256 variant (and its split-K copy) exists once more built from 16x16 atoms of twice the K depth: the
 # part holds a higher clock on them (fp16 4096^3 NT 100 against 112 us, NN 104 against 108; int8 gains nothing).  Listed first;
@@ -60,6 +76,13 @@ def square(bk, atom16=False, skinny_ta=(0,)):
     # 128x64 tile with K tiles twice as deep, 128x16384x4096 35.2 against 39.6 (vendor 36.0), 128x4096x16384 40.5 against 42.8
     out.append((0, 1, 64, 32, 4 * bk, 1, 1, 3, 0, 1, 4))
     out.append((0, 1, 128, 64, 2 * bk, 2, 2, 3, 0, 1, 1))
+    # M and N that are not multiples of the tile (K a multiple of the K tile, rows and pointers on 16-byte boundaries): the default
+    # 256x256 variant and the 128x128 one with 2 + 2 tiles once more with clamped lane offsets and checked stores.  (fp16
+    # 4000x4096x4096 ran 539 us on 32-row tiles and 4096x4000x4096 933 us on the guarded kernel, the vendor library 110 and 125.)
+    for ta in (0, 1):
+        for tb in (0, 1):
+            out.append(edge((ta, tb, 256, 256, bk, 2, 2, 2, 0, 0, 1, 3) + ((16,) if atom16 else ())))
+            out.append(edge((ta, tb, 128, 128, bk, 2, 2, 2, 0, 0, 1, 2)))
     # guarded variants: any shape, any leading dimension, element-aligned pointers
     for ta in (0, 1):
         for tb in (0, 1):
@@ -88,20 +111,13 @@ VARIANTS = {
             + [(ta, tb, 64, 64, 32, 2, 2, 3, 0, 1, 1) for ta in (0, 1) for tb in (0, 1)]
             + [(ta, tb, 32, 128, 32, 1, 4, 3, 0, 1, 1) for ta in (0, 1) for tb in (0, 1)]
             + [(0, 1, 32, 32, 128, 1, 1, 4, 0, 1, 4), (0, 1, 32, 32, 128, 1, 1, 2, 0, 1, 4), (0, 1, 64, 32, 128, 1, 1, 3, 0, 1, 4)]
+            + [edge((ta, tb, bm, bm, 32, 2, 2, 2, 0, 0, 1)) for bm in (128, 64) for ta in (0, 1) for tb in (0, 1)]
             + [(ta, tb, 64, 64, 32, 2, 2, 2, 1, 0, 1) for ta in (0, 1) for tb in (0, 1)]),
 }
 
-def full(v):
-    """(…, WK) -> (…, WK, stages of B, atom): B has as many stages as A and the atom is 32x32 unless the variant says otherwise"""
-    v = tuple(v)
-    if len(v) == 11:
-        v += (v[7],)
-    return v if len(v) == 13 else v + (32,)
-
-
 def cfg_of(enum, v):
-    ta, tb, bm, bn, bk, wm, wn, st, gd, sk, wk, sb, at = full(v)
-    return f"GemmCfg<{enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {'true' if gd else 'false'}, {'true' if sk else 'false'}, {wk}, {sb}" + (f", {at}>" if at != 32 else ">")
+    ta, tb, bm, bn, bk, wm, wn, st, gd, sk, wk, sb, at, eg = full(v)
+    return f"GemmCfg<{enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {'true' if gd else 'false'}, {'true' if sk else 'false'}, {wk}, {sb}" + (f", {at}, true>" if eg else (f", {at}>" if at != 32 else ">"))
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 for tag, (enum, suffix, variants) in VARIANTS.items():
@@ -112,11 +128,11 @@ for tag, (enum, suffix, variants) in VARIANTS.items():
     lines.append("#ifndef __HIP_DEVICE_COMPILE__")
     lines.append(f"const KernelEntry kKernels{suffix}[] = {{")
     for v in variants:
-        ta, tb, bm, bn, bk, wm, wn, st, gd, sk, wk, sb, at = full(v)
+        ta, tb, bm, bn, bk, wm, wn, st, gd, sk, wk, sb, at, eg = full(v)
         cfg = cfg_of(enum, v)
         waves = f"w{wm}x{wn}" + (f"x{wk}" if wk > 1 else "")
-        name = f"{tag}_{'t' if ta else 'n'}{'t' if tb else 'n'}_{bm}x{bn}x{bk}_{waves}_s{st}" + (f"x{sb}" if sb != st else "") + (f"_a{at}" if at != 32 else "") + ("_guard" if gd else "") + ("_splitk" if sk else "")
-        lines.append(f'    {{"{name}", {enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {sb}, {wk}, {gd}, {sk}, {at}, {cfg}::LDS_BYTES, {cfg}::MIN_K_TILES, &launch_gemm<{cfg}>, &prepare_gemm<{cfg}>}},')
+        name = f"{tag}_{'t' if ta else 'n'}{'t' if tb else 'n'}_{bm}x{bn}x{bk}_{waves}_s{st}" + (f"x{sb}" if sb != st else "") + (f"_a{at}" if at != 32 else "") + ("_guard" if gd else "") + ("_splitk" if sk else "") + ("_edge" if eg else "")
+        lines.append(f'    {{"{name}", {enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {sb}, {wk}, {gd}, {sk}, {at}, {eg}, {cfg}::LDS_BYTES, {cfg}::MIN_K_TILES, &launch_gemm<{cfg}>, &prepare_gemm<{cfg}>}},')
     lines.append("};")
     lines.append(f"const int kNumKernels{suffix} = sizeof(kKernels{suffix}) / sizeof(kKernels{suffix}[0]);")
     lines.append("#endif")

@@ -32,15 +32,15 @@ def from_dev(t, np_dtype, shape):
 
 
 def run_gemm(R, dtype, A, B, transA, transB, dtype_out, M, N, K, epilogue=0, sA=None, sB=None, C_init=None,
-             clear_accum=True, tile=(0, 0, 0), waves=(0, 0), pad=0, shift=0, split_k=0, workspace=True, stages=0, atom=0):
+             clear_accum=True, tile=(0, 0, 0), waves=(0, 0), pad=0, shift=0, split_k=0, workspace=True, stages=0, atom=0, pad_c=None):
     """launch through the C ABI; returns the output as a numpy array in storage type.
-    pad: extra elements at the end of every stored row of A, B and C (odd leading dimensions);
+    pad: extra elements at the end of every stored row of A, B and C (odd leading dimensions); pad_c: the same for C alone;
     shift: the operands start `shift` elements into their allocations (pointers only element-aligned);
     split_k: descriptor field (0 = planner's choice); workspace=False launches without one."""
     import torch
     out_np = O.NP_STORAGE[dtype_out]
 
-    def padded(x):
+    def padded(x, pad=pad):
         if pad == 0 and shift == 0:
             return np.ascontiguousarray(x), x.shape[1]
         buf = np.zeros(shift + x.shape[0] * (x.shape[1] + pad), dtype=x.dtype)
@@ -50,7 +50,7 @@ def run_gemm(R, dtype, A, B, transA, transB, dtype_out, M, N, K, epilogue=0, sA=
     hA, lda = padded(A)
     hB, ldb = padded(B)
     C0 = C_init if C_init is not None else np.full((M, N), 0xFF, dtype=np.uint8).repeat(np.dtype(out_np).itemsize, axis=1).view(out_np)
-    hC, ldc = padded(np.ascontiguousarray(C0).view(out_np).reshape(M, N))
+    hC, ldc = padded(np.ascontiguousarray(C0).view(out_np).reshape(M, N), pad if pad_c is None else pad_c)
     dA, dB, dC = to_dev(hA), to_dev(hB), to_dev(hC)
     es, osz = hA.dtype.itemsize, np.dtype(out_np).itemsize
     dsA = to_dev(np.asarray(sA, dtype=np.float32)) if sA is not None else None
@@ -68,7 +68,7 @@ def run_gemm(R, dtype, A, B, transA, transB, dtype_out, M, N, K, epilogue=0, sA=
     if M == 0 or N == 0:
         return np.zeros((M, N), dtype=out_np)
     got = full[shift:].reshape(M, ldc)
-    if pad:
+    if ldc > N:
         assert np.all(got[:, N:] == 0), "the kernel wrote into the padding of C"
     return np.ascontiguousarray(got[:, :N])
 

@@ -494,6 +494,62 @@ def test_fp32_small_grids_split_k(hip, transA, transB):
         check(O.F32, O.F32, run_gemm(hip, O.F32, A, B, transA, transB, O.F32, M, N, K, C_init=C0, clear_accum=False), ref + C0)
 
 
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.I8, O.E4M3, O.F32])
+@pytest.mark.parametrize("transA,transB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_edge_kernels_take_any_m_and_n(hip, dtype, transA, transB):
+    """M and N that are not multiples of any tile, K a multiple of the K tile, rows on 16-byte boundaries: the edge variants of the
+    256x256 and 128x128 kernels (fp32: 128x128 and 64x64) run, whose lanes fetch the last valid row or chunk instead of one beyond
+    the operand and whose stores are checked against M and N.  Planner's choice and both tiles by name, against the oracle; the
+    rows and columns of C beyond M and N (inside padded rows) stay untouched."""
+    M, N, K = 304, 400, 3 * BK[dtype]  # 304 = 2 * 128 + 48 = 256 + 48, 400 = 3 * 128 + 16 = 256 + 144; all rows multiples of 16 bytes
+    sa, sb = stored_shapes(M, N, K, transA, transB)
+    A = make_operand(dtype, *sa, seed=61, tensor=0, scale=0.5)
+    B = make_operand(dtype, *sb, seed=61, tensor=1, scale=0.5)
+    out_dt = DEFAULT_OUT[dtype]
+    ref = O.gemm_i32(A, B, transA, transB) if dtype == O.I8 else O.gemm_f64(dtype, A, B, transA, transB)
+    name = hip.kernel_names()[hip.plan(hip.make_desc(dtype, M, N, K, dtype_out=out_dt, transA=bool(transA), transB=bool(transB))).kernel_id]
+    assert name.endswith("_edge"), name
+    big = 128 if dtype == O.F32 else 256
+    for tile in ((0, 0, 0), (big, big, 0), (big // 2, big // 2, 0)):
+        note(f"case edge {NAMES[dtype]} tA={transA} tB={transB} M={M} N={N} K={K} tile={tile}")
+        got = run_gemm(hip, dtype, A, B, transA, transB, out_dt, M, N, K, tile=tile, pad_c=16)
+        if dtype == O.I8:
+            assert np.array_equal(got, ref)
+        else:
+            check(dtype, out_dt, got, ref)
+
+
+def test_edge_kernels_epilogues_accumulation_and_partial_chunks(hip):
+    """the edge kernels with scales, accumulation into C and an N that ends inside a lane's 16 bytes of output (the row length of
+    C padded to the boundary): int8 with row and column scales to f16 and exact to int32, fp8 with tensor scales to bf16, fp16 with
+    fp32 output accumulated into C"""
+    M, K = 200, 512
+    for N in (392, 396, 397):  # 397: B stored [N][K] only (its rows of C are padded, a B stored [K][N] would have rows of 397 elements)
+        Ai = make_operand(O.I8, M, K, seed=62, tensor=0)
+        Bi = make_operand(O.I8, N, K, seed=62, tensor=1)
+        sA, sB = O.uniform(M, 62, 2, 0.001, 0.02), O.uniform(N, 62, 3, 0.001, 0.02)
+        acc = O.gemm_i32(Ai, Bi, 0, 1)
+        pad_c = 400 - N
+        note(f"case edge epilogue i8 row/col scales N={N}")
+        got = run_gemm(hip, O.I8, Ai, Bi, 0, 1, O.F16, M, N, K, epilogue=hip.EPI_ROW_COL_SCALE, sA=sA, sB=sB, pad_c=pad_c)
+        assert np.array_equal(got, O.epilogue_rowcol_f16(acc, sA, sB))
+        C0 = (np.arange(M * N, dtype=np.int64).reshape(M, N) % 91 - 45).astype(np.int32)
+        note(f"case edge epilogue i8 -> i32 accumulate N={N}")
+        goti = run_gemm(hip, O.I8, Ai, Bi, 0, 1, O.I32, M, N, K, C_init=C0, clear_accum=False, pad_c=pad_c)
+        assert np.array_equal(goti, acc + C0)
+        Ae = make_operand(O.E4M3, M, K, seed=63, tensor=0, scale=0.5)
+        Be = make_operand(O.E4M3, N, K, seed=63, tensor=1, scale=0.5)
+        note(f"case edge epilogue e4m3 tensor scale N={N}")
+        gote = run_gemm(hip, O.E4M3, Ae, Be, 0, 1, O.BF16, M, N, K, epilogue=hip.EPI_TENSOR_SCALE, sA=np.array([0.5], np.float32), sB=np.array([0.25], np.float32), pad_c=pad_c)
+        check(O.E4M3, O.BF16, gote, O.gemm_f64(O.E4M3, Ae, Be, 0, 1) * 0.125)
+        Ah = make_operand(O.F16, M, K, seed=64, tensor=0, scale=0.5)
+        Bh = make_operand(O.F16, N, K, seed=64, tensor=1, scale=0.5)
+        C0f = O.uniform(M * N, 64, 2, -1.0, 1.0).reshape(M, N).astype(np.float32)
+        note(f"case edge epilogue f16 -> f32 accumulate N={N}")
+        goth = run_gemm(hip, O.F16, Ah, Bh, 0, 1, O.F32, M, N, K, C_init=C0f, clear_accum=False, pad_c=pad_c)
+        check(O.F16, O.F32, goth, O.gemm_f64(O.F16, Ah, Bh, 0, 1) + C0f)
+
+
 def test_split_k_epilogues_and_accumulate(hip):
     M, N, K = 32, 256, 2048
     A = make_operand(O.I8, M, K, seed=42, tensor=0)

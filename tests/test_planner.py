@@ -289,16 +289,19 @@ def test_planner_ranks_variants_by_estimated_time():
     assert p.split_k == 1 and p.workspace_bytes == 0
     # A stored [K][M]: fp32 and the 16-bit types have the 32- and 64-row tiles for it too (fp32 32x4096x4096: 249 us on the guarded
     # kernel before, 23.9 now, the vendor library 26.3); the 8-bit types do not (their transposed rows are shorter than the LDS
-    # swizzle needs) and take the guarded kernel there
+    # swizzle needs) and take the 128x128 edge kernel there
     for dt, (M, N, K, tB), want in ((R.F32, (32, 4096, 4096, 0), "f32_tn_32x128x32_w1x4_s3_splitk"), (R.F16, (32, 8192, 8192, 0), "f16_tn_32x128x64_w1x4_s3_splitk"),
                                     (R.F16, (64, 8192, 8192, 1), "f16_tt_64x128x64_w2x2_s3_splitk"), (R.BF16, (96, 4096, 4096, 0), "bf16_tn_32x128x64_w1x4_s3_splitk")):
         assert pick(dt, M, N, K, transA=True, transB=bool(tB)) == want
-    assert pick(R.I8, 32, 4096, 4096, transA=True).endswith("_guard")
+    assert pick(R.I8, 32, 4096, 4096, transA=True) == "i8_tn_128x128x128_w2x2_s2_edge"
     # whole rounds, more than half a round left over, or a descriptor that forbids splitting: no tail
     for shape, kw in (((8192, 8192, 8192), {}), ((5120, 5120, 5120), {}), ((6144, 6144, 6144), {"split_k": 1})):
         p = R.plan(R.make_desc(R.F16, *shape, **kw))
         assert (p.tail_tiles, p.tail_split) == (0, 1) and p.workspace_bytes == 0, shape
-    assert not pick(R.F16, 64, 384, 2048).endswith("_guard") and pick(R.F16, 65, 384, 2048).endswith("_guard")
+    # M or N off the tile: the edge kernels; K off the K tile, or rows off 16-byte boundaries: the guarded one
+    assert not pick(R.F16, 64, 384, 2048).endswith("_guard") and pick(R.F16, 65, 384, 2048) == "f16_nn_128x128x64_w2x2_s2_edge"
+    assert pick(R.F16, 4000, 4096, 4096) == "f16_nn_256x256x64_w2x2_s2x3_a16_edge" and pick(R.F16, 4096, 4000, 4096, transB=True) == "f16_nt_256x256x64_w2x2_s2x3_a16_edge"
+    assert pick(R.F16, 64, 384, 2050).endswith("_guard") and pick(R.F16, 64, 388, 2048).endswith("_guard") and pick(R.F16, 64, 392, 2048).endswith("_edge")
 
 
 def test_wave_policy_decides_the_wave_grid():
