@@ -451,7 +451,13 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
       const double span_a = (double)d->lda * es * (d->transA ? k->bk : k->bm), span_b = (double)d->ldb * es * (d->transB ? k->bn : k->bk);
       if (!k->guard && (span_a >= 4294967296.0 || span_b >= 4294967296.0)) continue;
       if (k->guard && best >= 0 && !ks[best]->guard) continue;  // never a guarded kernel when a fast one fits
-      const double cost = small && !want_split ? small_grid_cost(k, d, no_split) : estimated_cost(k, d, !want_split && !no_split && d->split_k == 0);
+      double cost = small && !want_split ? small_grid_cost(k, d, no_split) : estimated_cost(k, d, !want_split && !no_split && d->split_k == 0);
+      if (k->edge) {
+        // the models see whole tiles; rows and columns beyond M and N are work all the same (a 64-row tile on 32 rows is no
+        // better than the 32-row tile that fits): the square root of the covered area over M x N, as a penalty
+        const double covered = (double)((d->M + k->bm - 1) / k->bm * k->bm) * (double)((d->N + k->bn - 1) / k->bn * k->bn);
+        cost *= std::sqrt(covered / ((double)d->M * (double)d->N));
+      }
       // ties: the first listed variant is the tuned default
       if (best < 0 || (ks[best]->guard && !k->guard) || cost < best_cost) { best = (int)i; best_cost = cost; }
     }

@@ -83,6 +83,11 @@ def square(bk, atom16=False, skinny_ta=(0,)):
         for tb in (0, 1):
             out.append(edge((ta, tb, 256, 256, bk, 2, 2, 2, 0, 0, 1, 3) + ((16,) if atom16 else ())))
             out.append(edge((ta, tb, 128, 128, bk, 2, 2, 2, 0, 0, 1, 2)))
+    # ... and the 32x128 and 64x128 tiles with the split-K store path likewise: a number of rows that is no multiple of 32 against
+    # a large B (fp16 48x8192x8192: 68 us on 128x128 edge tiles, the vendor library 27-35)
+    for tb in (0, 1):
+        out.append(edge((0, tb, 32, 128, bk, 1, 4, 3, 0, 1, 1)))
+        out.append(edge((0, tb, 64, 128, bk, 2, 2, 3, 0, 1, 1)))
     # guarded variants: any shape, any leading dimension, element-aligned pointers
     for ta in (0, 1):
         for tb in (0, 1):
@@ -112,6 +117,7 @@ VARIANTS = {
             + [(ta, tb, 32, 128, 32, 1, 4, 3, 0, 1, 1) for ta in (0, 1) for tb in (0, 1)]
             + [(0, 1, 32, 32, 128, 1, 1, 4, 0, 1, 4), (0, 1, 32, 32, 128, 1, 1, 2, 0, 1, 4), (0, 1, 64, 32, 128, 1, 1, 3, 0, 1, 4)]
             + [edge((ta, tb, bm, bm, 32, 2, 2, 2, 0, 0, 1)) for bm in (128, 64) for ta in (0, 1) for tb in (0, 1)]
+            + [edge((0, tb, 32, 128, 32, 1, 4, 3, 0, 1, 1)) for tb in (0, 1)] + [edge((0, tb, 64, 64, 32, 2, 2, 3, 0, 1, 1)) for tb in (0, 1)]
             + [(ta, tb, 64, 64, 32, 2, 2, 2, 1, 0, 1) for ta in (0, 1) for tb in (0, 1)]),
 }
 

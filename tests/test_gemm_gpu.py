@@ -519,6 +519,33 @@ def test_edge_kernels_take_any_m_and_n(hip, dtype, transA, transB):
             check(dtype, out_dt, got, ref)
 
 
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.I8, O.E4M3, O.F32])
+@pytest.mark.parametrize("transB", [0, 1])
+def test_edge_kernels_with_split_k(hip, dtype, transB):
+    """a number of rows that is no multiple of 32 against a deep K: the 32- and 64-row tiles with the split-K store path exist as
+    edge kernels too, so the planner still splits K over the idle CUs; its own pair and both tiles by name at several splits
+    against the oracle (int8: the same bits)"""
+    N, K = 384, 128 * BK[dtype]
+    for M in (48, 100):
+        sa, sb = stored_shapes(M, N, K, 0, transB)
+        A = make_operand(dtype, *sa, seed=67, tensor=0, scale=0.5)
+        B = make_operand(dtype, *sb, seed=67, tensor=1, scale=0.5)
+        out_dt = DEFAULT_OUT[dtype]
+        ref = O.gemm_i32(A, B, 0, transB) if dtype == O.I8 else O.gemm_f64(dtype, A, B, 0, transB)
+        p = hip.plan(hip.make_desc(dtype, M, N, K, dtype_out=out_dt, transB=bool(transB)))
+        name = hip.kernel_names()[p.kernel_id]
+        assert name.endswith("_splitk_edge") and p.split_k > 1 and p.workspace_bytes == p.split_k * M * N * 4, (name, p.split_k)
+        tiles = ((32, 128, 0), (64, 64, 0)) if dtype == O.F32 else ((32, 128, 0), (64, 128, 0))
+        cases = [dict(), dict(workspace=False)] + [dict(tile=t, split_k=sk, stages=3) for t in tiles for sk in (1, 2, 8)]
+        for kw in cases:
+            note(f"case edge split-K {NAMES[dtype]} tB={transB} M={M} N={N} K={K} {kw}")
+            got = run_gemm(hip, dtype, A, B, 0, transB, out_dt, M, N, K, **kw)
+            if dtype == O.I8:
+                assert np.array_equal(got, ref)
+            else:
+                check(dtype, out_dt, got, ref)
+
+
 def test_edge_kernels_epilogues_accumulation_and_partial_chunks(hip):
     """the edge kernels with scales, accumulation into C and an N that ends inside a lane's 16 bytes of output (the row length of
     C padded to the boundary): int8 with row and column scales to f16 and exact to int32, fp8 with tensor scales to bf16, fp16 with
