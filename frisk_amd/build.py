@@ -28,7 +28,7 @@ COMMON = [
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
     "-Wno-unused-command-line-argument",
 ]
-SOURCES = ["kernels_f16.hip", "kernels_bf16.hip", "kernels_i8.hip", "kernels_e4m3.hip", "kernels_f32.hip", "splitk_reduce.hip", "tile_ops.hip", "elementwise.hip", "softmax.hip", "attention.hip", "capi.cpp"]
+SOURCES = ["kernels_f16.hip", "kernels_f16_2.hip", "kernels_bf16.hip", "kernels_bf16_2.hip", "kernels_i8.hip", "kernels_i8_2.hip", "kernels_e4m3.hip", "kernels_e4m3_2.hip", "kernels_f32.hip", "kernels_f32_2.hip", "splitk_reduce.hip", "tile_ops.hip", "elementwise.hip", "softmax.hip", "attention.hip", "capi.cpp"]
 
 
 def _compile(src):
@@ -44,7 +44,7 @@ def _compile(src):
 def build(jobs=None, verbose=True):
     os.makedirs(OBJDIR, exist_ok=True)
     os.makedirs(LIBDIR, exist_ok=True)
-    jobs = jobs or min(6, os.cpu_count() or 1)
+    jobs = jobs or min(8, os.cpu_count() or 1)
     objs = []
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
         for obj, err in pool.map(_compile, SOURCES):

@@ -57,10 +57,15 @@ static const std::vector<const KernelEntry*>& kernels() {
   static const std::vector<const KernelEntry*> all = [] {
     std::vector<const KernelEntry*> v;
     for (int i = 0; i < kNumKernelsF16; ++i) v.push_back(&kKernelsF16[i]);
+    for (int i = 0; i < kNumKernelsF16_2; ++i) v.push_back(&kKernelsF16_2[i]);
     for (int i = 0; i < kNumKernelsBF16; ++i) v.push_back(&kKernelsBF16[i]);
+    for (int i = 0; i < kNumKernelsBF16_2; ++i) v.push_back(&kKernelsBF16_2[i]);
     for (int i = 0; i < kNumKernelsI8; ++i) v.push_back(&kKernelsI8[i]);
+    for (int i = 0; i < kNumKernelsI8_2; ++i) v.push_back(&kKernelsI8_2[i]);
     for (int i = 0; i < kNumKernelsE4M3; ++i) v.push_back(&kKernelsE4M3[i]);
+    for (int i = 0; i < kNumKernelsE4M3_2; ++i) v.push_back(&kKernelsE4M3_2[i]);
     for (int i = 0; i < kNumKernelsF32; ++i) v.push_back(&kKernelsF32[i]);
+    for (int i = 0; i < kNumKernelsF32_2; ++i) v.push_back(&kKernelsF32_2[i]);
     return v;
   }();
   return all;

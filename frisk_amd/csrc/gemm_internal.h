@@ -72,16 +72,26 @@ hipError_t launch_splitk_reduce(const GemmParams& p, int acc_is_int, hipStream_t
 // the same for the tiles of a tail split
 hipError_t launch_tail_reduce(const GemmParams& p, int acc_is_int, hipStream_t stream);
 
-// defined in kernels_*.hip
+// defined in kernels_*.hip (two tables per element type: kernels_<type>.hip and kernels_<type>_2.hip)
 extern const KernelEntry kKernelsF16[];
 extern const int kNumKernelsF16;
+extern const KernelEntry kKernelsF16_2[];
+extern const int kNumKernelsF16_2;
 extern const KernelEntry kKernelsBF16[];
 extern const int kNumKernelsBF16;
+extern const KernelEntry kKernelsBF16_2[];
+extern const int kNumKernelsBF16_2;
 extern const KernelEntry kKernelsI8[];
 extern const int kNumKernelsI8;
+extern const KernelEntry kKernelsI8_2[];
+extern const int kNumKernelsI8_2;
 extern const KernelEntry kKernelsE4M3[];
 extern const int kNumKernelsE4M3;
+extern const KernelEntry kKernelsE4M3_2[];
+extern const int kNumKernelsE4M3_2;
 extern const KernelEntry kKernelsF32[];
 extern const int kNumKernelsF32;
+extern const KernelEntry kKernelsF32_2[];
+extern const int kNumKernelsF32_2;
 
 }  // namespace frisk

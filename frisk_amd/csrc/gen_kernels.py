@@ -126,23 +126,32 @@ def cfg_of(enum, v):
     return f"GemmCfg<{enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {'true' if gd else 'false'}, {'true' if sk else 'false'}, {wk}, {sb}" + (f", {at}, true>" if eg else (f", {at}>" if at != 32 else ">"))
 
 HERE = os.path.dirname(os.path.abspath(__file__))
+# A type's variants go into two translation units of about equal size (kernels_<type>.hip, kernels_<type>_2.hip), each with a
+# table of its own: the units compile in parallel, and the longest of them sets the time of a build.  The planner walks the
+# first table, then the second, so the order of the list above is the order it sees.
+written = []
 for tag, (enum, suffix, variants) in VARIANTS.items():
-    lines = [f"// {enum} kernel instantiations.  Generated by gen_kernels.py; do not edit by hand.",
-             '#include "gemm_kernel.hip.inc"', "namespace frisk {"]
-    for v in variants:
-        lines.append(f"template __global__ void gemm_kernel<{cfg_of(enum, v)}>(GemmParams);")
-    lines.append("#ifndef __HIP_DEVICE_COMPILE__")
-    lines.append(f"const KernelEntry kKernels{suffix}[] = {{")
-    for v in variants:
-        ta, tb, bm, bn, bk, wm, wn, st, gd, sk, wk, sb, at, eg = full(v)
-        cfg = cfg_of(enum, v)
-        waves = f"w{wm}x{wn}" + (f"x{wk}" if wk > 1 else "")
-        name = f"{tag}_{'t' if ta else 'n'}{'t' if tb else 'n'}_{bm}x{bn}x{bk}_{waves}_s{st}" + (f"x{sb}" if sb != st else "") + (f"_a{at}" if at != 32 else "") + ("_guard" if gd else "") + ("_splitk" if sk else "") + ("_edge" if eg else "")
-        lines.append(f'    {{"{name}", {enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {sb}, {wk}, {gd}, {sk}, {at}, {eg}, {cfg}::LDS_BYTES, {cfg}::MIN_K_TILES, &launch_gemm<{cfg}>, &prepare_gemm<{cfg}>}},')
-    lines.append("};")
-    lines.append(f"const int kNumKernels{suffix} = sizeof(kKernels{suffix}) / sizeof(kKernels{suffix}[0]);")
-    lines.append("#endif")
-    lines.append("}  // namespace frisk")
-    with open(os.path.join(HERE, f"kernels_{tag}.hip"), "w") as f:
-        f.write("\n".join(lines) + "\n")
-print("wrote", ", ".join(f"kernels_{t}.hip" for t in VARIANTS))
+    half = (len(variants) + 1) // 2
+    for part, chunk in ((1, variants[:half]), (2, variants[half:])):
+        ext = "" if part == 1 else "_2"
+        lines = [f"// {enum} kernel instantiations, part {part} of 2.  Generated by gen_kernels.py; do not edit by hand.",
+                 '#include "gemm_kernel.hip.inc"', "namespace frisk {"]
+        for v in chunk:
+            lines.append(f"template __global__ void gemm_kernel<{cfg_of(enum, v)}>(GemmParams);")
+        lines.append("#ifndef __HIP_DEVICE_COMPILE__")
+        lines.append(f"const KernelEntry kKernels{suffix}{ext}[] = {{")
+        for v in chunk:
+            ta, tb, bm, bn, bk, wm, wn, st, gd, sk, wk, sb, at, eg = full(v)
+            cfg = cfg_of(enum, v)
+            waves = f"w{wm}x{wn}" + (f"x{wk}" if wk > 1 else "")
+            name = f"{tag}_{'t' if ta else 'n'}{'t' if tb else 'n'}_{bm}x{bn}x{bk}_{waves}_s{st}" + (f"x{sb}" if sb != st else "") + (f"_a{at}" if at != 32 else "") + ("_guard" if gd else "") + ("_splitk" if sk else "") + ("_edge" if eg else "")
+            lines.append(f'    {{"{name}", {enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {sb}, {wk}, {gd}, {sk}, {at}, {eg}, {cfg}::LDS_BYTES, {cfg}::MIN_K_TILES, &launch_gemm<{cfg}>, &prepare_gemm<{cfg}>}},')
+        lines.append("};")
+        lines.append(f"const int kNumKernels{suffix}{ext} = sizeof(kKernels{suffix}{ext}) / sizeof(kKernels{suffix}{ext}[0]);")
+        lines.append("#endif")
+        lines.append("}  // namespace frisk")
+        fn = f"kernels_{tag}{ext}.hip"
+        with open(os.path.join(HERE, fn), "w") as f:
+            f.write("\n".join(lines) + "\n")
+        written.append(fn)
+print("wrote", ", ".join(written))
