@@ -451,6 +451,8 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
       // are left out where the plain twin fits); the guarded ones take anything
       const bool whole_mn = d->M % k->bm == 0 && d->N % k->bn == 0;
       if (!k->guard && (force_guard || !rows_aligned || d->K % k->bk || (k->edge ? whole_mn : !whole_mn))) continue;
+      // the guarded kernels that move whole 16-byte chunks: aligned rows and pointers, K a whole number of chunks
+      if (k->guard && k->edge && (force_guard || !rows_aligned || d->K % (16 / es))) continue;
       // ... and address a tile's chunks by 32-bit lane offsets from its first row: the stored rows of one tile must span
       // less than 4 GiB
       const double span_a = (double)d->lda * es * (d->transA ? k->bk : k->bm), span_b = (double)d->ldb * es * (d->transB ? k->bn : k->bk);
@@ -460,7 +462,7 @@ static int make_plan(const frisk_gemm_desc* d, frisk_gemm_plan* plan, bool with_
       // (a 32-row edge tile above 64 rows streams B once per 32 rows where the 64-row tile wastes at most as much: 130x11008x4096
       // NT 64.5 against 53.5 us)
       if (k->edge && k->bm == 32 && d->M > 64 && !d->tile_m) continue;
-      if (k->edge) {
+      if (k->edge && !k->guard) {
         // the models see whole tiles; rows and columns beyond M and N are work all the same (a 64-row tile on 32 rows is no
         // better than the 32-row tile that fits): the square root of the covered area over M x N, as a penalty
         const double covered = (double)((d->M + k->bm - 1) / k->bm * k->bm) * (double)((d->N + k->bn - 1) / k->bn * k->bn);

@@ -88,7 +88,11 @@ def square(bk, atom16=False, skinny_ta=(0,)):
     for tb in (0, 1):
         out.append(edge((0, tb, 32, 128, bk, 1, 4, 3, 0, 1, 1)))
         out.append(edge((0, tb, 64, 128, bk, 2, 2, 3, 0, 1, 1)))
-    # guarded variants: any shape, any leading dimension, element-aligned pointers
+    # guarded variants: any shape, any leading dimension, element-aligned pointers; listed first, the same with whole 16-byte chunks
+    # for rows and pointers on 16-byte boundaries and a K of whole chunks (K off the K tile, everything else in order)
+    for ta in (0, 1):
+        for tb in (0, 1):
+            out.append(edge((ta, tb, 128, 128, bk, 2, 2, 2, 1, 0, 1)))
     for ta in (0, 1):
         for tb in (0, 1):
             out.append((ta, tb, 128, 128, bk, 2, 2, 2, 1, 0, 1))
@@ -118,6 +122,7 @@ VARIANTS = {
             + [(0, 1, 32, 32, 128, 1, 1, 4, 0, 1, 4), (0, 1, 32, 32, 128, 1, 1, 2, 0, 1, 4), (0, 1, 64, 32, 128, 1, 1, 3, 0, 1, 4)]
             + [edge((ta, tb, bm, bm, 32, 2, 2, 2, 0, 0, 1)) for bm in (128, 64) for ta in (0, 1) for tb in (0, 1)]
             + [edge((0, tb, 32, 128, 32, 1, 4, 3, 0, 1, 1)) for tb in (0, 1)] + [edge((0, tb, 64, 64, 32, 2, 2, 3, 0, 1, 1)) for tb in (0, 1)]
+            + [edge((ta, tb, 64, 64, 32, 2, 2, 2, 1, 0, 1)) for ta in (0, 1) for tb in (0, 1)]
             + [(ta, tb, 64, 64, 32, 2, 2, 2, 1, 0, 1) for ta in (0, 1) for tb in (0, 1)]),
 }
 
@@ -144,7 +149,7 @@ for tag, (enum, suffix, variants) in VARIANTS.items():
             ta, tb, bm, bn, bk, wm, wn, st, gd, sk, wk, sb, at, eg = full(v)
             cfg = cfg_of(enum, v)
             waves = f"w{wm}x{wn}" + (f"x{wk}" if wk > 1 else "")
-            name = f"{tag}_{'t' if ta else 'n'}{'t' if tb else 'n'}_{bm}x{bn}x{bk}_{waves}_s{st}" + (f"x{sb}" if sb != st else "") + (f"_a{at}" if at != 32 else "") + ("_guard" if gd else "") + ("_splitk" if sk else "") + ("_edge" if eg else "")
+            name = f"{tag}_{'t' if ta else 'n'}{'t' if tb else 'n'}_{bm}x{bn}x{bk}_{waves}_s{st}" + (f"x{sb}" if sb != st else "") + (f"_a{at}" if at != 32 else "") + ("_guard_chunks" if gd and eg else "_guard" if gd else "") + ("_splitk" if sk else "") + ("_edge" if eg and not gd else "")
             lines.append(f'    {{"{name}", {enum}, {ta}, {tb}, {bm}, {bn}, {bk}, {wm}, {wn}, {st}, {sb}, {wk}, {gd}, {sk}, {at}, {eg}, {cfg}::LDS_BYTES, {cfg}::MIN_K_TILES, &launch_gemm<{cfg}>, &prepare_gemm<{cfg}>}},')
         lines.append("};")
         lines.append(f"const int kNumKernels{suffix}{ext} = sizeof(kKernels{suffix}{ext}) / sizeof(kKernels{suffix}{ext}[0]);")

@@ -546,6 +546,30 @@ def test_edge_kernels_with_split_k(hip, dtype, transB):
                 check(dtype, out_dt, got, ref)
 
 
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.I8, O.E4M3, O.F32])
+@pytest.mark.parametrize("transA,transB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_guarded_kernel_moves_whole_chunks_when_only_k_is_off_the_tile(hip, dtype, transA, transB):
+    """K a whole number of 16-byte chunks but no multiple of the K tile, rows on 16-byte boundaries, M and N arbitrary: the
+    guarded kernel that stages 16-byte chunks (zero beyond K, whole or not at all) runs instead of the element-wise one"""
+    es = {O.F32: 4, O.F16: 2, O.BF16: 2}.get(dtype, 1)
+    M, N, K = 208, 400, 2 * BK[dtype] + 3 * (16 // es)
+    sa, sb = stored_shapes(M, N, K, transA, transB)
+    A = make_operand(dtype, *sa, seed=71, tensor=0, scale=0.5)
+    B = make_operand(dtype, *sb, seed=71, tensor=1, scale=0.5)
+    out_dt = DEFAULT_OUT[dtype]
+    name = hip.kernel_names()[hip.plan(hip.make_desc(dtype, M, N, K, dtype_out=out_dt, transA=bool(transA), transB=bool(transB))).kernel_id]
+    assert name.endswith("_guard_chunks"), name
+    note(f"case guarded chunks {NAMES[dtype]} tA={transA} tB={transB} M={M} N={N} K={K}")
+    got = run_gemm(hip, dtype, A, B, transA, transB, out_dt, M, N, K)
+    if dtype == O.I8:
+        assert np.array_equal(got, O.gemm_i32(A, B, transA, transB))
+        sA, sB = O.uniform(M, 71, 2, 0.001, 0.02), O.uniform(N, 71, 3, 0.001, 0.02)
+        got = run_gemm(hip, dtype, A, B, transA, transB, O.F16, M, N, K, epilogue=hip.EPI_ROW_COL_SCALE, sA=sA, sB=sB)
+        assert np.array_equal(got, O.epilogue_rowcol_f16(O.gemm_i32(A, B, transA, transB), sA, sB))
+    else:
+        check(dtype, out_dt, got, O.gemm_f64(dtype, A, B, transA, transB))
+
+
 def test_edge_kernels_epilogues_accumulation_and_partial_chunks(hip):
     """the edge kernels with scales, accumulation into C and an N that ends inside a lane's 16 bytes of output (the row length of
     C padded to the boundary): int8 with row and column scales to f16 and exact to int32, fp8 with tensor scales to bf16, fp16 with

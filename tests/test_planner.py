@@ -301,7 +301,7 @@ def test_planner_ranks_variants_by_estimated_time():
     # M or N off the tile: the edge kernels; K off the K tile, or rows off 16-byte boundaries: the guarded one
     assert not pick(R.F16, 64, 384, 2048).endswith("_guard") and pick(R.F16, 65, 384, 2048) == "f16_nn_64x128x64_w2x2_s3_splitk_edge" and pick(R.F16, 17, 384, 2048) == "f16_nn_32x128x64_w1x4_s3_splitk_edge"
     assert pick(R.F16, 4000, 4096, 4096) == "f16_nn_256x256x64_w2x2_s2x3_a16_edge" and pick(R.F16, 4096, 4000, 4096, transB=True) == "f16_nt_256x256x64_w2x2_s2x3_a16_edge"
-    assert pick(R.F16, 64, 384, 2050).endswith("_guard") and pick(R.F16, 64, 388, 2048).endswith("_guard") and pick(R.F16, 64, 392, 2048).endswith("_edge")
+    assert pick(R.F16, 64, 384, 2056) == "f16_nn_128x128x64_w2x2_s2_guard_chunks" and pick(R.F16, 64, 384, 2050).endswith("_guard") and pick(R.F16, 64, 388, 2048).endswith("_guard") and pick(R.F16, 64, 392, 2048).endswith("_edge")
 
 
 def test_wave_policy_decides_the_wave_grid():
