@@ -518,6 +518,39 @@ def main():
             del Asm, Csm, Cvm, wsm, Bs
         legs["fp32_small_grid"] = small32
 
+        # shapes off the tiles, fp16 NN: M off every tile (edge variant of the 256x256 kernel), 48 rows against a large B rotating over
+        # 3 buffers (edge variant of a skinny split-K kernel), K off the K tile (the guarded kernel that stages whole 16-byte chunks)
+        ragged = {}
+        for Mr, Nr, Kr, nbuf in ((4000, 4096, 4096, 1), (48, 8192, 8192, 3), (4096, 4096, 4000, 1)):
+            Bs = [(torch.randn(Kr, Nr, device=dev, generator=g) / 64).half() for _ in range(nbuf)]
+            Ar = (torch.randn(Mr, Kr, device=dev, generator=g) / 64).half()
+            Cr = torch.empty(Mr, Nr, device=dev, dtype=torch.float16)
+            Cvr = torch.empty_like(Cr)
+            dr = R.make_desc(R.F16, Mr, Nr, Kr, dtype_out=R.F16)
+            pr = R.plan(dr)
+            wr_bytes = R.workspace_bytes(dr)
+            wr = torch.empty(max(wr_bytes, 16), dtype=torch.uint8, device=dev)
+            turn = [0, 0]
+
+            def ours_ragged():
+                b_ = Bs[turn[0] % len(Bs)]
+                turn[0] += 1
+                R.gemm(dr, Ar.data_ptr(), b_.data_ptr(), Cr.data_ptr(), None, None, wr.data_ptr() if wr_bytes else None, wr_bytes, cs)
+
+            def vendor_ragged():
+                b_ = Bs[turn[1] % len(Bs)]
+                turn[1] += 1
+                return torch.matmul(Ar, b_, out=Cvr)
+            trg = time_launches(torch, ours_ragged, a.steps, a.warmup, stream)
+            key = "%dx%dx%d" % (Mr, Nr, Kr)
+            ragged[key] = {"kernel": R.kernel_names()[pr.kernel_id], "split_k": pr.split_k, "kernel_ms": round(trg["mean_ms"], 5),
+                           "kernel_ms_median": round(trg["median_ms"], 5), "kernel_ms_min": round(trg["min_ms"], 5),
+                           "TFLOPs": round(2.0 * Mr * Nr * Kr / (trg["mean_ms"] * 1e-3) / 1e12, 1)}
+            vendor["fp16_ragged_" + key + "_nn"] = vendor_leg(torch, "torch.matmul(A, B, out=C), fp16 %s NN" % key, vendor_ragged, 2.0 * Mr * Nr * Kr,
+                                                              a.steps, a.warmup, stream, trg["mean_ms"])
+            del Ar, Cr, Cvr, wr, Bs
+        legs["fp16_ragged_nn"] = ragged
+
         # the dialect's data-movement ops on a 32768 x 8192 f16 view (512 MiB per array: twice the last-level cache)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
