@@ -88,7 +88,6 @@ def square(bk, atom16=False, skinny_ta=(0,)):
     for tb in (0, 1):
         out.append(edge((0, tb, 32, 128, bk, 1, 4, 3, 0, 1, 1)))
         out.append(edge((0, tb, 64, 128, bk, 2, 2, 3, 0, 1, 1)))
-        out.append(edge((0, tb, 128, 128, bk, 2, 2, 3, 0, 1, 1, 3)))  # 65 to 128 rows: one row of tiles, B streamed once
     # guarded variants: any shape, any leading dimension, element-aligned pointers; listed first, the same with whole 16-byte chunks
     # for rows and pointers on 16-byte boundaries and a K of whole chunks (K off the K tile, everything else in order)
     for ta in (0, 1):
