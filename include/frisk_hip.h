@@ -73,9 +73,12 @@ typedef enum frisk_status {
  * Supported (dtype_ab -> dtype_acc -> dtype_out):
  *   F32->F32->F32, F16->F32->{F16,F32}, BF16->F32->{BF16,F32},
  *   I8->I32->{I32, F16 with ROW_COL_SCALE}, E4M3->F32->{BF16,F32} (NONE or TENSOR_SCALE)
- * tile_* and waves_* = 0 let the planner choose.  Shapes that are whole tiles with 16-byte aligned rows and
- * pointers run the fast kernels; anything else (ragged M, N, K, odd leading dimensions, K = 0) runs a
- * bounds-checked kernel with the same arithmetic.
+ * tile_* and waves_* = 0 let the planner choose.  With rows and pointers on 16-byte boundaries and K a multiple of
+ * the K tile (64 elements of 16 bits, 128 of 8 bits, 32 of fp32) the fast kernels run, for any M and N (where those
+ * are no multiples of the tile, variants of the same kernels whose stores are checked against M and N); anything
+ * else (K off the K tile, odd leading dimensions, element-aligned pointers, K = 0) runs a bounds-checked kernel with
+ * the same arithmetic: one that moves 16-byte chunks while rows and pointers are aligned and K is a whole number of
+ * chunks, an element-wise one otherwise.
  */
 typedef struct frisk_gemm_desc {
   int32_t abi_version; /* FRISK_HIP_ABI_VERSION */
@@ -125,7 +128,7 @@ typedef struct frisk_gemm_plan {
   int32_t grid_x, grid_y;            /* work-group grid (tiles along N, tiles along M) */
   int32_t split_k;                   /* >1: partial sums go through the workspace */
   int32_t xcd_remap;                 /* 1: work-group ids are remapped so each XCD owns a compact block of tiles */
-  int32_t guarded;                   /* 1: the bounds-checked kernel runs (ragged shape, unaligned rows or pointers) */
+  int32_t guarded;                   /* 1: a bounds-checked kernel runs (K off the K tile, unaligned rows or pointers) */
   frisk_lds_layout lds_a, lds_b;
   size_t workspace_bytes;
   double flops;                      /* 2.M.N.K */
